@@ -1,0 +1,247 @@
+// Row-wise kernels around the matrix products: embedding gather, RMSNorm with the
+// residual sum fused in, the rotary table, the fused per-head norm + rotation + cache
+// write, and SwiGLU.  All arithmetic is in 32-bit floats (angles in double); storage
+// is float or bfloat16.
+#include "common.h"
+
+// ---------------------------------------------------------------- embedding
+// out[t, :] = table[ids[t], :] as float.  One block per token.
+// (reference: Daisi.Llogos.Cuda/kernels/elementwise.cu:402-457, one row per call)
+template <typename T>
+__global__ void embed_kernel(float* __restrict__ out, const T* __restrict__ table,
+                             const int* __restrict__ ids, int H) {
+    const int t = blockIdx.x;
+    const T* row = table + (size_t)ids[t] * H;
+    float* o = out + (size_t)t * H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = load_f32(row + i);
+}
+
+LLOGOS_EXPORT int llogos_embed(float* out, const void* table, int table_dtype, const int* ids,
+                               int T, int H, hipStream_t stream) {
+    if (T <= 0 || H <= 0) return LLOGOS_BAD_ARGUMENT;
+    if (table_dtype == DT_F32)
+        embed_kernel<float><<<T, 256, 0, stream>>>(out, (const float*)table, ids, H);
+    else if (table_dtype == DT_BF16)
+        embed_kernel<bf16_t><<<T, 256, 0, stream>>>(out, (const bf16_t*)table, ids, H);
+    else
+        return LLOGOS_BAD_ARGUMENT;
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------- RMSNorm (+ residual add)
+// For output row r (source row s = rows ? rows[r] : r):
+//   v = x[s] + delta[s]   (delta optional; written back to x when write_back)
+//   out[r] = v * rsqrt(mean(v^2) + eps) * w
+// The residual stream x stays in float; out has the matrix products' input type.
+// (reference: rms_norm / add_rms_norm_residual, Daisi.Llogos.Cuda/kernels/elementwise.cu:18-171,
+//  668-733; eps inside the root, weight multiplies as it is.)
+template <typename TO, typename TD>
+__global__ void rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ x, const TD* __restrict__ delta,
+                               const int* __restrict__ rows, const float* __restrict__ w,
+                               float eps, int H, int write_back) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const size_t s = rows ? (size_t)rows[r] : (size_t)r;
+    float* xr = x + s * H;
+    const TD* dr = delta ? delta + s * H : nullptr;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        float v = xr[i];
+        if (dr) {
+            v += load_f32(dr + i);
+            if (write_back) xr[i] = v;
+        }
+        ss += v * v;
+    }
+    const float total = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(total / (float)H + eps);
+    TO* o = out + (size_t)r * H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        float v = xr[i];
+        if (dr && !write_back) v += load_f32(dr + i);
+        store_f32(o + i, v * inv * w[i]);
+    }
+}
+
+LLOGOS_EXPORT int llogos_rmsnorm(void* out, int out_dtype, float* x, const void* delta, int delta_dtype,
+                                 const int* rows, const float* w, float eps, int R, int H,
+                                 int write_back, hipStream_t stream) {
+    if (R <= 0 || H <= 0) return LLOGOS_BAD_ARGUMENT;
+    const int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
+#define LAUNCH(TO, TD) rmsnorm_kernel<TO, TD><<<R, threads, 0, stream>>>( \
+        (TO*)out, x, (const TD*)delta, rows, w, eps, H, write_back)
+    if (out_dtype == DT_F32 && delta_dtype == DT_F32) LAUNCH(float, float);
+    else if (out_dtype == DT_BF16 && delta_dtype == DT_BF16) LAUNCH(bf16_t, bf16_t);
+    else if (out_dtype == DT_BF16 && delta_dtype == DT_F32) LAUNCH(bf16_t, float);
+    else if (out_dtype == DT_F32 && delta_dtype == DT_BF16) LAUNCH(float, bf16_t);
+    else return LLOGOS_BAD_ARGUMENT;
+#undef LAUNCH
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+// x[s] += delta[s] for all rows (the last residual sum, when no norm follows).
+template <typename TD>
+__global__ void residual_add_kernel(float* __restrict__ x, const TD* __restrict__ delta, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] += load_f32(delta + i);
+}
+
+LLOGOS_EXPORT int llogos_residual_add(float* x, const void* delta, int delta_dtype, long long n,
+                                      hipStream_t stream) {
+    if (n <= 0) return LLOGOS_BAD_ARGUMENT;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (delta_dtype == DT_F32) residual_add_kernel<float><<<blocks, 256, 0, stream>>>(x, (const float*)delta, (size_t)n);
+    else if (delta_dtype == DT_BF16) residual_add_kernel<bf16_t><<<blocks, 256, 0, stream>>>(x, (const bf16_t*)delta, (size_t)n);
+    else return LLOGOS_BAD_ARGUMENT;
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------- rotary table
+// cs[t, i] = (cos, sin)(pos[t] * inv_freq[i]) with the angle, cosine and sine in double
+// (reference: Daisi.Llogos.Cpu/Rope.cs:147-152; Daisi.Llogos.Cuda/kernels/elementwise.cu:258-261).
+// One table serves every layer that shares the rotary parameters.
+__global__ void rope_table_kernel(float2* __restrict__ cs, const int* __restrict__ pos,
+                                  const double* __restrict__ inv_freq, int T, int half) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= T * half) return;
+    const int t = idx / half, i = idx % half;
+    const double a = (double)pos[t] * inv_freq[i];
+    cs[idx] = make_float2((float)cos(a), (float)sin(a));
+}
+
+LLOGOS_EXPORT int llogos_rope_table(void* cs, const int* pos, const double* inv_freq, int T, int half,
+                                    hipStream_t stream) {
+    if (T <= 0 || half <= 0) return LLOGOS_BAD_ARGUMENT;
+    const int n = T * half;
+    rope_table_kernel<<<(n + 255) / 256, 256, 0, stream>>>((float2*)cs, pos, inv_freq, T, half);
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------- per-head norm + rotation + cache write
+// One wave per (token, head) of the fused projection row [q heads | k heads | v heads]:
+//   q, k heads: optional RMSNorm over head_dim with a shared weight, then rotation of the
+//               first `rot` dimensions; q goes back in place, k goes to its cache page;
+//   v heads:    copied to the cache.
+// pairing 0: (i, i + rot/2) for checkpoints that are not row-permuted; 1: (2i, 2i+1), the
+// reference's default (Daisi.Llogos.Cuda/kernels/elementwise.cu:243-349; per_head_rms_norm
+// composite_ops.cu:106-136; kv_cache_write composite_ops.cu:198-264).
+constexpr int kHeadsPerBlock = 4;
+constexpr int kMaxHeadDim = 512;
+
+template <typename T>
+__global__ void qk_rope_cache_kernel(T* __restrict__ qkv, int row_stride, int n_heads, int n_kv_heads,
+                                     int head_dim, int rot, int pairing,
+                                     const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w,
+                                     float eps, const float2* __restrict__ cs,
+                                     T* __restrict__ k_pool, T* __restrict__ v_pool, PagedKV cache,
+                                     const int* __restrict__ tok_seq, const int* __restrict__ tok_pos) {
+    extern __shared__ float smem[];
+    const int t = blockIdx.x;
+    const int head = blockIdx.y * kHeadsPerBlock + threadIdx.y;
+    const int lane = threadIdx.x;
+    const int total_heads = n_heads + 2 * n_kv_heads;
+    const bool active = head < total_heads;
+    float* buf = smem + threadIdx.y * head_dim;
+    const int half = rot / 2;
+
+    T* src = qkv + (size_t)t * row_stride + (size_t)(active ? head : 0) * head_dim;
+    const bool is_q = head < n_heads;
+    const bool is_k = !is_q && head < n_heads + n_kv_heads;
+    const float* norm_w = is_q ? q_norm_w : (is_k ? k_norm_w : nullptr);
+
+    float ss = 0.f;
+    if (active) {
+        for (int d = lane; d < head_dim; d += kWave) {
+            const float v = load_f32(src + d);
+            buf[d] = v;
+            ss += v * v;
+        }
+    }
+    ss = wave_sum(ss);
+    __syncthreads();
+    if (active && norm_w) {
+        const float inv = 1.0f / sqrtf(ss / (float)head_dim + eps);
+        for (int d = lane; d < head_dim; d += kWave) buf[d] = buf[d] * inv * norm_w[d];
+    }
+    __syncthreads();
+    if (!active) return;
+
+    T* dst;
+    if (is_q) {
+        dst = src;
+    } else {
+        const int kvh = is_k ? head - n_heads : head - n_heads - n_kv_heads;
+        const size_t off = paged_offset(cache, tok_seq[t], kvh, tok_pos[t]);
+        dst = (is_k ? k_pool : v_pool) + off;
+    }
+    if (is_q || is_k) {
+        const float2* c = cs + (size_t)t * half;
+        for (int d = lane; d < head_dim; d += kWave) {
+            float v = buf[d];
+            if (d < rot) {
+                if (pairing == 0) {
+                    if (d < half) v = buf[d] * c[d].x - buf[d + half] * c[d].y;
+                    else          v = buf[d - half] * c[d - half].y + buf[d] * c[d - half].x;
+                } else {
+                    const int i = d >> 1;
+                    if ((d & 1) == 0) v = buf[d] * c[i].x - buf[d + 1] * c[i].y;
+                    else              v = buf[d - 1] * c[i].y + buf[d] * c[i].x;
+                }
+            }
+            store_f32(dst + d, v);
+        }
+    } else {
+        for (int d = lane; d < head_dim; d += kWave) store_f32(dst + d, buf[d]);
+    }
+}
+
+LLOGOS_EXPORT int llogos_qk_rope_cache(void* qkv, int dtype, int row_stride, int n_heads, int n_kv_heads,
+                                       int head_dim, int rot, int pairing,
+                                       const float* q_norm_w, const float* k_norm_w, float eps,
+                                       const void* cs, void* k_pool, void* v_pool,
+                                       const int* table, int table_stride,
+                                       const int* tok_seq, const int* tok_pos, int T, hipStream_t stream) {
+    if (T <= 0 || n_heads <= 0 || n_kv_heads < 0 || head_dim <= 0 || head_dim > kMaxHeadDim) return LLOGOS_BAD_ARGUMENT;
+    if (rot < 0 || rot > head_dim || (rot & 1)) return LLOGOS_BAD_ARGUMENT;
+    if (n_kv_heads > 0 && (!k_pool || !v_pool || !table)) return LLOGOS_BAD_ARGUMENT;
+    if (row_stride < (n_heads + 2 * n_kv_heads) * head_dim) return LLOGOS_BAD_ARGUMENT;
+    PagedKV cache{table, table_stride, n_kv_heads, head_dim};
+    const int total_heads = n_heads + 2 * n_kv_heads;
+    dim3 grid(T, (total_heads + kHeadsPerBlock - 1) / kHeadsPerBlock), block(kWave, kHeadsPerBlock);
+    const size_t smem = (size_t)kHeadsPerBlock * head_dim * sizeof(float);
+    if (dtype == DT_F32)
+        qk_rope_cache_kernel<float><<<grid, block, smem, stream>>>(
+            (float*)qkv, row_stride, n_heads, n_kv_heads, head_dim, rot, pairing, q_norm_w, k_norm_w, eps,
+            (const float2*)cs, (float*)k_pool, (float*)v_pool, cache, tok_seq, tok_pos);
+    else if (dtype == DT_BF16)
+        qk_rope_cache_kernel<bf16_t><<<grid, block, smem, stream>>>(
+            (bf16_t*)qkv, row_stride, n_heads, n_kv_heads, head_dim, rot, pairing, q_norm_w, k_norm_w, eps,
+            (const float2*)cs, (bf16_t*)k_pool, (bf16_t*)v_pool, cache, tok_seq, tok_pos);
+    else
+        return LLOGOS_BAD_ARGUMENT;
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------- SwiGLU
+// out[t, i] = silu(gu[t, i]) * gu[t, I + i] from the fused row [gate | up].
+// (reference: split_swiglu, Daisi.Llogos.Cuda/kernels/elementwise.cu:1084-1110; silu(z) = z / (1 + exp(-z)))
+template <typename T>
+__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ gu, int I, size_t n) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n) return;
+    const size_t t = idx / I;
+    const int i = (int)(idx % I);
+    const float g = load_f32(gu + t * 2 * I + i);
+    const float u = load_f32(gu + t * 2 * I + I + i);
+    store_f32(out + idx, g / (1.0f + expf(-g)) * u);
+}
+
+LLOGOS_EXPORT int llogos_swiglu(void* out, const void* gu, int dtype, int T, int I, hipStream_t stream) {
+    if (T <= 0 || I <= 0) return LLOGOS_BAD_ARGUMENT;
+    const size_t n = (size_t)T * I;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (dtype == DT_F32) swiglu_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)gu, I, n);
+    else if (dtype == DT_BF16) swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, I, n);
+    else return LLOGOS_BAD_ARGUMENT;
+    return LLOGOS_LAUNCH_CHECK();
+}

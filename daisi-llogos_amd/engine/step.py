@@ -1,0 +1,168 @@
+"""The step function: a batch of sequences, each with its next tokens, run as one batch
+from the cache; logits come back for the wanted places.
+
+The reference has two step shapes for one sequence: a whole prompt
+(ForwardBatchedPrefill, Daisi.Llogos/Inference/ForwardPass.cs:630-697) and one token
+(Forward, :174-184).  Here a step takes any number of sequences with unequal token
+counts; no padding token enters any kernel."""
+from __future__ import annotations
+
+import os
+from typing import List, Optional, Sequence, Tuple, Union
+
+import numpy as np
+import torch
+
+from ..cache.kv_cache import Cache
+from ..config.model_config import read_config_json
+from ..config.registry import architecture_of
+from ..models.model import Model
+from ..ops import library
+from ..parts.base import Runtime, StepContext
+from ..weights.loader import Checkpoint
+
+_DTYPES = {"float32": torch.float32, "fp32": torch.float32, "f32": torch.float32,
+           "bfloat16": torch.bfloat16, "bf16": torch.bfloat16}
+
+
+class StepError(ValueError):
+    """A step that cannot run: empty token list, token out of range, slot used twice."""
+
+
+def resolve_dtype(dtype: Union[str, torch.dtype]) -> torch.dtype:
+    if isinstance(dtype, torch.dtype):
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"dtype {dtype} is not supported (float32 or bfloat16)")
+        return dtype
+    try:
+        return _DTYPES[str(dtype).lower()]
+    except KeyError:
+        raise ValueError(f"dtype '{dtype}' is not supported (float32 or bfloat16)") from None
+
+
+def require_gpu(device: Union[str, torch.device] = "cuda:0") -> torch.device:
+    """The device the engine runs on.  There is no CPU path: without a GPU or without the
+    kernel library this raises."""
+    device = torch.device(device)
+    if device.type != "cuda" or not torch.cuda.is_available():
+        raise RuntimeError("the engine runs on an AMD GPU only (no CPU fallback); no GPU is visible")
+    library.load()
+    return device
+
+
+class Engine:
+    """A bound model with its cache.  `step` is the only way tokens reach the model."""
+
+    def __init__(self, model: Model, rt: Runtime, max_tokens: int, n_slots: int = 64, config=None):
+        self.model, self.rt, self.config = model, rt, config
+        reads_from = [e.cache_of for e in model.schedule]
+        self.cache = Cache(model.cache_needs(), reads_from, max_tokens, rt, n_slots)
+        self.vocab_size = model.spec.vocab_size
+        self.steps_run = 0
+
+    # ---- construction ---------------------------------------------------------------
+    @classmethod
+    def from_folder(cls, folder: str, dtype: Union[str, torch.dtype] = "bfloat16", max_tokens: int = 4096,
+                    n_slots: int = 64, device: Union[str, torch.device] = "cuda:0", **spec_options) -> "Engine":
+        """config.json chooses the model class through the registry; model.safetensors is
+        checked against what the model needs before any tensor is read."""
+        dev = require_gpu(device)
+        data = read_config_json(folder)
+        arch = architecture_of(data)
+        config = arch.read_config(data)
+        model = Model(arch.model_spec(config, **spec_options))
+        ckpt = Checkpoint(folder)
+        try:
+            tied = model.spec.head_name + ".weight" if model.spec.tie_head else None
+            ckpt.check(model.tensor_specs(), tied_head=tied)
+            rt = Runtime(dev, resolve_dtype(dtype))
+            with torch.cuda.device(dev):
+                model.bind(ckpt.get, rt)
+                torch.cuda.synchronize()
+        finally:
+            ckpt.close()
+        return cls(model, rt, max_tokens, n_slots, config)
+
+    # ---- slots ---------------------------------------------------------------------
+    def alloc_slot(self) -> int:
+        return self.cache.alloc_slot()
+
+    def free_slot(self, slot: int) -> None:
+        self.cache.free_slot(slot)
+
+    # ---- the step --------------------------------------------------------------------
+    def step(self, entries: Sequence[Tuple[int, Sequence[int]]],
+             want: Union[str, Sequence[Sequence[int]], None] = "last") -> Optional[torch.Tensor]:
+        """entries: (slot, next tokens) for each sequence of the batch.  want: 'last', 'all',
+        None, or for each entry the places among its tokens whose logits are asked for.
+        Returns float32 logits [wanted places, vocab] in the order of the entries and of
+        `want`, or None when nothing is wanted."""
+        if not entries:
+            raise StepError("a step needs at least one sequence")
+        slot_ids = [int(s) for s, _ in entries]
+        if len(set(slot_ids)) != len(slot_ids):
+            raise StepError("a slot appears twice in one step")
+        counts = [len(t) for _, t in entries]
+        if min(counts) <= 0:
+            raise StepError("every sequence of a step must bring at least one token")
+        ids = np.concatenate([np.asarray(t, dtype=np.int64).reshape(-1) for _, t in entries])
+        if ids.min() < 0 or ids.max() >= self.vocab_size:
+            raise StepError(f"token id outside 0..{self.vocab_size - 1}")
+        starts = [self.cache.length(s) for s in slot_ids]
+        new_lens = [s + c for s, c in zip(starts, counts)]
+        cu = np.zeros(len(entries) + 1, dtype=np.int64)
+        np.cumsum(counts, out=cu[1:])
+        rows = self._want_rows(want, counts, cu)
+
+        self.cache.reserve(slot_ids, new_lens)
+        T, B = int(cu[-1]), len(entries)
+        tok_seq = np.repeat(np.arange(B, dtype=np.int32), counts)
+        tok_pos = np.concatenate([np.arange(s, s + c, dtype=np.int32) for s, c in zip(starts, counts)])
+        tables = self.cache.step_tables(slot_ids)
+        parts = [ids.astype(np.int32), tok_seq, tok_pos, np.asarray(slot_ids, dtype=np.int32),
+                 np.asarray(rows, dtype=np.int32)] + [t.reshape(-1) for t in tables]
+        dev = self._upload(parts)
+        with torch.cuda.device(self.rt.device):
+            ctx = StepContext(runtime=self.rt, n_tokens=T, batch=B, ids=dev[0], tok_seq=dev[1], tok_pos=dev[2],
+                              slots=dev[3], cu_seqlens=[int(c) for c in cu], starts=starts, slot_ids=slot_ids,
+                              is_decode=max(counts) == 1, max_context=max(new_lens))
+            dev_tables = [d.view(t.shape) for d, t in zip(dev[5:], tables)]
+            caches = self.cache.layer_caches(dev_tables)
+            logits = self.model.forward(ctx, caches, dev[4] if len(rows) else None)
+        self.cache.commit(slot_ids, new_lens)
+        self.steps_run += 1
+        return logits
+
+    def _want_rows(self, want, counts: List[int], cu: np.ndarray) -> List[int]:
+        if want is None:
+            return []
+        if isinstance(want, str):
+            if want == "last":
+                return [int(cu[i + 1]) - 1 for i in range(len(counts))]
+            if want == "all":
+                return list(range(int(cu[-1])))
+            if want == "none":
+                return []
+            raise StepError(f"want must be 'last', 'all', 'none' or lists of places, got '{want}'")
+        if len(want) != len(counts):
+            raise StepError("want must have one list of places for each sequence")
+        rows = []
+        for i, places in enumerate(want):
+            for p in places:
+                p = int(p)
+                if not 0 <= p < counts[i]:
+                    raise StepError(f"wanted place {p} is outside the {counts[i]} tokens of sequence {i}")
+                rows.append(int(cu[i]) + p)
+        return rows
+
+    def _upload(self, parts: List[np.ndarray]) -> List[torch.Tensor]:
+        """One host-to-device copy for all of a step's integer arrays."""
+        sizes = [p.size for p in parts]
+        flat = np.concatenate(parts) if len(parts) > 1 else parts[0]
+        host = torch.from_numpy(np.ascontiguousarray(flat, dtype=np.int32))
+        dev = host.to(self.rt.device, non_blocking=False)
+        out, o = [], 0
+        for n in sizes:
+            out.append(dev[o:o + n])
+            o += n
+        return out

@@ -1,0 +1,233 @@
+"""Python face of the HIP kernels: argument checks, then one call into the library.
+
+Every function checks on the host that shapes, element types and devices match what the
+kernel and its grid assume, and raises before anything is launched.  Tensors are torch
+tensors used as device memory; launches go to torch's current stream.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import library
+
+F32, BF16 = 0, 1
+_DT = {torch.float32: F32, torch.bfloat16: BF16}
+PAGE_TOKENS = 64
+MAX_HEAD_DIM = 512
+
+
+class KernelError(RuntimeError):
+    """A kernel refused its arguments or failed to launch."""
+
+
+def _lib():
+    return library.load()
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise KernelError(f"element type {t.dtype} is not supported (float32 or bfloat16)") from None
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev(*tensors) -> None:
+    for t in tensors:
+        if t is not None:
+            _need(t.is_cuda, "kernel arguments must live on the GPU")
+            _need(t.is_contiguous(), "kernel arguments must be contiguous")
+
+
+def _check(code: int, name: str) -> None:
+    if code != 0:
+        if code == -1:
+            raise KernelError(f"{name}: bad argument")
+        if code == -2:
+            raise KernelError(f"{name}: size not supported")
+        raise KernelError(f"{name}: HIP error {code}")
+
+
+def _i32(t: Optional[torch.Tensor], name: str) -> None:
+    if t is not None:
+        _need(t.dtype == torch.int32, f"{name} must be int32")
+
+
+# ----------------------------------------------------------------------------
+def embed(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    """float32 rows of `table` ([V, H], float32 or bfloat16) at int32 `ids`."""
+    _dev(table, ids)
+    _i32(ids, "ids")
+    _need(table.dim() == 2 and ids.dim() == 1, "embed: table [V, H], ids [T]")
+    T, H = ids.numel(), table.shape[1]
+    out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    _check(_lib().llogos_embed(_p(out), _p(table), _dt(table), _p(ids), T, H, _stream()), "embed")
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+            delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
+            write_back: bool = True) -> torch.Tensor:
+    """RMSNorm of the float32 residual stream `x` [T, H] with the pending `delta` added
+    first (and written back to `x` when `write_back`).  With `rows` only those rows are
+    normed, into a compact output."""
+    _dev(x, weight, delta, rows)
+    _i32(rows, "rows")
+    _need(x.dtype == torch.float32 and x.dim() == 2, "rmsnorm: x must be float32 [T, H]")
+    T, H = x.shape
+    _need(weight.dtype == torch.float32 and weight.shape == (H,), "rmsnorm: weight must be float32 [H]")
+    if delta is not None:
+        _need(delta.shape == x.shape, "rmsnorm: delta must have x's shape")
+    R = rows.numel() if rows is not None else T
+    out = torch.empty((R, H), dtype=out_dtype, device=x.device)
+    if R == 0:
+        return out
+    _check(_lib().llogos_rmsnorm(_p(out), _DT[out_dtype], _p(x), _p(delta), _dt(delta) if delta is not None else F32,
+                                 _p(rows), _p(weight), ctypes.c_float(eps), R, H, int(write_back), _stream()),
+           "rmsnorm")
+    return out
+
+
+def residual_add(x: torch.Tensor, delta: torch.Tensor) -> None:
+    _dev(x, delta)
+    _need(x.dtype == torch.float32 and delta.shape == x.shape, "residual_add: x float32, same shapes")
+    _check(_lib().llogos_residual_add(_p(x), _p(delta), _dt(delta), ctypes.c_longlong(x.numel()), _stream()),
+           "residual_add")
+
+
+def gemm_generic(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype,
+                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """a [M, K] . w [N, K]^T (+ bias) with plain 32-bit FMAs."""
+    _dev(w, bias)
+    _need(a.is_cuda and a.dim() == 2 and a.stride(1) == 1, "gemm: a must be [M, K] with unit inner stride")
+    M, K = a.shape
+    _need(w.dim() == 2 and w.shape[1] == K, f"gemm: w must be [N, {K}], got {tuple(w.shape)}")
+    N = w.shape[0]
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.shape == (N,), "gemm: bias must be float32 [N]")
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    else:
+        _need(out.shape == (M, N) and out.dtype == out_dtype and out.stride(1) == 1, "gemm: bad out")
+    if M == 0:
+        return out
+    _check(_lib().llogos_gemm_generic(_p(out), _dt(out), _p(a), _dt(a), _p(w), _dt(w), _p(bias),
+                                      M, N, K, a.stride(0), out.stride(0), _stream()), "gemm_generic")
+    return out
+
+
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+    """[T, half, 2] float32 (cos, sin) of positions[t] * inv_freq[i], computed in double."""
+    _dev(positions, inv_freq)
+    _i32(positions, "positions")
+    _need(inv_freq.dtype == torch.float64 and inv_freq.dim() == 1, "rope_table: inv_freq must be float64 [half]")
+    T, half = positions.numel(), inv_freq.numel()
+    cs = torch.empty((T, half, 2), dtype=torch.float32, device=positions.device)
+    _check(_lib().llogos_rope_table(_p(cs), _p(positions), _p(inv_freq), T, half, _stream()), "rope_table")
+    return cs
+
+
+def qk_rope_cache(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, rot: int, pairing: int,
+                  q_norm_w: Optional[torch.Tensor], k_norm_w: Optional[torch.Tensor], eps: float,
+                  cs: torch.Tensor, k_pool: Optional[torch.Tensor], v_pool: Optional[torch.Tensor],
+                  table: Optional[torch.Tensor], tok_seq: torch.Tensor, tok_pos: torch.Tensor) -> None:
+    """Per-head norm (optional), rotation and cache write on the fused projection rows
+    [q | k | v] in place: q stays in `qkv`, k and v go to their pages."""
+    _dev(qkv, q_norm_w, k_norm_w, cs, k_pool, v_pool, table, tok_seq, tok_pos)
+    _i32(tok_seq, "tok_seq"); _i32(tok_pos, "tok_pos"); _i32(table, "table")
+    T = qkv.shape[0]
+    width = (n_heads + 2 * n_kv_heads) * head_dim
+    _need(qkv.dim() == 2 and qkv.shape[1] == width, f"qk_rope_cache: qkv must be [T, {width}]")
+    _need(0 < head_dim <= MAX_HEAD_DIM, f"qk_rope_cache: head_dim {head_dim} not in 1..{MAX_HEAD_DIM}")
+    _need(rot % 2 == 0 and 0 <= rot <= head_dim, "qk_rope_cache: rotary dimension must be even and <= head_dim")
+    _need(cs.dtype == torch.float32 and cs.shape == (T, rot // 2, 2), "qk_rope_cache: rotary table shape")
+    _need(tok_seq.numel() == T and tok_pos.numel() == T, "qk_rope_cache: per-token arrays must have T entries")
+    for wgt in (q_norm_w, k_norm_w):
+        if wgt is not None:
+            _need(wgt.dtype == torch.float32 and wgt.shape == (head_dim,), "qk_rope_cache: norm weight float32 [head_dim]")
+    if n_kv_heads > 0:
+        _need(k_pool is not None and v_pool is not None and table is not None, "qk_rope_cache: cache missing")
+        _need(k_pool.dtype == qkv.dtype and v_pool.dtype == qkv.dtype, "qk_rope_cache: cache type differs")
+        _need(tuple(k_pool.shape[1:]) == (n_kv_heads, PAGE_TOKENS, head_dim) and k_pool.shape == v_pool.shape,
+              "qk_rope_cache: pool must be [pages, kv_heads, 64, head_dim]")
+        _need(table.dim() == 2, "qk_rope_cache: page table must be [batch, pages]")
+    _check(_lib().llogos_qk_rope_cache(
+        _p(qkv), _dt(qkv), qkv.stride(0), n_heads, n_kv_heads, head_dim, rot, pairing,
+        _p(q_norm_w), _p(k_norm_w), ctypes.c_float(eps), _p(cs), _p(k_pool), _p(v_pool),
+        _p(table), table.stride(0) if table is not None else 0, _p(tok_seq), _p(tok_pos), T, _stream()),
+        "qk_rope_cache")
+
+
+def attention_generic(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                      table: torch.Tensor, tok_seq: torch.Tensor, tok_pos: torch.Tensor,
+                      n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
+                      window: int = 0, sinks: int = 0) -> torch.Tensor:
+    """Attention of T query rows (row stride `q_stride` elements, heads first) over the
+    paged cache; returns [T, n_heads * head_dim] in the cache's element type."""
+    _dev(k_pool, v_pool, table, tok_seq, tok_pos)
+    _i32(tok_seq, "tok_seq"); _i32(tok_pos, "tok_pos"); _i32(table, "table")
+    T = tok_seq.numel()
+    _need(q.is_cuda and q.dtype == k_pool.dtype, "attention: q and cache types differ")
+    _need(n_heads % n_kv_heads == 0, "attention: heads must be a multiple of kv heads")
+    _need(0 < head_dim <= MAX_HEAD_DIM, f"attention: head_dim {head_dim} not in 1..{MAX_HEAD_DIM}")
+    _need(tuple(k_pool.shape[1:]) == (n_kv_heads, PAGE_TOKENS, head_dim) and k_pool.shape == v_pool.shape,
+          "attention: pool must be [pages, kv_heads, 64, head_dim]")
+    _need(q_stride >= n_heads * head_dim and q.numel() >= (T - 1) * q_stride + n_heads * head_dim,
+          "attention: q too small")
+    out = torch.empty((T, n_heads * head_dim), dtype=q.dtype, device=q.device)
+    _check(_lib().llogos_attention_generic(
+        _p(out), _p(q), _dt(q), q_stride, _p(k_pool), _p(v_pool), _p(table), table.stride(0),
+        _p(tok_seq), _p(tok_pos), T, n_heads, n_kv_heads, head_dim, ctypes.c_float(scale),
+        window, sinks, _stream()), "attention_generic")
+    return out
+
+
+def swiglu(gu: torch.Tensor) -> torch.Tensor:
+    """silu(gate) * up from fused rows [gate | up]."""
+    _dev(gu)
+    _need(gu.dim() == 2 and gu.shape[1] % 2 == 0, "swiglu: rows must be [gate | up]")
+    T, I = gu.shape[0], gu.shape[1] // 2
+    out = torch.empty((T, I), dtype=gu.dtype, device=gu.device)
+    _check(_lib().llogos_swiglu(_p(out), _p(gu), _dt(gu), T, I, _stream()), "swiglu")
+    return out
+
+
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    """int32 index of the first maximum of each row of float32 logits."""
+    _dev(logits)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "argmax: logits must be float32 [R, V]")
+    R, V = logits.shape
+    out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    _check(_lib().llogos_argmax(_p(out), _p(logits), R, V, _stream()), "argmax")
+    return out
+
+
+# ----------------------------------------------------------------------------
+# dispatch: which kernel serves a call
+# ----------------------------------------------------------------------------
+def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype) -> torch.Tensor:
+    """a [M, K] . w [N, K]^T (+ bias [N]) -> [M, N] of `out_dtype`."""
+    return gemm_generic(a, w, bias, out_dtype)
+
+
+def attention(ctx, q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
+              table: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
+              window: int = 0, sinks: int = 0) -> torch.Tensor:
+    """Attention of the step's query rows over the cache pages of their sequences."""
+    return attention_generic(q, q_stride, k_pool, v_pool, table, ctx.tok_seq, ctx.tok_pos,
+                             n_heads, n_kv_heads, head_dim, scale, window, sinks)

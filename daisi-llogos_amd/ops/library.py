@@ -1,0 +1,186 @@
+"""Builds and loads the HIP kernel library (gfx950) that every device op calls.
+
+`build()` always compiles; `load()` uses the library that is there and compiles only
+when none is.  There is no fallback: without the library the ops raise.
+"""
+from __future__ import annotations
+
+import ctypes
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import threading
+import time
+from concurrent.futures import ThreadPoolExecutor
+
+_CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
+_PKG = os.path.dirname(_CSRC)
+LIB_NAME = "libllogos_hip.so"
+ARCH = "gfx950"
+
+HIPCC_FLAGS = [
+    "-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
+    # packed 32-bit float instructions are kept out of the generated code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
+]
+
+_lock = threading.Lock()
+_lib = None
+
+
+class KernelLibraryError(RuntimeError):
+    """The HIP kernel library is missing and could not be built, or failed to load."""
+
+
+def _log(msg: str) -> None:
+    print(f"[llogos] {msg}", file=sys.stderr, flush=True)
+
+
+def sources() -> list:
+    return sorted(f for f in os.listdir(_CSRC) if f.endswith(".hip"))
+
+
+def _source_hash() -> str:
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(_CSRC)):
+        if name.endswith((".hip", ".h")):
+            h.update(name.encode())
+            with open(os.path.join(_CSRC, name), "rb") as fh:
+                h.update(fh.read())
+    h.update(" ".join(HIPCC_FLAGS).encode())
+    return h.hexdigest()
+
+
+def _writable(path: str) -> bool:
+    try:
+        os.makedirs(path, exist_ok=True)
+        probe = os.path.join(path, f".probe{os.getpid()}")
+        with open(probe, "w"):
+            pass
+        os.remove(probe)
+        return True
+    except OSError:
+        return False
+
+
+def build_dirs() -> list:
+    """Where a built library may live: in the tree, else a per-user folder under the
+    temporary directory (for a tree the user cannot write to)."""
+    dirs = [os.path.join(_PKG, "_build")]
+    tmp = os.path.join(tempfile.gettempdir(), f"llogos_build_{os.getuid()}_{_source_hash()[:12]}")
+    dirs.append(tmp)
+    return dirs
+
+
+def find_library() -> str | None:
+    env = os.environ.get("LLOGOS_KERNEL_LIBRARY")
+    if env:
+        return env if os.path.isfile(env) else None
+    for d in build_dirs():
+        p = os.path.join(d, LIB_NAME)
+        if os.path.isfile(p):
+            return p
+    return None
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.isfile(cand):
+            return cand
+    raise KernelLibraryError("hipcc not found: the HIP kernel library cannot be built")
+
+
+def _run_with_progress(cmd: list, what: str, env: dict) -> None:
+    start = time.time()
+    proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, env=env, text=True)
+    done = threading.Event()
+
+    def ticker():
+        while not done.wait(20.0):
+            _log(f"still compiling {what} ({time.time() - start:.0f} s)")
+    th = threading.Thread(target=ticker, daemon=True)
+    th.start()
+    out, _ = proc.communicate()
+    done.set()
+    if proc.returncode != 0:
+        raise KernelLibraryError(f"hipcc failed on {what}:\n{out}")
+    noise = ("packed-fp32-ops", "is not a recognized feature")
+    for line in out.splitlines():
+        if line.strip() and not any(n in line for n in noise):
+            print(line, file=sys.stderr)
+
+
+def build(verbose: bool = True) -> str:
+    """Compile every .hip source for gfx950 and link the shared library.  Returns its path."""
+    hipcc = _hipcc()
+    out_dir = next((d for d in build_dirs() if _writable(d)), None)
+    if out_dir is None:
+        raise KernelLibraryError("no writable folder for the kernel library")
+    env = dict(os.environ)
+    # an empty or unwritable HOME must not stop the compiler from keeping its temporaries
+    env.setdefault("TMPDIR", tempfile.gettempdir())
+    srcs = sources()
+    obj_dir = os.path.join(out_dir, "obj")
+    os.makedirs(obj_dir, exist_ok=True)
+    if verbose:
+        _log(f"building {LIB_NAME} for {ARCH} from {len(srcs)} sources into {out_dir}")
+    t0 = time.time()
+    counter = {"n": 0}
+
+    def compile_one(name: str) -> str:
+        obj = os.path.join(obj_dir, name[:-4] + ".o")
+        cmd = [hipcc, *HIPCC_FLAGS, "-I", _CSRC, "-c", os.path.join(_CSRC, name), "-o", obj]
+        _run_with_progress(cmd, name, env)
+        with _lock:
+            counter["n"] += 1
+            if verbose:
+                _log(f"compiled {name} ({counter['n']}/{len(srcs)}, {time.time() - t0:.0f} s)")
+        return obj
+
+    workers = max(1, min(len(srcs), int(os.environ.get("MAX_JOBS", os.cpu_count() or 4)), 16))
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        objs = list(pool.map(compile_one, srcs))
+    tmp_lib = os.path.join(out_dir, f".{LIB_NAME}.{os.getpid()}")
+    _run_with_progress([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", tmp_lib, *objs], "link", env)
+    lib_path = os.path.join(out_dir, LIB_NAME)
+    os.replace(tmp_lib, lib_path)
+    with open(os.path.join(out_dir, "sources.sha256"), "w") as fh:
+        fh.write(_source_hash())
+    if verbose:
+        _log(f"built {lib_path} in {time.time() - t0:.0f} s")
+    global _lib
+    _lib = None
+    return lib_path
+
+
+def is_stale(lib_path: str) -> bool:
+    stamp = os.path.join(os.path.dirname(lib_path), "sources.sha256")
+    try:
+        with open(stamp) as fh:
+            return fh.read().strip() != _source_hash()
+    except OSError:
+        return True
+
+
+def load() -> ctypes.CDLL:
+    """The loaded kernel library; built first if no built library exists."""
+    global _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+    path = find_library()
+    if path is None:
+        path = build()
+    elif is_stale(path):
+        _log(f"warning: {path} is older than the sources in {_CSRC}; run __graft_entry__.build() to refresh it")
+    try:
+        lib = ctypes.CDLL(path)
+    except OSError as e:
+        raise KernelLibraryError(f"cannot load {path}: {e}") from e
+    with _lock:
+        _lib = lib
+    return lib

@@ -1,0 +1,172 @@
+"""What every part of a layer has in common: the tensors it asks for, the runtime it is
+bound to, and the description of a step that is handed through the layers.
+
+A part knows its own sizes, constants and tensor names (by a prefix it is given) and
+nothing about the model that holds it.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Callable, Dict, List, Optional, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class TensorSpec:
+    """One tensor a part reads from the checkpoint.
+
+    kind drives random initialisation: 'matrix' and 'table' N(0, std), 'bias' N(0, std),
+    'norm' 1 + U(-0.1, 0.1).  `optional` tensors may be absent."""
+    name: str
+    shape: Tuple[int, ...]
+    kind: str = "matrix"
+    optional: bool = False
+
+
+@dataclass
+class Runtime:
+    """Where and in which element type a model computes."""
+    device: torch.device
+    dtype: torch.dtype                  # torch.float32 or torch.bfloat16: matrices, activations, cache
+
+    @property
+    def is_f32(self) -> bool:
+        return self.dtype == torch.float32
+
+
+@dataclass(frozen=True)
+class KVSpec:
+    """Key/value storage a mixer needs for each sequence.  Layers with equal specs share a
+    group of the cache; a windowed spec keeps the first `sinks` and the last `window`
+    positions of a sequence and gives older pages back."""
+    n_kv_heads: int
+    head_dim: int
+    window: int = 0
+    sinks: int = 0
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """Fixed-size state a mixer keeps for each sequence: one tensor of `shape` per slot,
+    zeroed when the slot is handed out."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class GroupView:
+    """A cache group's part of a step: page table rows of the step's sequences."""
+    table: torch.Tensor                 # int32 [batch, pages]
+
+
+@dataclass
+class LayerCache:
+    """What one scheduled layer sees of the cache in a step."""
+    k_pool: Optional[torch.Tensor] = None     # [pages, kv_heads, 64, head_dim]
+    v_pool: Optional[torch.Tensor] = None
+    table: Optional[torch.Tensor] = None      # int32 [batch, pages]
+    writes: bool = True                       # False: reads the pages another layer wrote
+    state: Optional[torch.Tensor] = None      # [slots, *StateSpec.shape]
+
+
+@dataclass
+class StepContext:
+    """One step's batch, on the device and on the host.
+
+    The step's tokens lie one sequence after the other: token t belongs to sequence
+    tok_seq[t] (index into the step's batch) and stands at position tok_pos[t]."""
+    runtime: Runtime
+    n_tokens: int
+    batch: int
+    ids: torch.Tensor                   # int32 [T]
+    tok_seq: torch.Tensor               # int32 [T]
+    tok_pos: torch.Tensor               # int32 [T]
+    slots: torch.Tensor                 # int32 [B] cache slot of each sequence
+    cu_seqlens: List[int]               # host: token offsets of the sequences, B + 1 entries
+    starts: List[int]                   # host: position of each sequence's first token in this step
+    slot_ids: List[int]                 # host copy of `slots`
+    is_decode: bool                     # every sequence brings exactly one token
+    max_context: int                    # largest position + 1 in the step
+    shared: Dict[object, object] = field(default_factory=dict)   # per-step tables shared by layers
+
+
+class Part:
+    """Base of mixers, feed-forwards, norms and position encodings."""
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return []
+
+    def bind(self, get: Callable[[str], Optional[torch.Tensor]], rt: Runtime) -> None:
+        """Take the tensors named in tensor_specs() from `get` (host tensors as stored in the
+        checkpoint, None for an absent optional one) and keep device copies in the layout
+        the kernels want."""
+        self.rt = rt
+
+
+class Mixer(Part):
+    """Token mixer: forward(ctx, h [T, H] in the runtime's type, cache) -> [T, H]."""
+
+    def kv_spec(self) -> Optional[KVSpec]:
+        return None
+
+    def state_spec(self) -> Optional[StateSpec]:
+        return None
+
+    def forward(self, ctx: StepContext, h: torch.Tensor, cache: LayerCache) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """forward(ctx, h [T, H]) -> [T, H]."""
+
+    def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Norm(Part):
+    """forward(x, delta, rows) -> normed rows in the runtime's type.  `x` is the float32
+    residual stream; a pending `delta` is added to it first (in place)."""
+
+    def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None,
+                rows: Optional[torch.Tensor] = None, write_back: bool = True) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """prepare(ctx) -> whatever the mixer's kernels need for this step's positions."""
+
+    def prepare(self, ctx: StepContext):
+        raise NotImplementedError
+
+
+# ---------------------------------------------------------------------------
+# registries: a kind name -> the class that builds the part from keyword parameters
+# ---------------------------------------------------------------------------
+MIXERS: Dict[str, type] = {}
+FEED_FORWARDS: Dict[str, type] = {}
+NORMS: Dict[str, type] = {}
+POSITIONS: Dict[str, type] = {}
+BLOCKS: Dict[str, type] = {}
+
+
+def _register(table: Dict[str, type], what: str):
+    def deco(name: str):
+        def wrap(cls):
+            table[name] = cls
+            return cls
+        return wrap
+    return deco
+
+
+register_mixer = _register(MIXERS, "mixer")
+register_feed_forward = _register(FEED_FORWARDS, "feed-forward")
+register_norm = _register(NORMS, "norm")
+register_position = _register(POSITIONS, "position encoding")
+register_block = _register(BLOCKS, "block")
+
+
+def make(table: Dict[str, type], what: str, kind: str, **params):
+    if kind not in table:
+        raise KeyError(f"unknown {what} '{kind}'; known: {sorted(table)}")
+    return table[kind](**params)

@@ -1,0 +1,38 @@
+"""Arrangement of a layer's parts.  The pre-norm residual block:
+
+    x += pending;  a = mixer(norm1(x));  x += a;  d = ffn(norm2(x));  pending = d
+
+Each residual sum is done inside the following norm's kernel, in float32, so the
+feed-forward's output is handed on as `pending` and added by whoever norms next
+(reference: the deferred adds of Daisi.Llogos/Inference/ForwardPass.cs:214-252)."""
+from __future__ import annotations
+
+from typing import Callable, List, Optional, Tuple
+
+import torch
+
+from .base import FeedForward, LayerCache, Mixer, Norm, Part, Runtime, StepContext, TensorSpec, register_block
+
+
+@register_block("pre_norm")
+class PreNormBlock(Part):
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm, ffn: FeedForward):
+        self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+
+    def parts(self) -> List[Part]:
+        return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn]
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [s for p in self.parts() for s in p.tensor_specs()]
+
+    def bind(self, get: Callable[[str], Optional[torch.Tensor]], rt: Runtime) -> None:
+        super().bind(get, rt)
+        for p in self.parts():
+            p.bind(get, rt)
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, pending: Optional[torch.Tensor],
+                cache: LayerCache) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+        h = self.mixer_norm.forward(x, pending)
+        a = self.mixer.forward(ctx, h, cache)
+        h = self.ffn_norm.forward(x, a)
+        return x, self.ffn.forward(ctx, h)

@@ -1,0 +1,68 @@
+"""Matrix products with checkpoint matrices: y = x . W^T (+ b), W stored [out, in]
+(reference: Daisi.Llogos/Inference/ForwardPass.cs:890-895)."""
+from __future__ import annotations
+
+from typing import Callable, List, Optional, Sequence
+
+import torch
+
+from ..ops import kernels as K
+from .base import Part, Runtime, TensorSpec
+
+
+class Linear(Part):
+    """One or several checkpoint matrices applied as one product.  Several matrices with
+    the same input width are stacked by rows at bind time ([Wq; Wk; Wv], [Wgate; Wup]), so
+    the output row is the concatenation of their outputs."""
+
+    def __init__(self, names: Sequence[str], in_features: int, out_features: Sequence[int],
+                 bias: bool = False, suffix: str = ".weight"):
+        self.names = list(names)
+        self.in_features = in_features
+        self.out_features = list(out_features)
+        self.has_bias = bias
+        self.weight: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+
+    @property
+    def total_out(self) -> int:
+        return sum(self.out_features)
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        specs = []
+        for n, o in zip(self.names, self.out_features):
+            specs.append(TensorSpec(n + ".weight", (o, self.in_features), "matrix"))
+            if self.has_bias:
+                specs.append(TensorSpec(n + ".bias", (o,), "bias"))
+        return specs
+
+    def bind(self, get: Callable[[str], Optional[torch.Tensor]], rt: Runtime) -> None:
+        super().bind(get, rt)
+        mats = [get(n + ".weight") for n in self.names]
+        self.weight = _to_device(mats, rt.dtype, rt.device)
+        if self.has_bias:
+            self.bias = _to_device([get(n + ".bias") for n in self.names], torch.float32, rt.device)
+
+    def bind_shared(self, weight: torch.Tensor, rt: Runtime) -> None:
+        """Use a matrix that another part already holds on the device (tied embeddings)."""
+        self.rt = rt
+        self.weight = weight
+
+    def forward(self, a: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+                rows_out: Optional[int] = None) -> torch.Tensor:
+        """a [M, in] -> [M, out]; `rows_out` uses only the first rows of the stacked matrix."""
+        w = self.weight if rows_out is None else self.weight[:rows_out]
+        b = self.bias if (self.bias is None or rows_out is None) else self.bias[:rows_out]
+        return K.gemm(a, w, b, out_dtype or self.rt.dtype)
+
+
+def _to_device(parts: List[torch.Tensor], dtype: torch.dtype, device: torch.device) -> torch.Tensor:
+    """Stack host tensors by rows into one device tensor of `dtype` without a second host copy."""
+    rows = sum(p.shape[0] for p in parts)
+    shape = (rows,) + tuple(parts[0].shape[1:])
+    out = torch.empty(shape, dtype=dtype, device=device)
+    r = 0
+    for p in parts:
+        out[r:r + p.shape[0]].copy_(p)       # converts on the device side of the copy
+        r += p.shape[0]
+    return out

@@ -1,0 +1,33 @@
+"""SwiGLU feed-forward: d = (silu(x Wg^T) * (x Wu^T)) Wd^T without biases
+(reference: Daisi.Llogos/Inference/ForwardPass.cs:240-246; silu Daisi.Llogos.Cpu/Silu.cs:9-16).
+Gate and up are one stacked product whose row is [gate | up]."""
+from __future__ import annotations
+
+from typing import Callable, List, Optional
+
+import torch
+
+from ..ops import kernels as K
+from .base import FeedForward, Runtime, StepContext, TensorSpec, register_feed_forward
+from .linear import Linear
+
+
+@register_feed_forward("swiglu")
+class SwiGLU(FeedForward):
+    def __init__(self, prefix: str, hidden: int, intermediate: int):
+        self.prefix = prefix
+        self.hidden, self.intermediate = hidden, intermediate
+        self.gate_up = Linear([prefix + "gate_proj", prefix + "up_proj"], hidden, [intermediate, intermediate])
+        self.down = Linear([prefix + "down_proj"], intermediate, [hidden])
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return self.gate_up.tensor_specs() + self.down.tensor_specs()
+
+    def bind(self, get: Callable[[str], Optional[torch.Tensor]], rt: Runtime) -> None:
+        super().bind(get, rt)
+        self.gate_up.bind(get, rt)
+        self.down.bind(get, rt)
+
+    def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
+        gu = self.gate_up.forward(h)
+        return self.down.forward(K.swiglu(gu))
