@@ -1,0 +1,137 @@
+"""The generation loop above the step function: batches of unequal prompts, stop tokens,
+sequences that end earlier, and as many batches one after another as there are requests.
+
+One sequence of the loop is the reference's (Daisi.Llogos/Inference/TextGenerator.cs:26-121):
+prefill, then sample -> stop check (a sampled stop token ends the sequence and is not
+emitted, :78-79) -> emit -> forward, at most MaxTokens times (:73); statistics as :118-120."""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Callable, Iterator, List, Optional, Sequence, Tuple
+
+from ..cache.pages import pages_for
+from ..sampling.params import GenerationParams
+
+
+@dataclass
+class GenerationResult:
+    tokens: List[List[int]]
+    finish_reasons: List[str]                 # 'stop' (a stop token was drawn) or 'length'
+    prompt_tokens: int = 0
+    generated_tokens: int = 0
+    prefill_seconds: float = 0.0
+    decode_seconds: float = 0.0
+    batches: List[List[int]] = field(default_factory=list)
+
+    @property
+    def prefill_tokens_per_second(self) -> float:
+        return self.prompt_tokens / self.prefill_seconds if self.prefill_seconds > 0 else 0.0
+
+    @property
+    def decode_tokens_per_second(self) -> float:
+        return self.generated_tokens / self.decode_seconds if self.decode_seconds > 0 else 0.0
+
+
+def plan_batches(prompt_lens: Sequence[int], max_new_tokens: int, max_batch: int, pool_pages: int) -> List[List[int]]:
+    """Requests in their order, cut into batches: at most `max_batch` sequences, and the pages
+    all of a batch's sequences can come to hold (prompt + new tokens, rounded up to pages)
+    fit the pool.  A request that cannot fit alone is an error."""
+    if max_batch <= 0:
+        raise ValueError("max_batch must be positive")
+    batches: List[List[int]] = []
+    cur: List[int] = []
+    used = 0
+    for i, n in enumerate(prompt_lens):
+        if n <= 0:
+            raise ValueError(f"request {i} has an empty prompt")
+        need = pages_for(n + max_new_tokens)
+        if need > pool_pages:
+            raise ValueError(f"request {i} needs {need} cache pages ({n} prompt + {max_new_tokens} new tokens), "
+                             f"the cache has {pool_pages}")
+        if cur and (len(cur) >= max_batch or used + need > pool_pages):
+            batches.append(cur)
+            cur, used = [], 0
+        cur.append(i)
+        used += need
+    if cur:
+        batches.append(cur)
+    return batches
+
+
+class Generator:
+    """Drives an engine (anything with alloc_slot, free_slot, step and cache.n_pages) and a
+    sampler (anything with sample(logits, requests, indices, histories) -> ids)."""
+
+    def __init__(self, engine, max_batch: int = 64, synchronize: Optional[Callable[[], None]] = None):
+        self.engine = engine
+        self.max_batch = max_batch
+        self._sync = synchronize or (lambda: None)
+
+    def stop_tokens(self, params: GenerationParams) -> Tuple[int, ...]:
+        if params.stop_tokens is not None:
+            return tuple(params.stop_tokens)
+        spec = getattr(getattr(self.engine, "model", None), "spec", None)
+        return tuple(getattr(spec, "eos_token_ids", ()) or ())
+
+    def generate(self, prompts: Sequence[Sequence[int]], params: GenerationParams, sampler=None,
+                 on_token: Optional[Callable[[int, int], None]] = None) -> GenerationResult:
+        if sampler is None:
+            from ..sampling.sampler import Sampler
+            sampler = Sampler(params, self.stop_tokens(params))
+        stops = set(self.stop_tokens(params))
+        prompts = [list(p) for p in prompts]
+        result = GenerationResult(tokens=[[] for _ in prompts], finish_reasons=["length"] * len(prompts))
+        result.batches = plan_batches([len(p) for p in prompts], params.max_tokens, self.max_batch,
+                                      self.engine.cache.n_pages)
+        for batch in result.batches:
+            self._run_batch(batch, prompts, params, sampler, stops, result, on_token)
+        return result
+
+    def _run_batch(self, batch, prompts, params, sampler, stops, result, on_token) -> None:
+        eng = self.engine
+        slots = {r: eng.alloc_slot() for r in batch}
+        live = list(batch)
+        need_history = params.has_penalties
+        try:
+            if params.max_tokens == 0:
+                return
+            self._sync()
+            t0 = time.perf_counter()
+            logits = eng.step([(slots[r], prompts[r]) for r in live], want="last")
+            ids = self._sample(sampler, logits, live, prompts, result, need_history)
+            t1 = time.perf_counter()
+            result.prefill_seconds += t1 - t0
+            result.prompt_tokens += sum(len(prompts[r]) for r in live)
+            while True:
+                nxt = []
+                for r, tok in zip(live, ids):
+                    if tok in stops:
+                        result.finish_reasons[r] = "stop"
+                        eng.free_slot(slots.pop(r))          # an ended sequence gives its pages back at once
+                        continue
+                    result.tokens[r].append(tok)
+                    result.generated_tokens += 1
+                    if on_token is not None:
+                        on_token(r, tok)
+                    if len(result.tokens[r]) >= params.max_tokens:
+                        eng.free_slot(slots.pop(r))
+                        continue
+                    nxt.append((r, tok))
+                if not nxt:
+                    break
+                live = [r for r, _ in nxt]
+                logits = eng.step([(slots[r], [tok]) for r, tok in nxt], want="last")
+                ids = self._sample(sampler, logits, live, prompts, result, need_history)
+            self._sync()
+            result.decode_seconds += time.perf_counter() - t1
+        finally:
+            for r in list(slots):
+                eng.free_slot(slots.pop(r))
+
+    @staticmethod
+    def _sample(sampler, logits, live, prompts, result, need_history) -> List[int]:
+        indices = [len(result.tokens[r]) for r in live]
+        histories = [prompts[r] + result.tokens[r] for r in live] if need_history else None
+        ids = sampler.sample(logits, live, indices, histories)
+        return [int(t) for t in (ids.tolist() if hasattr(ids, "tolist") else ids)]

@@ -7,7 +7,7 @@ tensors used as device memory; launches go to torch's current stream.
 from __future__ import annotations
 
 import ctypes
-from typing import Optional
+from typing import Optional, Sequence
 
 import torch
 
@@ -231,3 +231,48 @@ def attention(ctx, q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool:
     """Attention of the step's query rows over the cache pages of their sequences."""
     return attention_generic(q, q_stride, k_pool, v_pool, table, ctx.tok_seq, ctx.tok_pos,
                              n_heads, n_kv_heads, head_dim, scale, window, sinks)
+
+
+# ----------------------------------------------------------------------------
+# sampling
+# ----------------------------------------------------------------------------
+def sample_prepare(logits: torch.Tensor, history: Optional[torch.Tensor], history_len: Optional[torch.Tensor],
+                   repetition: float, frequency: float, presence: float, temperature: float,
+                   penalize_newline: bool, banned: Sequence[int] = ()) -> torch.Tensor:
+    """A copy of float32 logits [R, V] with penalties over each row's recent tokens
+    (`history` int32 [R, W], `history_len` int32 [R]), banned ids at -inf, times 1/temperature."""
+    _dev(logits, history, history_len)
+    _i32(history, "history"); _i32(history_len, "history_len")
+    _need(logits.dtype == torch.float32 and logits.dim() == 2, "sample_prepare: logits must be float32 [R, V]")
+    _need(len(banned) <= 8, "sample_prepare: at most 8 banned ids")
+    R, V = logits.shape
+    if history is not None:
+        _need(history.dim() == 2 and history.shape[0] == R and history_len is not None
+              and history_len.numel() == R, "sample_prepare: history [R, W] with lengths [R]")
+    work = torch.empty_like(logits)
+    ban = (ctypes.c_int * 8)(*list(banned))
+    inv_t = 1.0 / temperature if temperature > 0 else 1.0
+    _check(_lib().llogos_sample_prepare(
+        _p(work), _p(logits), R, V, _p(history), _p(history_len), history.stride(0) if history is not None else 0,
+        ctypes.c_float(repetition), ctypes.c_float(frequency), ctypes.c_float(presence), ctypes.c_float(inv_t),
+        int(penalize_newline), ban, len(banned), _stream()), "sample_prepare")
+    return work
+
+
+def sample_pipeline(work: torch.Tensor, uniforms: torch.Tensor, top_k: int, top_p: float, min_p: float,
+                    typical_p: float, min_keep: int) -> torch.Tensor:
+    """Token ids int32 [R] drawn from prepared rows `work` (overwritten) with one uniform
+    number per row: top-k, min-p, softmax, typical-p, top-p, draw."""
+    _dev(work, uniforms)
+    _need(work.dtype == torch.float32 and work.dim() == 2, "sample_pipeline: work must be float32 [R, V]")
+    R, V = work.shape
+    _need(uniforms.dtype == torch.float32 and uniforms.numel() == R, "sample_pipeline: one float32 uniform per row")
+    n_pad = 1
+    while n_pad < V:
+        n_pad <<= 1
+    scratch = torch.empty((R, n_pad), dtype=torch.int64, device=work.device)
+    out = torch.empty((R,), dtype=torch.int32, device=work.device)
+    _check(_lib().llogos_sample_pipeline(
+        _p(out), _p(work), R, V, _p(scratch), n_pad, _p(uniforms), int(top_k), ctypes.c_float(top_p),
+        ctypes.c_float(min_p), ctypes.c_float(typical_p), int(min_keep), _stream()), "sample_pipeline")
+    return out

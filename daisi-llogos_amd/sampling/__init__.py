@@ -1,0 +1,3 @@
+from .params import GenerationParams
+from .rng import uniform
+from .sampler import Sampler

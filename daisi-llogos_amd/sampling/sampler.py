@@ -1,0 +1,54 @@
+"""Token selection for a batch of logit rows, on the device.
+
+The pipeline is the reference's (Daisi.Llogos/Inference/Sampler.cs:26-85): greedy short cut,
+penalties, temperature, top-k, min-p, softmax over candidates, typical-p, top-p, draw."""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..ops import kernels as K
+from .params import GenerationParams
+from .rng import uniform
+
+
+class Sampler:
+    def __init__(self, params: GenerationParams, stop_tokens: Sequence[int] = ()):
+        self.params = params
+        self.stop_tokens = tuple(stop_tokens)
+        self._fresh_seed = None
+        if params.seed is None and params.temperature > 0:
+            self._fresh_seed = int(np.random.SeedSequence().generate_state(1)[0])
+
+    def uniforms(self, requests: Sequence[int], indices: Sequence[int]) -> List[float]:
+        seed = self.params.seed if self.params.seed is not None else self._fresh_seed
+        return [uniform(seed, r, i) for r, i in zip(requests, indices)]
+
+    def sample(self, logits: torch.Tensor, requests: Sequence[int], indices: Sequence[int],
+               histories: Optional[Sequence[Sequence[int]]] = None) -> torch.Tensor:
+        """int32 token ids [R] for float32 logits [R, V].  requests/indices: which request each
+        row belongs to and which of its generated tokens this is (for the random stream);
+        histories: each row's prompt + generated tokens (for penalties)."""
+        p = self.params
+        if p.is_greedy:
+            return K.argmax(logits)
+        hist = hist_len = None
+        if p.has_penalties:
+            if histories is None:
+                raise ValueError("penalties need each row's token history")
+            win = [list(h[-p.penalty_count:]) if 0 < p.penalty_count < len(h) else list(h) for h in histories]
+            width = max(1, max(len(w) for w in win))
+            arr = np.zeros((len(win), width), dtype=np.int32)
+            for i, w in enumerate(win):
+                arr[i, :len(w)] = w
+            hist = torch.from_numpy(arr).to(logits.device)
+            hist_len = torch.tensor([len(w) for w in win], dtype=torch.int32, device=logits.device)
+        banned = self.stop_tokens[:8] if p.prevent_eos else ()
+        work = K.sample_prepare(logits, hist, hist_len, p.repetition_penalty, p.frequency_penalty,
+                                p.presence_penalty, p.temperature, p.penalize_newline, banned)
+        if p.temperature == 0:
+            return K.argmax(work)
+        u = torch.tensor(self.uniforms(requests, indices), dtype=torch.float32, device=logits.device)
+        return K.sample_pipeline(work, u, p.top_k, p.top_p, p.min_p, p.typical_p, p.min_keep)

@@ -1,0 +1,55 @@
+"""The command line's options carry the reference's names and defaults
+(Daisi.Llogos.Cli/Program.cs:444-530, 800-827)."""
+import importlib
+
+import pytest
+
+cli = importlib.import_module("daisi-llogos_amd.__main__")
+api = importlib.import_module("daisi-llogos_amd.api")
+
+
+def test_defaults():
+    a = cli.parse_args(["--model", "m", "--prompt", "1 2"])
+    assert (a.max_tokens, a.max_context, a.temperature, a.top_k, a.top_p, a.repeat_penalty) == \
+           (256, 2048, 0.7, 40, 0.9, 1.1)
+    assert a.seed is None and not a.bench and a.attention == "full"
+
+
+def test_short_and_long_names():
+    a = cli.parse_args(["-m", "dir", "-p", "5,6", "-n", "7", "-t", "0", "--top-k", "3", "--top-p", "0.5",
+                        "--repeat-penalty", "1.0", "--seed", "9", "--max-context", "128", "--bench", "-b", "hip"])
+    assert (a.model, a.prompt, a.max_tokens, a.temperature, a.top_k, a.top_p) == ("dir", "5,6", 7, 0.0, 3, 0.5)
+    assert (a.repeat_penalty, a.seed, a.max_context, a.bench, a.backend) == (1.0, 9, 128, True, "hip")
+    with pytest.raises(ValueError, match="Missing value"):
+        cli.parse_args(["--model"])
+    with pytest.raises(ValueError, match="unknown"):
+        cli.parse_args(["--frobnicate"])
+
+
+def test_exit_codes(tmp_path, capsys):
+    assert cli.main(["--prompt", "1"]) == 1                             # no model
+    assert cli.main(["--model", str(tmp_path / "nope"), "--prompt", "1"]) == 1
+    assert cli.main(["--model", str(tmp_path)]) == 1                    # no prompt and no --bench
+    assert cli.main(["--model", str(tmp_path), "--prompt", "1", "--backend", "cuda"]) == 1
+    assert cli.main(["--help"]) == 0
+    assert "--repeat-penalty" in capsys.readouterr().err
+
+
+def test_prompts(tmp_path):
+    assert cli.parse_prompts("1 2 3", ".") == [[1, 2, 3]]
+    assert cli.parse_prompts("1,2; 3 4 ;5", ".") == [[1, 2], [3, 4], [5]]
+    f = tmp_path / "p.txt"
+    f.write_text("7 8\n9")
+    assert cli.parse_prompts("@" + str(f), ".") == [[7, 8, 9]]
+    with pytest.raises(ValueError, match="tokenizer"):
+        cli.parse_prompts("hello there", str(tmp_path))
+
+
+def test_attention_strategy_strings():
+    # Daisi.Llogos/Inference/AttentionStrategy.cs:75-100
+    assert api.parse_attention("full") == (None, 0)
+    assert api.parse_attention("window:128") == (128, 0)
+    assert api.parse_attention("sinks:4,60") == (64, 4)
+    for bad in ("window:0", "sinks:4", "ring", "sinks:-1,5"):
+        with pytest.raises(ValueError):
+            api.parse_attention(bad)

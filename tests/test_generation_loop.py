@@ -1,0 +1,157 @@
+"""The generation loop's decisions, with a stand-in engine: batching, stop tokens, sequences
+that end earlier, slots given back and used again."""
+import importlib
+
+import numpy as np
+import pytest
+
+gen = importlib.import_module("daisi-llogos_amd.engine.generate")
+kvc = importlib.import_module("daisi-llogos_amd.cache.kv_cache")
+base = importlib.import_module("daisi-llogos_amd.parts.base")
+params_mod = importlib.import_module("daisi-llogos_amd.sampling.params")
+GenerationParams = params_mod.GenerationParams
+
+VOCAB = 50
+
+
+class FakeEngine:
+    """Next token = (sum of the sequence's tokens so far) % VOCAB; the cache is the real
+    bookkeeping without device memory."""
+
+    def __init__(self, max_tokens=64 * 8, n_slots=2):
+        self.cache = kvc.Cache([(base.KVSpec(1, 16), None)], [None], max_tokens, rt=None, n_slots=n_slots)
+        self.sums = {}
+        self.log = []
+
+    def alloc_slot(self):
+        s = self.cache.alloc_slot()
+        self.sums[s] = 0
+        return s
+
+    def free_slot(self, s):
+        self.cache.free_slot(s)
+        del self.sums[s]
+
+    def step(self, entries, want="last"):
+        assert want == "last"
+        slots = [s for s, _ in entries]
+        lens = [self.cache.length(s) + len(t) for s, t in entries]
+        self.cache.reserve(slots, lens)
+        self.cache.commit(slots, lens)
+        self.log.append([(s, len(t)) for s, t in entries])
+        out = np.full((len(entries), VOCAB), -1.0, dtype=np.float32)
+        for i, (s, t) in enumerate(entries):
+            self.sums[s] += sum(t)
+            out[i, self.sums[s] % VOCAB] = 1.0
+        return out
+
+
+class ArgmaxSampler:
+    def sample(self, logits, requests, indices, histories):
+        self.last = (list(requests), list(indices))
+        return np.argmax(logits, axis=-1)
+
+
+def expected(prompt, n, stops=()):
+    seq, out = list(prompt), []
+    for _ in range(n):
+        t = sum(seq) % VOCAB
+        if t in stops:
+            return out, "stop"
+        out.append(t)
+        seq.append(t)
+    return out, "length"
+
+
+def test_plan_batches():
+    assert gen.plan_batches([5, 5, 5, 5, 5], 10, 2, 100) == [[0, 1], [2, 3], [4]]
+    # pages: 70 + 10 -> 2 pages each, the pool has 5
+    assert gen.plan_batches([70, 70, 70], 10, 8, 5) == [[0, 1], [2]]
+    with pytest.raises(ValueError, match="cache"):
+        gen.plan_batches([70, 600], 10, 8, 5)
+    with pytest.raises(ValueError, match="empty"):
+        gen.plan_batches([3, 0], 10, 8, 5)
+
+
+def test_unequal_prompts_lengths_and_stops():
+    eng = FakeEngine()
+    g = gen.Generator(eng, max_batch=8)
+    prompts = [[1, 2, 3], [7], [4, 4, 4, 4, 4, 4], [9, 9]]
+    stops = (13, 30)
+    res = g.generate(prompts, GenerationParams.greedy(max_tokens=12, stop_tokens=stops), sampler=ArgmaxSampler())
+    for p, toks, why in zip(prompts, res.tokens, res.finish_reasons):
+        want, reason = expected(p, 12, stops)
+        assert toks == want and why == reason
+        assert not set(toks) & set(stops)                              # a stop token is never emitted
+    assert {"stop", "length"} <= set(res.finish_reasons) or len(set(res.finish_reasons)) == 1
+    assert res.prompt_tokens == 12 and res.generated_tokens == sum(len(t) for t in res.tokens)
+    assert eng.cache.live_slots == [] and eng.cache.free_pages() == [8]
+    # the first step holds all prompts whole, later steps one token for each live sequence
+    assert eng.log[0] == [(0, 3), (1, 1), (2, 6), (3, 2)]
+    assert all(n == 1 for step in eng.log[1:] for _, n in step)
+    sizes = [len(step) for step in eng.log]
+    assert sizes == sorted(sizes, reverse=True)                        # the batch only shrinks
+
+
+def test_ended_sequences_leave_and_slots_are_used_again():
+    eng = FakeEngine(n_slots=2)
+    g = gen.Generator(eng, max_batch=2)
+    prompts = [[1], [2, 2], [3, 3, 3], [5], [8, 1]]
+    res = g.generate(prompts, GenerationParams.greedy(max_tokens=5, stop_tokens=(4,)), sampler=ArgmaxSampler())
+    assert res.batches == [[0, 1], [2, 3], [4]]
+    for p, toks, why in zip(prompts, res.tokens, res.finish_reasons):
+        assert (toks, why) == expected(p, 5, (4,))
+    assert {s for step in eng.log for s, _ in step} == {0, 1}           # two slots serve five requests
+    assert eng.cache.slots.n_slots == 2 and eng.cache.live_slots == []
+
+
+def test_max_tokens_zero_and_one():
+    eng = FakeEngine()
+    g = gen.Generator(eng)
+    res = g.generate([[1, 2]], GenerationParams.greedy(max_tokens=0), sampler=ArgmaxSampler())
+    assert res.tokens == [[]] and eng.log == []
+    res = g.generate([[1, 2]], GenerationParams.greedy(max_tokens=1, stop_tokens=()), sampler=ArgmaxSampler())
+    assert res.tokens == [[3]] and len(eng.log) == 1                    # no step after the last token
+
+
+def test_sampler_sees_request_and_token_index():
+    eng = FakeEngine()
+    s = ArgmaxSampler()
+    gen.Generator(eng).generate([[1], [2], [3]], GenerationParams.greedy(max_tokens=3, stop_tokens=(4,)), sampler=s)
+    # request 1 (prompt [2]) draws 2, then 4 = stop: at the last step only requests 0 and 2 are live
+    assert s.last == ([0, 2], [2, 2])
+
+
+def test_slots_are_given_back_when_a_step_fails():
+    eng = FakeEngine(max_tokens=64 * 2)
+    g = gen.Generator(eng)
+
+    class Boom(Exception):
+        pass
+
+    def bad(entries, want="last"):
+        raise Boom()
+    eng.step = bad
+    with pytest.raises(Boom):
+        g.generate([[1, 2, 3]], GenerationParams.greedy(max_tokens=4), sampler=ArgmaxSampler())
+    assert eng.cache.live_slots == []
+
+
+def test_params_follow_the_reference_defaults():
+    p = GenerationParams()
+    assert (p.max_tokens, p.temperature, p.top_k, p.top_p, p.repetition_penalty) == (256, 0.8, 40, 0.95, 1.1)
+    assert (p.penalty_count, p.min_keep, p.typical_p, p.min_p) == (64, 1, 1.0, 0.0)
+    assert not p.is_greedy and GenerationParams.greedy().is_greedy
+    assert not GenerationParams(temperature=0).is_greedy               # penalties still apply
+    with pytest.raises(ValueError):
+        GenerationParams(temperature=-1)
+
+
+def test_uniform_stream_is_per_request():
+    rng = importlib.import_module("daisi-llogos_amd.sampling.rng")
+    a = [rng.uniform(7, 2, i) for i in range(50)]
+    assert a == [rng.uniform(7, 2, i) for i in range(50)]
+    assert all(0 <= u < 1 for u in a) and len(set(a)) == 50
+    assert a != [rng.uniform(8, 2, i) for i in range(50)] and a != [rng.uniform(7, 3, i) for i in range(50)]
+    us = [rng.uniform(1, r, i) for r in range(40) for i in range(50)]
+    assert abs(sum(us) / len(us) - 0.5) < 0.02
