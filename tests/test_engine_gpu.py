@@ -1,0 +1,202 @@
+"""The engine against the plain implementation, in float32 and in bfloat16: each request
+alone and whole; the last 32 tokens one by one; batches of unequal lengths whose shorter
+requests end earlier, one batch after another so that slots and pages are used again;
+long decoding; the first tokens of a sequence; greedy generation through the entry point."""
+import numpy as np
+import pytest
+import torch
+
+import gpu_helpers as H
+import plain_model as pm
+import tiny_configs as tc
+
+pytestmark = pytest.mark.gpu
+CONFIGS = ["tiny_a", "tiny_b", "tiny_c", "tiny_w"]
+
+
+def _np(t):
+    return t.detach().cpu().double().numpy()
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+@pytest.mark.parametrize("name", CONFIGS)
+def test_whole_requests(name, dtype):
+    eng = H.engine(name, dtype)
+    for n, seed in ((5, 1), (17, 2), (1, 3), (32, 4), (100, 5)):
+        toks = H.tokens(name, n, seed)
+        s = eng.alloc_slot()
+        got = _np(eng.step([(s, toks)], want="all"))
+        eng.free_slot(s)
+        H.close(got, H.plain_logits(name, toks), dtype, f"{name} whole n={n}")
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+@pytest.mark.parametrize("name", CONFIGS)
+def test_last_32_tokens_one_by_one(name, dtype):
+    eng = H.engine(name, dtype)
+    toks = H.tokens(name, 120, 7)
+    want = H.plain_logits(name, toks)
+    s = eng.alloc_slot()
+    rows = [_np(eng.step([(s, toks[:88])], want="all"))]
+    for t in toks[88:]:
+        rows.append(_np(eng.step([(s, [t])], want="last")))
+    got = np.concatenate(rows)
+    H.close(got, want, dtype, f"{name} decode")
+    # the same positions in one step: cutting changes nothing beyond rounding
+    s2 = eng.alloc_slot()
+    whole = _np(eng.step([(s2, toks)], want="all"))
+    tol = 1e-5 if dtype == "float32" else H.TOL[dtype]
+    assert np.abs(whole - got).max() <= tol
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+@pytest.mark.parametrize("name", CONFIGS)
+def test_unequal_batches_one_after_another(name, dtype):
+    """Batches of unequal prompts; shorter requests end earlier; the pool is so small that
+    the next batch must take the slots and pages the last one gave back."""
+    eng = H.engine(name, dtype, max_tokens=64 * 5, n_slots=4)
+    plans = [
+        [(5, 16), (17, 3), (1, 9), (32, 12)],       # (prompt length, decoded tokens) per request
+        [(40, 24), (3, 5), (9, 30)],
+        [(64, 2), (63, 1), (60, 30)],          # 2 + 1 + 2 pages: the pool is full at the end
+    ]
+    seed = 20
+    for plan in plans:
+        reqs = []
+        for n_prompt, n_dec in plan:
+            seed += 1
+            toks = H.tokens(name, n_prompt + n_dec, seed)
+            reqs.append(dict(toks=toks, n_prompt=n_prompt, slot=eng.alloc_slot(), rows=[], fed=0))
+        assert sorted(r["slot"] for r in reqs) == list(range(len(reqs)))       # slots are used again
+        out = eng.step([(r["slot"], r["toks"][:r["n_prompt"]]) for r in reqs], want="all")
+        o = 0
+        for r in reqs:
+            r["rows"].append(_np(out[o:o + r["n_prompt"]]))
+            o += r["n_prompt"]
+            r["fed"] = r["n_prompt"]
+        live = list(reqs)
+        while live:
+            for r in [r for r in live if r["fed"] == len(r["toks"])]:
+                eng.free_slot(r["slot"])                                         # ends earlier than the others
+                live.remove(r)
+            if not live:
+                break
+            out = eng.step([(r["slot"], [r["toks"][r["fed"]]]) for r in live], want="last")
+            for i, r in enumerate(live):
+                r["rows"].append(_np(out[i:i + 1]))
+                r["fed"] += 1
+        for r in reqs:
+            H.close(np.concatenate(r["rows"]), H.plain_logits(name, r["toks"]), dtype,
+                    f"{name} batch request of {len(r['toks'])}")
+        assert eng.cache.live_slots == [] and eng.cache.free_pages() == [5] * len(eng.cache.groups)
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+def test_batch_composition_and_slot_do_not_change_float_results(dtype):
+    """A request alone in slot 0 and the same request last in a batch, in another slot and in
+    other pages: equal logits (each row's arithmetic is its own)."""
+    name = "tiny_a"
+    eng = H.engine(name, dtype, n_slots=8)
+    toks = H.tokens(name, 70, 31)
+    s = eng.alloc_slot()
+    alone = [_np(eng.step([(s, toks[:50])], want="all"))] + [_np(eng.step([(s, [t])])) for t in toks[50:]]
+    eng.free_slot(s)
+    others = [H.tokens(name, n, 40 + n) for n in (90, 3, 66)]
+    slots = [eng.alloc_slot() for _ in range(4)]
+    out = eng.step([(slots[i], o) for i, o in enumerate(others)] + [(slots[3], toks[:50])],
+                   want=[[], [], [], list(range(50))])
+    mixed = [_np(out)]
+    for i, t in enumerate(toks[50:]):
+        batch = [(slots[j], [others[j][(i + j) % len(others[j])]]) for j in range(3)] + [(slots[3], [t])]
+        mixed.append(_np(eng.step(batch, want=[[], [], [], [0]])))
+    a, b = np.concatenate(alone), np.concatenate(mixed)
+    assert np.array_equal(a, b), f"max difference {np.abs(a - b).max()}"
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+@pytest.mark.parametrize("name", ["tiny_c", "tiny_w"])
+def test_long_decoding(name, dtype):
+    """300 positions, most of them decoded one by one: crosses page borders, and in the
+    windowed configuration pages leave the window and are given back meanwhile."""
+    eng = H.engine(name, dtype, max_tokens=64 * 6, n_slots=1)
+    toks = H.tokens(name, 300, 9)
+    want = H.plain_logits(name, toks)
+    s = eng.alloc_slot()
+    rows = [_np(eng.step([(s, toks[:3])], want="all"))]
+    for t in toks[3:]:
+        rows.append(_np(eng.step([(s, [t])], want="last")))
+    H.close(np.concatenate(rows), want, dtype, f"{name} long decode")
+    if name == "tiny_w":
+        assert eng.cache.free_pages()[1] > eng.cache.free_pages()[0]           # the window group gave pages back
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+@pytest.mark.parametrize("name", CONFIGS)
+def test_first_tokens(name, dtype):
+    eng = H.engine(name, dtype)
+    toks = H.tokens(name, 6, 13)
+    want = H.plain_logits(name, toks)
+    s = eng.alloc_slot()
+    rows = [_np(eng.step([(s, [t])], want=[[0]])) for t in toks]               # from the very first token on
+    H.close(np.concatenate(rows), want, dtype, f"{name} first tokens")
+    s2 = eng.alloc_slot()
+    assert eng.step([(s2, toks[:2])], want=None) is None                       # nothing wanted: no logits
+    got = _np(eng.step([(s2, toks[2:])], want=[[3, 0]]))                       # places in the asked order
+    H.close(got, want[[5, 2]], dtype, f"{name} wanted places")
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+def test_window_and_sinks_as_run_time_strategy(dtype):
+    name = "tiny_a"
+    cfg, w = H.plain(name)
+    toks = H.tokens(name, 100, 17)
+    want = pm.forward(cfg, w, list(toks), window=24, sinks=3)
+    eng = H.engine(name, dtype, attention_window=24, attention_sinks=3)
+    s = eng.alloc_slot()
+    rows = [_np(eng.step([(s, toks[:70])], want="all"))] + [_np(eng.step([(s, [t])])) for t in toks[70:]]
+    H.close(np.concatenate(rows), want, dtype, "window 24 sinks 3")
+    assert np.abs(want - H.plain_logits(name, toks)).max() > 1e-3              # the window matters here
+
+
+def test_step_errors():
+    eng = H.engine("tiny_a", "float32", max_tokens=128, n_slots=2)
+    s = eng.alloc_slot()
+    with pytest.raises(H.llogos.StepError, match="token id"):
+        eng.step([(s, [256])])
+    with pytest.raises(H.llogos.StepError, match="at least one token"):
+        eng.step([(s, [])])
+    with pytest.raises(H.llogos.StepError, match="twice"):
+        eng.step([(s, [1]), (s, [2])])
+    with pytest.raises(H.llogos.StepError, match="outside"):
+        eng.step([(s, [1, 2])], want=[[2]])
+    with pytest.raises(H.llogos.CacheError):
+        eng.step([(5, [1])])
+    with pytest.raises(H.llogos.CacheFull):
+        eng.step([(s, list(range(129)))])
+    assert eng.cache.length(s) == 0 and eng.cache.free_pages() == [2]          # refused steps change nothing
+    eng.step([(s, [1, 2, 3])])
+    assert eng.cache.length(s) == 3
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+@pytest.mark.parametrize("name", ["tiny_a", "tiny_b"])
+def test_greedy_generation_through_the_entry_point(name, dtype):
+    cfg, w = H.plain(name)
+    prompts = [list(H.tokens(name, n, 50 + n)) for n in (5, 17, 1, 32, 8)]
+    llm = H.llogos.Llogos(H.folder(name), dtype=dtype, max_context=64, max_batch=3)
+    res = llm.generate(prompts, max_tokens=12, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0,
+                       stop_tokens=())
+    assert res.batches == [[0, 1, 2], [3, 4]] and all(len(t) == 12 for t in res.tokens)
+    for p, toks in zip(prompts, res.tokens):
+        logits = pm.forward(cfg, w, p + toks)
+        for i, t in enumerate(toks):
+            row = logits[len(p) + i - 1]
+            # the chosen token is the plain implementation's maximum, up to the dtype's rounding
+            assert row.max() - row[t] <= (0 if dtype == "float32" else 2 * H.TOL[dtype]), (name, dtype, i)
+    # stop tokens end a sequence and are not emitted
+    first = res.tokens[0]
+    res2 = llm.generate([prompts[0]], max_tokens=12, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0,
+                        stop_tokens=(first[4],))
+    cut = first.index(first[4])
+    assert res2.tokens[0] == first[:cut] and res2.finish_reasons == ["stop"]
+    assert llm.engine.cache.live_slots == []
