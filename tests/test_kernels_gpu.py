@@ -1,0 +1,271 @@
+"""Each kernel alone against a plain float64 / torch reference of the same op, at sizes
+other than the engine's tests use (head sizes in steps of 16, widths and vocabularies that
+are no power of two, many heads and groups)."""
+import importlib
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_model as pm
+
+pytestmark = pytest.mark.gpu
+K = importlib.import_module("daisi-llogos_amd.ops.kernels")
+DEV = "cuda:0"
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+RT = {"float32": 2e-6, "bfloat16": 1e-2}        # relative to the result's scale
+
+
+def _t(a, dtype=torch.float32):
+    return torch.tensor(np.asarray(a), dtype=dtype, device=DEV)
+
+
+def _np(t):
+    return t.detach().cpu().double().numpy()
+
+
+def _close(got, want, dtype, scale=None):
+    want = np.asarray(want, dtype=np.float64)
+    scale = scale if scale is not None else max(1e-6, np.abs(want).max())
+    err = np.abs(_np(got) - want).max() / scale
+    assert err <= RT[dtype], f"relative error {err:.3e} > {RT[dtype]}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embed(dtype):
+    rng = np.random.default_rng(0)
+    table = _t(rng.standard_normal((331, 200)), DT[dtype])
+    ids = _t([0, 330, 7, 7, 129], torch.int32)
+    out = K.embed(table, ids)
+    assert out.dtype == torch.float32 and torch.equal(out, table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H", [80, 1000, 4100])
+def test_rmsnorm(dtype, H):
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal((7, H)) * 3
+    d = rng.standard_normal((7, H))
+    w = 1 + 0.1 * rng.standard_normal(H)
+    xd, dd, wd = _t(x), _t(d, DT[dtype]), _t(w)
+    want = pm.rms_norm(x, w, 1e-5)
+    _close(K.rmsnorm(xd, wd, 1e-5, DT[dtype]), want, dtype)
+    # with a pending delta: the sum is written back in float32 and the norm is of the sum
+    xs = x + _np(dd)
+    out = K.rmsnorm(xd, wd, 1e-5, DT[dtype], delta=dd)
+    assert np.abs(_np(xd) - xs).max() < 1e-6
+    _close(out, pm.rms_norm(xs, w, 1e-5), dtype)
+    # selected rows, no write back
+    x2 = _t(x)
+    rows = _t([6, 0, 3], torch.int32)
+    out = K.rmsnorm(x2, wd, 1e-5, DT[dtype], delta=dd, rows=rows, write_back=False)
+    assert torch.equal(x2, _t(x))
+    _close(out, pm.rms_norm(xs[[6, 0, 3]], w, 1e-5), dtype)
+    z = K.rmsnorm(torch.zeros(2, H, device=DEV), wd, 1e-6, DT[dtype])
+    assert torch.count_nonzero(z) == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("M,N,K_", [(1, 331, 80), (5, 96, 1000), (70, 130, 67), (200, 257, 129)])
+def test_gemm(dtype, M, N, K_):
+    rng = np.random.default_rng(2)
+    a = _t(rng.standard_normal((M, K_)), DT[dtype])
+    w = _t(rng.standard_normal((N, K_)) * 0.1, DT[dtype])
+    b = _t(rng.standard_normal(N))
+    want = pm.linear(_np(a), _np(w), _np(b))
+    _close(K.gemm(a, w, b, DT[dtype]), want, dtype)
+    _close(K.gemm(a, w, None, torch.float32), pm.linear(_np(a), _np(w)), "float32" if dtype == "float32" else dtype)
+    # a view with a row stride (the first columns of a wider buffer) and the first rows of w
+    wide = _t(rng.standard_normal((M, K_ + 13)), DT[dtype])
+    _close(K.gemm(wide[:, :K_], w[:N // 2], None, DT[dtype]), pm.linear(_np(wide)[:, :K_], _np(w)[:N // 2]), dtype)
+    # reference vector (tests/Daisi.Llogos.Tests/Cpu/MathOpsTests.cs:10-28)
+    o = K.gemm(_t([[1, 2, 3], [4, 5, 6]], DT[dtype]), _t([[7, 9, 11], [8, 10, 12]], DT[dtype]), None, torch.float32)
+    assert _np(o).tolist() == [[58, 64], [139, 154]]
+
+
+def test_rope_table_is_double_precision():
+    pos = _t([0, 1, 4095, 100000], torch.int32)
+    f = pm.rope_frequencies(64, 5e5)
+    cs = _np(K.rope_table(pos, _t(f, torch.float64)))
+    ang = np.array([0, 1, 4095, 100000])[:, None] * f[None, :]
+    assert np.abs(cs[..., 0] - np.cos(ang)).max() < 1e-7 and np.abs(cs[..., 1] - np.sin(ang)).max() < 1e-7
+
+
+def _pages(n_seqs, max_len, rng):
+    """A shuffled page table: sequences' pages lie anywhere in the pool."""
+    per = (max_len + 63) // 64
+    ids = rng.permutation(n_seqs * per + 3)[:n_seqs * per].reshape(n_seqs, per)
+    return ids.astype(np.int32), n_seqs * per + 3
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,hd,rot,pairing,norm", [
+    (4, 2, 16, 16, 0, False), (6, 1, 32, 32, 0, True), (5, 5, 48, 24, 0, True), (8, 2, 80, 80, 1, False),
+    (3, 3, 128, 64, 1, True), (2, 1, 256, 256, 0, False)])
+def test_qk_rope_cache(dtype, nh, nkv, hd, rot, pairing, norm):
+    rng = np.random.default_rng(3)
+    lens = [70, 3]                                      # two sequences; this step brings the last 5 and 3 tokens
+    new = [5, 3]
+    T = sum(new)
+    tok_seq = np.repeat(np.arange(2), new).astype(np.int32)
+    tok_pos = np.concatenate([np.arange(l - n, l) for l, n in zip(lens, new)]).astype(np.int32)
+    table, n_pages = _pages(2, 70, rng)
+    qkv = _t(rng.standard_normal((T, (nh + 2 * nkv) * hd)), DT[dtype])
+    orig = _np(qkv)
+    qw = 1 + 0.1 * rng.standard_normal(hd)
+    kw = 1 + 0.1 * rng.standard_normal(hd)
+    f = pm.rope_frequencies(rot, 1e4)
+    cs = K.rope_table(_t(tok_pos, torch.int32), _t(f, torch.float64))
+    kp = torch.zeros((n_pages, nkv, 64, hd), dtype=DT[dtype], device=DEV)
+    vp = torch.zeros_like(kp)
+    K.qk_rope_cache(qkv, nh, nkv, hd, rot, pairing, _t(qw) if norm else None, _t(kw) if norm else None, 1e-5,
+                    cs, kp, vp, _t(table, torch.int32), _t(tok_seq, torch.int32), _t(tok_pos, torch.int32))
+    q, k, v = orig[:, :nh * hd], orig[:, nh * hd:(nh + nkv) * hd], orig[:, (nh + nkv) * hd:]
+    if norm:
+        q = pm.per_head_rms_norm(q, qw, nh, hd, 1e-5)
+        k = pm.per_head_rms_norm(k, kw, nkv, hd, 1e-5)
+    rope = pm.rope_split_half if pairing == 0 else pm.rope_interleaved
+    q, k = rope(q, tok_pos, nh, hd, f), rope(k, tok_pos, nkv, hd, f)
+    _close(qkv[:, :nh * hd], q, dtype)
+    kc, vc = _np(kp), _np(vp)
+    for t in range(T):
+        page = table[tok_seq[t], tok_pos[t] // 64]
+        got_k = kc[page, :, tok_pos[t] % 64, :].reshape(-1)
+        got_v = vc[page, :, tok_pos[t] % 64, :].reshape(-1)
+        assert np.abs(got_k - k[t]).max() <= RT[dtype] * max(1, np.abs(k).max())
+        assert np.abs(got_v - v[t]).max() <= RT[dtype] * max(1, np.abs(v).max())
+    assert np.count_nonzero(kc) == T * nkv * hd                         # nothing else was written
+
+
+def _attention_case(dtype, nh, nkv, hd, lens, new, window=0, sinks=0, seed=4, scale_q=1.0):
+    """Fills a paged cache with random keys and values for sequences of `lens` positions, of
+    which the last `new` are this step's queries; returns the kernel's and the plain result."""
+    rng = np.random.default_rng(seed)
+    B, T = len(lens), sum(new)
+    table, n_pages = _pages(B, max(lens), rng)
+    kp = torch.zeros((n_pages, nkv, 64, hd), dtype=DT[dtype], device=DEV)
+    vp = torch.zeros_like(kp)
+    ks = [rng.standard_normal((l, nkv * hd)) for l in lens]
+    vs = [rng.standard_normal((l, nkv * hd)) for l in lens]
+    for b in range(B):
+        kb, vb = _t(ks[b], DT[dtype]), _t(vs[b], DT[dtype])
+        ks[b], vs[b] = _np(kb), _np(vb)
+        for p in range(lens[b]):
+            kp[table[b, p // 64], :, p % 64, :] = kb[p].view(nkv, hd)
+            vp[table[b, p // 64], :, p % 64, :] = vb[p].view(nkv, hd)
+    stride = nh * hd + 24                                               # queries sit in a wider row
+    qbuf = _t(rng.standard_normal((T, stride)) * scale_q, DT[dtype])
+    tok_seq = np.repeat(np.arange(B), new).astype(np.int32)
+    tok_pos = np.concatenate([np.arange(l - n, l) for l, n in zip(lens, new)]).astype(np.int32)
+    return dict(q=qbuf, stride=stride, kp=kp, vp=vp, table=_t(table, torch.int32), ks=ks, vs=vs,
+                tok_seq=tok_seq, tok_pos=tok_pos, new=new, lens=lens)
+
+
+def _plain_attention(c, nh, nkv, hd, window=0, sinks=0, scale=None):
+    outs = []
+    q = _np(c["q"])[:, :nh * hd]
+    o = 0
+    for b, (l, n) in enumerate(zip(c["lens"], c["new"])):
+        full_q = np.zeros((l, nh * hd))
+        full_q[l - n:] = q[o:o + n]
+        outs.append(pm.attention(full_q, c["ks"][b], c["vs"][b], nh, nkv, hd, scale=scale, window=window,
+                                 sinks=sinks)[l - n:])
+        o += n
+    return np.concatenate(outs)
+
+
+ATTN_SHAPES = [(4, 2, 16), (6, 1, 32), (5, 5, 48), (8, 2, 64), (6, 3, 80), (4, 1, 96), (7, 7, 112),
+               (32, 8, 128), (3, 1, 256)]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nh,nkv,hd", ATTN_SHAPES)
+def test_attention_whole_prompts_and_single_tokens(dtype, nh, nkv, hd):
+    for lens, new in (([70, 3, 130], [70, 3, 130]),                     # whole prompts
+                      ([300, 1, 65, 64], [1, 1, 1, 1]),                 # one token each
+                      ([200, 90], [72, 5])):                            # continued prompts
+        c = _attention_case(dtype, nh, nkv, hd, lens, new)
+        ctx = type("Ctx", (), dict(tok_seq=_t(c["tok_seq"], torch.int32), tok_pos=_t(c["tok_pos"], torch.int32),
+                                   is_decode=max(new) == 1, max_context=max(lens), batch=len(lens),
+                                   n_tokens=sum(new), cu_seqlens=np.concatenate([[0], np.cumsum(new)]).tolist(),
+                                   starts=[l - n for l, n in zip(lens, new)], shared={}))()
+        out = K.attention(ctx, c["q"], c["stride"], c["kp"], c["vp"], c["table"], nh, nkv, hd, 1 / math.sqrt(hd))
+        _close(out, _plain_attention(c, nh, nkv, hd), dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_attention_finds_a_far_key_among_hundreds(dtype):
+    """One early key matches the query strongly; the output must be its value."""
+    nh, nkv, hd, L = 4, 2, 64, 700
+    c = _attention_case(dtype, nh, nkv, hd, [L], [1], scale_q=0.01)
+    q = c["q"]
+    far = 5
+    page, off = int(c["table"][0, far // 64]), far % 64
+    key = torch.zeros(hd, device=DEV); key[3] = 40.0
+    c["kp"][page, :, off, :] = key.to(c["kp"].dtype)
+    q[0, :nh * hd] = (key.repeat(nh) * 2).to(q.dtype)                   # score 40 * 80 / 8 = 400 for that key
+    ctx = type("Ctx", (), dict(tok_seq=_t(c["tok_seq"], torch.int32), tok_pos=_t(c["tok_pos"], torch.int32),
+                               is_decode=True, max_context=L, batch=1, n_tokens=1, cu_seqlens=[0, 1],
+                               starts=[L - 1], shared={}))()
+    out = _np(K.attention(ctx, q, c["stride"], c["kp"], c["vp"], c["table"], nh, nkv, hd, 1 / math.sqrt(hd)))
+    want = np.concatenate([c["vs"][0][far].reshape(nkv, hd)[h // 2] for h in range(nh)])
+    assert np.abs(out[0] - want).max() < 1e-5
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("window,sinks", [(64, 0), (70, 0), (5, 2), (128, 64), (1, 0)])
+def test_attention_window_edges(dtype, window, sinks):
+    nh, nkv, hd = 4, 2, 32
+    for lens, new in (([300, 66], [1, 1]), ([200, 10], [200, 10]), ([257], [100])):
+        c = _attention_case(dtype, nh, nkv, hd, lens, new, seed=9)
+        # keys just outside and just inside the window stand out, so an off-by-one shows
+        for b, l in enumerate(lens):
+            for p in (l - 1 - window, l - window):
+                if p >= max(sinks, 0) and p >= 0:
+                    page, off = int(c["table"][b, p // 64]), p % 64
+                    c["kp"][page, :, off, :] *= 6.0
+                    c["ks"][b][p] = _np(c["kp"][page, :, off, :]).reshape(-1)    # as stored
+        ctx = type("Ctx", (), dict(tok_seq=_t(c["tok_seq"], torch.int32), tok_pos=_t(c["tok_pos"], torch.int32),
+                                   is_decode=max(new) == 1, max_context=max(lens), batch=len(lens),
+                                   n_tokens=sum(new), cu_seqlens=np.concatenate([[0], np.cumsum(new)]).tolist(),
+                                   starts=[l - n for l, n in zip(lens, new)], shared={}))()
+        out = K.attention(ctx, c["q"], c["stride"], c["kp"], c["vp"], c["table"], nh, nkv, hd, 1 / math.sqrt(hd),
+                          window, sinks)
+        _close(out, _plain_attention(c, nh, nkv, hd, window, sinks), dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_swiglu(dtype):
+    rng = np.random.default_rng(5)
+    gu = _t(rng.standard_normal((9, 2 * 137)) * 4, DT[dtype])
+    g, u = _np(gu)[:, :137], _np(gu)[:, 137:]
+    _close(K.swiglu(gu), pm.silu(g) * u, dtype)
+
+
+def test_argmax_first_maximum_wins():
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((5, 128257)).astype(np.float32)
+    x[1, 4000] = x[1, 90000] = 9.0                                      # a tie: the first wins
+    x[2, 128256] = 10.0
+    x[3, :] = 0.25                                                      # all equal
+    x[4, 0] = 11.0
+    got = K.argmax(_t(x)).cpu().tolist()
+    assert got == [int(np.argmax(x[0])), 4000, 128256, 0, 0]
+    assert K.argmax(_t([[1., 5., 3., 2.]])).item() == 1                 # tests/.../SamplerTests.cs:8-18
+
+
+def test_kernels_refuse_what_they_cannot_do():
+    x = torch.zeros(4, 64, device=DEV)
+    with pytest.raises(K.KernelError, match="GPU"):
+        K.rmsnorm(torch.zeros(4, 64), torch.ones(64), 1e-6, torch.float32)
+    with pytest.raises(K.KernelError, match="weight"):
+        K.rmsnorm(x, torch.ones(63, device=DEV), 1e-6, torch.float32)
+    with pytest.raises(K.KernelError, match="w must be"):
+        K.gemm(x, torch.zeros(8, 65, device=DEV), None, torch.float32)
+    with pytest.raises(K.KernelError, match="not supported"):
+        K.gemm(x.half(), torch.zeros(8, 64, device=DEV).half(), None, torch.float16)
+    with pytest.raises(K.KernelError, match="head_dim"):
+        K.qk_rope_cache(torch.zeros(1, 3 * 1024, device=DEV), 1, 1, 1024, 2, 0, None, None, 1e-6,
+                        torch.zeros(1, 1, 2, device=DEV), None, None, None,
+                        torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV))
