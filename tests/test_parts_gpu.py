@@ -1,0 +1,346 @@
+"""Each part alone against its plain counterpart, the order of layers as data (a layer run
+twice, a layer reading another's cache), and a toy mixer with state of its own that is
+registered, built and stepped without a change to the library's files."""
+import dataclasses
+import importlib
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import gpu_helpers as H
+import plain_model as pm
+import tiny_configs as tc
+
+pytestmark = pytest.mark.gpu
+L = H.llogos
+P = importlib.import_module("daisi-llogos_amd.parts")
+K = importlib.import_module("daisi-llogos_amd.ops.kernels")
+DEV = torch.device("cuda:0")
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+TOL = {"float32": 2e-5, "bfloat16": 3e-2}
+
+
+def _np(t):
+    return t.detach().cpu().double().numpy()
+
+
+def _rand(rng, shape, dtype, scale=1.0):
+    t = torch.tensor(rng.standard_normal(shape) * scale, dtype=DT[dtype])
+    return t, t.double().numpy()
+
+
+def _ctx(rt, lens, new, slots=None):
+    B, T = len(lens), sum(new)
+    tok_seq = np.repeat(np.arange(B), new).astype(np.int32)
+    tok_pos = np.concatenate([np.arange(l - n, l) for l, n in zip(lens, new)]).astype(np.int32)
+    i32 = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=DEV)
+    return P.StepContext(runtime=rt, n_tokens=T, batch=B, ids=i32(np.zeros(T)), tok_seq=i32(tok_seq),
+                         tok_pos=i32(tok_pos), slots=i32(slots or list(range(B))),
+                         cu_seqlens=np.concatenate([[0], np.cumsum(new)]).tolist(),
+                         starts=[l - n for l, n in zip(lens, new)], slot_ids=slots or list(range(B)),
+                         is_decode=max(new) == 1, max_context=max(lens))
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+def test_linear_stacks_matrices_by_rows(dtype):
+    rng = np.random.default_rng(0)
+    rt = P.Runtime(DEV, DT[dtype])
+    wa, wa_ = _rand(rng, (24, 40), dtype, 0.1)
+    wb, wb_ = _rand(rng, (8, 40), dtype, 0.1)
+    ba, ba_ = _rand(rng, (24,), dtype)
+    bb, bb_ = _rand(rng, (8,), dtype)
+    lin = P.Linear(["a", "b"], 40, [24, 8], bias=True)
+    assert [(s.name, s.shape, s.kind) for s in lin.tensor_specs()] == [
+        ("a.weight", (24, 40), "matrix"), ("a.bias", (24,), "bias"), ("b.weight", (8, 40), "matrix"),
+        ("b.bias", (8,), "bias")]
+    lin.bind({"a.weight": wa, "b.weight": wb, "a.bias": ba, "b.bias": bb}.get, rt)
+    x, x_ = _rand(rng, (5, 40), dtype)
+    want = np.concatenate([pm.linear(x_, wa_, ba_), pm.linear(x_, wb_, bb_)], axis=1)
+    assert np.abs(_np(lin.forward(x.to(DEV))) - want).max() <= TOL[dtype] * 3
+    assert np.abs(_np(lin.forward(x.to(DEV), rows_out=24)) - want[:, :24]).max() <= TOL[dtype] * 3
+    assert lin.bias.dtype == torch.float32 and lin.weight.dtype == DT[dtype]
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+def test_rmsnorm_part(dtype):
+    rng = np.random.default_rng(1)
+    rt = P.Runtime(DEV, DT[dtype])
+    w, w_ = _rand(rng, (72,), dtype)
+    norm = P.RMSNorm("n", 72, 3e-4)
+    norm.bind({"n.weight": w}.get, rt)
+    x = torch.tensor(rng.standard_normal((6, 72)), dtype=torch.float32, device=DEV)
+    x_ = _np(x)
+    d, d_ = _rand(rng, (6, 72), dtype)
+    out = norm.forward(x, d.to(DEV))
+    assert np.abs(_np(out) - pm.rms_norm(x_ + d_, w_, 3e-4)).max() <= TOL[dtype] * 3
+    assert np.abs(_np(x) - (x_ + d_)).max() < 1e-6                      # the residual stream took the sum
+
+
+def test_rotary_part_tables():
+    rt = P.Runtime(DEV, torch.float32)
+    plain_f = pm.rope_frequencies(24, 5e5)
+    rot = P.Rotary(48, 24, 5e5)
+    assert np.allclose(rot.freqs, plain_f, rtol=1e-15)
+    sc = dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+              original_max_position_embeddings=64)
+    rot3 = P.Rotary(48, 24, 5e5, scaling=sc)
+    want = plain_f / pm.llama3_frequency_factors(plain_f, 8.0, 1.0, 4.0, 64)
+    assert np.allclose(rot3.freqs, want, rtol=1e-15) and not np.allclose(want, plain_f)
+    assert np.allclose(P.Rotary(48, 24, 5e5, scaling=dict(rope_type="linear", factor=4.0)).freqs, plain_f / 4)
+    rot3.bind(lambda n: None, rt)
+    ctx = _ctx(rt, [70, 3], [5, 3])
+    cs = _np(rot3.prepare(ctx))
+    ang = _np(ctx.tok_pos)[:, None] * want[None, :]
+    assert np.abs(cs[..., 0] - np.cos(ang)).max() < 1e-7 and np.abs(cs[..., 1] - np.sin(ang)).max() < 1e-7
+    assert rot3.prepare(ctx) is rot3.prepare(ctx)                       # made once per step
+    with pytest.raises(ValueError):
+        P.Rotary(48, 50, 1e4)
+    with pytest.raises(ValueError):
+        P.Rotary(48, 24, 1e4, scaling=dict(rope_type="yarn", factor=2.0))
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd,bias,qk_norm,window", [(4, 2, 16, True, False, 0), (6, 1, 32, False, True, 0),
+                                                           (5, 5, 48, True, True, 20)])
+def test_attention_part_alone(dtype, nh, nkv, hd, bias, qk_norm, window):
+    """The mixer alone: a prompt in one step, then two single tokens, against plain parts."""
+    rng = np.random.default_rng(2)
+    rt = P.Runtime(DEV, DT[dtype])
+    hidden, T = 40, 70
+    rot = P.Rotary(hd, hd, 1e4)
+    att = P.Attention("a.", hidden, nh, nkv, hd, rot, bias=bias, qk_norm=qk_norm, eps=1e-5, window=window)
+    tensors, plain = {}, {}
+    for spec in att.tensor_specs():
+        scale = 0.2 if spec.kind == "matrix" else 1.0
+        t, a = _rand(rng, spec.shape, dtype, scale)
+        if spec.kind == "norm":
+            t = (1 + 0.1 * t.float()).to(DT[dtype]); a = t.double().numpy()
+        tensors[spec.name], plain[spec.name] = t, a
+    att.bind(tensors.get, rt)
+    assert att.kv_spec() == P.KVSpec(nkv, hd, window, 0) and att.state_spec() is None
+    x, x_ = _rand(rng, (T, hidden), dtype)
+    # plain: projections, norm, rotation, attention, output projection
+    q = pm.linear(x_, plain["a.q_proj.weight"], plain.get("a.q_proj.bias"))
+    k = pm.linear(x_, plain["a.k_proj.weight"], plain.get("a.k_proj.bias"))
+    v = pm.linear(x_, plain["a.v_proj.weight"], plain.get("a.v_proj.bias"))
+    if qk_norm:
+        q = pm.per_head_rms_norm(q, plain["a.q_norm.weight"], nh, hd, 1e-5)
+        k = pm.per_head_rms_norm(k, plain["a.k_norm.weight"], nkv, hd, 1e-5)
+    f = pm.rope_frequencies(hd, 1e4)
+    q, k = pm.rope_split_half(q, range(T), nh, hd, f), pm.rope_split_half(k, range(T), nkv, hd, f)
+    want = pm.linear(pm.attention(q, k, v, nh, nkv, hd, window=window), plain["a.o_proj.weight"])
+    # engine part, with a cache of its own
+    pool = lambda: torch.zeros((3, nkv, 64, hd), dtype=DT[dtype], device=DEV)
+    cache = P.LayerCache(k_pool=pool(), v_pool=pool(), table=torch.tensor([[2, 0]], dtype=torch.int32, device=DEV))
+    outs = [att.forward(_ctx(rt, [68], [68]), x[:68].to(DEV), cache)]
+    for t in (68, 69):
+        outs.append(att.forward(_ctx(rt, [t + 1], [1]), x[t:t + 1].to(DEV), cache))
+    got = _np(torch.cat(outs))
+    assert np.abs(got - want).max() <= TOL[dtype] * max(1.0, np.abs(want).max())
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+def test_swiglu_part_alone(dtype):
+    rng = np.random.default_rng(3)
+    rt = P.Runtime(DEV, DT[dtype])
+    ffn = P.SwiGLU("m.", 40, 72)
+    tensors, plain = {}, {}
+    for spec in ffn.tensor_specs():
+        tensors[spec.name], plain[spec.name] = _rand(rng, spec.shape, dtype, 0.2)
+    ffn.bind(tensors.get, rt)
+    x, x_ = _rand(rng, (9, 40), dtype)
+    want = pm.swiglu_mlp(x_, plain["m.gate_proj.weight"], plain["m.up_proj.weight"], plain["m.down_proj.weight"])
+    assert np.abs(_np(ffn.forward(None, x.to(DEV))) - want).max() <= TOL[dtype] * max(1.0, np.abs(want).max())
+
+
+# ---------------------------------------------------------------------------
+# the order of layers is data
+# ---------------------------------------------------------------------------
+def _scheduled_arch(name, schedule):
+    models = importlib.import_module("daisi-llogos_amd.models")
+
+    def spec(cfg, **kw):
+        s = L.dense_decoder_spec(cfg, **kw)
+        s.schedule = [models.ScheduleEntry(l, c) for l, c in schedule]
+        return s
+    L.register_architecture(name, L.ARCHITECTURES["Qwen2ForCausalLM"].read_config, spec)
+
+
+def _plain_scheduled(cfg, w, tokens, schedule):
+    """Plain forward in which the order of layers is a list; an entry may read the keys and
+    values another entry made."""
+    T = len(tokens)
+    f = cfg.frequencies()
+    x = pm.embedding(w["model.embed_tokens.weight"], tokens)
+    kv = {}
+    for e, (i, src) in enumerate(schedule):
+        p = f"model.layers.{i}."
+        n = pm.rms_norm(x, w[p + "input_layernorm.weight"], cfg.eps)
+        q = pm.rope_split_half(pm.linear(n, w[p + "self_attn.q_proj.weight"], w.get(p + "self_attn.q_proj.bias")),
+                               range(T), cfg.n_heads, cfg.head_dim, f)
+        if src is None:
+            k = pm.rope_split_half(pm.linear(n, w[p + "self_attn.k_proj.weight"], w.get(p + "self_attn.k_proj.bias")),
+                                   range(T), cfg.n_kv_heads, cfg.head_dim, f)
+            v = pm.linear(n, w[p + "self_attn.v_proj.weight"], w.get(p + "self_attn.v_proj.bias"))
+            kv[e] = (k, v)
+        else:
+            k, v = kv[src]
+        a = pm.attention(q, k, v, cfg.n_heads, cfg.n_kv_heads, cfg.head_dim)
+        x = x + pm.linear(a, w[p + "self_attn.o_proj.weight"])
+        n = pm.rms_norm(x, w[p + "post_attention_layernorm.weight"], cfg.eps)
+        x = x + pm.swiglu_mlp(n, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    return pm.linear(pm.rms_norm(x, w["model.norm.weight"], cfg.eps), w["lm_head.weight"])
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+def test_a_layer_twice_and_a_layer_reading_anothers_cache(tmp_path, dtype):
+    schedule = [(0, None), (1, None), (1, None), (0, 0)]        # layer 1 twice; layer 0 again on entry 0's cache
+    _scheduled_arch("ScheduledToyForCausalLM", schedule)
+    cfg_json = dict(tc.TINY_A, architectures=["ScheduledToyForCausalLM"])
+    folder = L.write_random_model(str(tmp_path / "m"), cfg_json, seed=4)
+    import json
+    from safetensors.torch import load_file
+    pcfg = pm.PlainConfig(dict(tc.TINY_A))
+    w = {k: v.double().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    toks = list(H.tokens("tiny_a", 80, 5))
+    want = _plain_scheduled(pcfg, w, toks, schedule)
+    eng = L.Engine.from_folder(folder, dtype=dtype, max_tokens=256)
+    assert len(eng.cache.groups) == 1 and eng.cache.groups[0].k.shape[0] == 3      # three caches for four runs
+    s = eng.alloc_slot()
+    rows = [_np(eng.step([(s, toks[:66])], want="all"))] + [_np(eng.step([(s, [t])])) for t in toks[66:]]
+    H.close(np.concatenate(rows), want, dtype, "scheduled layers")
+    models = importlib.import_module("daisi-llogos_amd.models")
+    spec = L.dense_decoder_spec(L.ARCHITECTURES["Qwen2ForCausalLM"].read_config(tc.TINY_A))
+    spec.schedule = [models.ScheduleEntry(0), models.ScheduleEntry(1, cache_of=1)]
+    with pytest.raises(ValueError, match="before"):
+        L.Model(spec)
+
+
+# ---------------------------------------------------------------------------
+# a toy mixer with state of its own, defined here
+# ---------------------------------------------------------------------------
+@P.register_mixer("toy_running_mean")
+class RunningMean(P.Mixer):
+    """out_t = W . mean(h_0 .. h_t): the running sum is the sequence's fixed-size state."""
+
+    def __init__(self, prefix, hidden):
+        self.prefix, self.hidden = prefix, hidden
+
+    def tensor_specs(self):
+        return [P.TensorSpec(self.prefix + "mix.weight", (self.hidden, self.hidden), "matrix")]
+
+    def state_spec(self):
+        return P.StateSpec((self.hidden,), torch.float32)
+
+    def bind(self, get, rt):
+        self.rt = rt
+        self.w = get(self.prefix + "mix.weight").to(device=rt.device, dtype=torch.float32)
+
+    def forward(self, ctx, h, cache):
+        out = torch.empty_like(h)
+        for b in range(ctx.batch):
+            lo, hi = ctx.cu_seqlens[b], ctx.cu_seqlens[b + 1]
+            slot = ctx.slot_ids[b]
+            run = torch.cumsum(h[lo:hi].float(), 0) + cache.state[slot]
+            cache.state[slot] = run[-1]
+            count = torch.arange(ctx.starts[b] + 1, ctx.starts[b] + hi - lo + 1, device=h.device)[:, None]
+            out[lo:hi] = ((run / count) @ self.w.T).to(h.dtype)
+        return out
+
+
+@dataclasses.dataclass(frozen=True)
+class ToyConfig:
+    vocab_size: int
+    hidden_size: int
+    n_layers: int
+    architecture: str = "ToyStateForCausalLM"
+    num_hidden_layers: int = 0
+    num_attention_heads: int = 2
+    num_key_value_heads: int = 1
+
+
+def _toy_spec(cfg, **kw):
+    models = importlib.import_module("daisi-llogos_amd.models")
+    rot = P.Rotary(16, 16, 1e4)
+    layers = []
+    for i in range(cfg.n_layers):
+        p = f"layers.{i}."
+        mixer = ("toy_running_mean", dict(prefix=p, hidden=cfg.hidden_size)) if i % 2 == 0 else \
+            ("attention", dict(prefix=p + "attn.", hidden=cfg.hidden_size, n_heads=2, n_kv_heads=1, head_dim=16,
+                               position=rot))
+        layers.append(models.LayerSpec(
+            mixer=mixer, ffn=("swiglu", dict(prefix=p + "ffn.", hidden=cfg.hidden_size, intermediate=56)),
+            mixer_norm=("rmsnorm", dict(name=p + "n1", width=cfg.hidden_size, eps=1e-6)),
+            ffn_norm=("rmsnorm", dict(name=p + "n2", width=cfg.hidden_size, eps=1e-6))))
+    return models.ModelSpec(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size, embed_name="embed.weight",
+                            layers=layers, final_norm=("rmsnorm", dict(name="norm", width=cfg.hidden_size, eps=1e-6)),
+                            head_name="head", tie_head=False)
+
+
+L.register_architecture("ToyStateForCausalLM",
+                        lambda d: ToyConfig(d["vocab_size"], d["hidden_size"], d["n_layers"]), _toy_spec)
+
+
+def _plain_toy(w, tokens, n_layers):
+    T = len(tokens)
+    x = pm.embedding(w["embed.weight"], tokens)
+    f = pm.rope_frequencies(16, 1e4)
+    for i in range(n_layers):
+        p = f"layers.{i}."
+        n = pm.rms_norm(x, w[p + "n1.weight"], 1e-6)
+        if i % 2 == 0:
+            a = pm.linear(np.cumsum(n, axis=0) / np.arange(1, T + 1)[:, None], w[p + "mix.weight"])
+        else:
+            q = pm.rope_split_half(pm.linear(n, w[p + "attn.q_proj.weight"]), range(T), 2, 16, f)
+            k = pm.rope_split_half(pm.linear(n, w[p + "attn.k_proj.weight"]), range(T), 1, 16, f)
+            a = pm.linear(pm.attention(q, k, pm.linear(n, w[p + "attn.v_proj.weight"]), 2, 1, 16), w[p + "attn.o_proj.weight"])
+        x = x + a
+        n = pm.rms_norm(x, w[p + "n2.weight"], 1e-6)
+        x = x + pm.swiglu_mlp(n, w[p + "ffn.gate_proj.weight"], w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
+    return pm.linear(pm.rms_norm(x, w["norm.weight"], 1e-6), w["head.weight"])
+
+
+def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
+    from safetensors.torch import load_file
+    cfg = {"architectures": ["ToyStateForCausalLM"], "vocab_size": 90, "hidden_size": 40, "n_layers": 3,
+           "torch_dtype": "float32"}
+    folder = L.write_random_model(str(tmp_path / "toy"), cfg, seed=2)
+    w = {k: v.double().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    eng = L.Engine.from_folder(folder, dtype="float32", max_tokens=512, n_slots=2)
+    needs = eng.model.cache_needs()
+    assert [st is not None for _, st in needs] == [True, False, True]
+    assert [kv is not None for kv, _ in needs] == [False, True, False]
+    rng = np.random.default_rng(0)
+    seqs = [rng.integers(0, 90, size=n).tolist() for n in (30, 7, 75)]
+    want = [_plain_toy(w, s, 3) for s in seqs]
+    # whole and alone
+    for s, wnt in zip(seqs, want):
+        slot = eng.alloc_slot()
+        H.close(_np(eng.step([(slot, s)], want="all")), wnt, "float32", "toy whole")
+        eng.free_slot(slot)
+    # a batch of unequal lengths, prompts then one token each; shorter ones end earlier; slots were used before,
+    # so a state that is not zeroed when its slot is handed out again would show
+    slots = [eng.alloc_slot() for _ in seqs]
+    cut = [20, 3, 70]
+    out = eng.step([(sl, s[:c]) for sl, s, c in zip(slots, seqs, cut)], want="all")
+    rows = [[] for _ in seqs]
+    o = 0
+    for i, c in enumerate(cut):
+        rows[i].append(_np(out[o:o + c])); o += c
+    fed = list(cut)
+    live = [0, 1, 2]
+    while live:
+        for i in [i for i in live if fed[i] == len(seqs[i])]:
+            eng.free_slot(slots[i]); live.remove(i)
+        if not live:
+            break
+        out = eng.step([(slots[i], [seqs[i][fed[i]]]) for i in live], want="last")
+        for j, i in enumerate(live):
+            rows[i].append(_np(out[j:j + 1])); fed[i] += 1
+    for i in range(3):
+        H.close(np.concatenate(rows[i]), want[i], "float32", f"toy batch seq {i}")
+    with pytest.raises(L.CacheError, match="state"):
+        s = eng.alloc_slot(); eng.step([(s, [1, 2, 3])]); eng.cache.truncate(s, 1)
