@@ -62,7 +62,8 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
                 for (int jj = 0; jj < n_keys; ++jj) {
                     const float pj = p_lds[jj];
                     if (pj != 0.f)
-                        a = fmaf(pj, load_f32(v_pool + paged_offset(cache, seq, kvh, j0 + jj) + d), a);
+                        a = fmaf(pj, load_f32(v_pool + paged_v_offset(cache, seq, kvh, j0 + jj)
+                                              + (size_t)d * kPageTokens), a);
                 }
                 acc[r] = a;
             }

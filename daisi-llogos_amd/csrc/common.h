@@ -76,9 +76,11 @@ __device__ __forceinline__ float block_max(float v, float* red) {
     return t;
 }
 
-// A layer's keys (or values) live in pages of kPageTokens tokens:
-// pool[page][kv_head][token in page][head_dim].  A sequence's pages are listed in
-// its row of the step's page table.
+// A layer's keys and values live in pages of kPageTokens tokens.  A sequence's pages are
+// listed in its row of the step's page table.
+//   keys:   pool[page][kv_head][token in page][head_dim]
+//   values: pool[page][kv_head][head_dim][token in page]   (transposed, so that the
+//           matrix cores can take eight consecutive tokens of one dimension in one load)
 struct PagedKV {
     const int* table;      // [batch, table_stride] page ids of this step's sequences
     int table_stride;
@@ -89,6 +91,12 @@ struct PagedKV {
 __device__ __forceinline__ size_t paged_offset(const PagedKV& c, int seq, int kv_head, int pos) {
     const int page = c.table[(size_t)seq * c.table_stride + pos / kPageTokens];
     return (((size_t)page * c.n_kv_heads + kv_head) * kPageTokens + (pos % kPageTokens)) * c.head_dim;
+}
+
+// offset of dimension 0 of a value vector; dimension d lies d * kPageTokens further
+__device__ __forceinline__ size_t paged_v_offset(const PagedKV& c, int seq, int kv_head, int pos) {
+    const int page = c.table[(size_t)seq * c.table_stride + pos / kPageTokens];
+    return ((size_t)page * c.n_kv_heads + kv_head) * kPageTokens * c.head_dim + (pos % kPageTokens);
 }
 
 // A query at q_pos sees key k_pos when it is not in the future and, with a window,

@@ -35,8 +35,18 @@ LLOGOS_EXPORT int llogos_embed(float* out, const void* table, int table_dtype, c
 // The residual stream x stays in float; out has the matrix products' input type.
 // (reference: rms_norm / add_rms_norm_residual, Daisi.Llogos.Cuda/kernels/elementwise.cu:18-171,
 //  668-733; eps inside the root, weight multiplies as it is.)
+// sum of the `parts` partial products of element i (parts lie part_stride elements apart),
+// added in ascending order
+template <typename TD>
+__device__ __forceinline__ float sum_parts(const TD* p, size_t i, int parts, size_t part_stride) {
+    float v = load_f32(p + i);
+    for (int q = 1; q < parts; ++q) v += load_f32(p + q * part_stride + i);
+    return v;
+}
+
 template <typename TO, typename TD>
 __global__ void rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ x, const TD* __restrict__ delta,
+                               int parts, size_t part_stride,
                                const int* __restrict__ rows, const float* __restrict__ w,
                                float eps, int H, int write_back) {
     __shared__ float red[16];
@@ -48,7 +58,7 @@ __global__ void rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ x, cons
     for (int i = threadIdx.x; i < H; i += blockDim.x) {
         float v = xr[i];
         if (dr) {
-            v += load_f32(dr + i);
+            v += sum_parts(dr, i, parts, part_stride);
             if (write_back) xr[i] = v;
         }
         ss += v * v;
@@ -58,18 +68,21 @@ __global__ void rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ x, cons
     TO* o = out + (size_t)r * H;
     for (int i = threadIdx.x; i < H; i += blockDim.x) {
         float v = xr[i];
-        if (dr && !write_back) v += load_f32(dr + i);
+        if (dr && !write_back) v += sum_parts(dr, i, parts, part_stride);
         store_f32(o + i, v * inv * w[i]);
     }
 }
 
+// delta: `parts` partial products [parts][T][H] (part_stride elements apart) that are summed
+// on the way; parts = 1 for a plain delta.
 LLOGOS_EXPORT int llogos_rmsnorm(void* out, int out_dtype, float* x, const void* delta, int delta_dtype,
+                                 int parts, long long part_stride,
                                  const int* rows, const float* w, float eps, int R, int H,
                                  int write_back, hipStream_t stream) {
-    if (R <= 0 || H <= 0) return LLOGOS_BAD_ARGUMENT;
+    if (R <= 0 || H <= 0 || parts < 1) return LLOGOS_BAD_ARGUMENT;
     const int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
 #define LAUNCH(TO, TD) rmsnorm_kernel<TO, TD><<<R, threads, 0, stream>>>( \
-        (TO*)out, x, (const TD*)delta, rows, w, eps, H, write_back)
+        (TO*)out, x, (const TD*)delta, parts, (size_t)part_stride, rows, w, eps, H, write_back)
     if (out_dtype == DT_F32 && delta_dtype == DT_F32) LAUNCH(float, float);
     else if (out_dtype == DT_BF16 && delta_dtype == DT_BF16) LAUNCH(bf16_t, bf16_t);
     else if (out_dtype == DT_BF16 && delta_dtype == DT_F32) LAUNCH(bf16_t, float);
@@ -128,9 +141,10 @@ LLOGOS_EXPORT int llogos_rope_table(void* cs, const int* pos, const double* inv_
 constexpr int kHeadsPerBlock = 4;
 constexpr int kMaxHeadDim = 512;
 
-template <typename T>
-__global__ void qk_rope_cache_kernel(T* __restrict__ qkv, int row_stride, int n_heads, int n_kv_heads,
-                                     int head_dim, int rot, int pairing,
+template <typename TI, typename T>
+__global__ void qk_rope_cache_kernel(const TI* __restrict__ qkv, int parts, size_t part_stride, int row_stride,
+                                     const float* __restrict__ bias, T* __restrict__ q_out,
+                                     int n_heads, int n_kv_heads, int head_dim, int rot, int pairing,
                                      const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w,
                                      float eps, const float2* __restrict__ cs,
                                      T* __restrict__ k_pool, T* __restrict__ v_pool, PagedKV cache,
@@ -144,7 +158,8 @@ __global__ void qk_rope_cache_kernel(T* __restrict__ qkv, int row_stride, int n_
     float* buf = smem + threadIdx.y * head_dim;
     const int half = rot / 2;
 
-    T* src = qkv + (size_t)t * row_stride + (size_t)(active ? head : 0) * head_dim;
+    const size_t col0 = (size_t)(active ? head : 0) * head_dim;
+    const TI* src = qkv + (size_t)t * row_stride + col0;
     const bool is_q = head < n_heads;
     const bool is_k = !is_q && head < n_heads + n_kv_heads;
     const float* norm_w = is_q ? q_norm_w : (is_k ? k_norm_w : nullptr);
@@ -152,7 +167,8 @@ __global__ void qk_rope_cache_kernel(T* __restrict__ qkv, int row_stride, int n_
     float ss = 0.f;
     if (active) {
         for (int d = lane; d < head_dim; d += kWave) {
-            const float v = load_f32(src + d);
+            float v = sum_parts(src, (size_t)d, parts, part_stride);
+            if (bias) v += bias[col0 + d];
             buf[d] = v;
             ss += v * v;
         }
@@ -168,80 +184,115 @@ __global__ void qk_rope_cache_kernel(T* __restrict__ qkv, int row_stride, int n_
 
     T* dst;
     if (is_q) {
-        dst = src;
+        dst = q_out + ((size_t)t * n_heads + head) * head_dim;
+    } else if (is_k) {
+        dst = k_pool + paged_offset(cache, tok_seq[t], head - n_heads, tok_pos[t]);
     } else {
-        const int kvh = is_k ? head - n_heads : head - n_heads - n_kv_heads;
-        const size_t off = paged_offset(cache, tok_seq[t], kvh, tok_pos[t]);
-        dst = (is_k ? k_pool : v_pool) + off;
+        // values are stored transposed: dimension d of this token lies d * kPageTokens further
+        T* vdst = v_pool + paged_v_offset(cache, tok_seq[t], head - n_heads - n_kv_heads, tok_pos[t]);
+        for (int d = lane; d < head_dim; d += kWave) store_f32(vdst + (size_t)d * kPageTokens, buf[d]);
+        return;
     }
-    if (is_q || is_k) {
-        const float2* c = cs + (size_t)t * half;
-        for (int d = lane; d < head_dim; d += kWave) {
-            float v = buf[d];
-            if (d < rot) {
-                if (pairing == 0) {
-                    if (d < half) v = buf[d] * c[d].x - buf[d + half] * c[d].y;
-                    else          v = buf[d - half] * c[d - half].y + buf[d] * c[d - half].x;
-                } else {
-                    const int i = d >> 1;
-                    if ((d & 1) == 0) v = buf[d] * c[i].x - buf[d + 1] * c[i].y;
-                    else              v = buf[d - 1] * c[i].y + buf[d] * c[i].x;
-                }
+    const float2* c = cs + (size_t)t * half;
+    for (int d = lane; d < head_dim; d += kWave) {
+        float v = buf[d];
+        if (d < rot) {
+            if (pairing == 0) {
+                if (d < half) v = buf[d] * c[d].x - buf[d + half] * c[d].y;
+                else          v = buf[d - half] * c[d - half].y + buf[d] * c[d - half].x;
+            } else {
+                const int i = d >> 1;
+                if ((d & 1) == 0) v = buf[d] * c[i].x - buf[d + 1] * c[i].y;
+                else              v = buf[d - 1] * c[i].y + buf[d] * c[i].x;
             }
-            store_f32(dst + d, v);
         }
-    } else {
-        for (int d = lane; d < head_dim; d += kWave) store_f32(dst + d, buf[d]);
+        store_f32(dst + d, v);
     }
 }
 
-LLOGOS_EXPORT int llogos_qk_rope_cache(void* qkv, int dtype, int row_stride, int n_heads, int n_kv_heads,
-                                       int head_dim, int rot, int pairing,
+// qkv: the fused projection [parts][T][row_stride] in float32 or in the cache's type (parts are
+// summed, then `bias` [width] is added); q_out [T, n_heads * head_dim] and the pools have the
+// cache's type `dtype`.
+LLOGOS_EXPORT int llogos_qk_rope_cache(const void* qkv, int in_dtype, int parts, long long part_stride,
+                                       int row_stride, const float* bias, void* q_out, int dtype,
+                                       int n_heads, int n_kv_heads, int head_dim, int rot, int pairing,
                                        const float* q_norm_w, const float* k_norm_w, float eps,
                                        const void* cs, void* k_pool, void* v_pool,
                                        const int* table, int table_stride,
                                        const int* tok_seq, const int* tok_pos, int T, hipStream_t stream) {
     if (T <= 0 || n_heads <= 0 || n_kv_heads < 0 || head_dim <= 0 || head_dim > kMaxHeadDim) return LLOGOS_BAD_ARGUMENT;
-    if (rot < 0 || rot > head_dim || (rot & 1)) return LLOGOS_BAD_ARGUMENT;
+    if (rot < 0 || rot > head_dim || (rot & 1) || parts < 1) return LLOGOS_BAD_ARGUMENT;
     if (n_kv_heads > 0 && (!k_pool || !v_pool || !table)) return LLOGOS_BAD_ARGUMENT;
     if (row_stride < (n_heads + 2 * n_kv_heads) * head_dim) return LLOGOS_BAD_ARGUMENT;
     PagedKV cache{table, table_stride, n_kv_heads, head_dim};
     const int total_heads = n_heads + 2 * n_kv_heads;
     dim3 grid(T, (total_heads + kHeadsPerBlock - 1) / kHeadsPerBlock), block(kWave, kHeadsPerBlock);
     const size_t smem = (size_t)kHeadsPerBlock * head_dim * sizeof(float);
-    if (dtype == DT_F32)
-        qk_rope_cache_kernel<float><<<grid, block, smem, stream>>>(
-            (float*)qkv, row_stride, n_heads, n_kv_heads, head_dim, rot, pairing, q_norm_w, k_norm_w, eps,
-            (const float2*)cs, (float*)k_pool, (float*)v_pool, cache, tok_seq, tok_pos);
-    else if (dtype == DT_BF16)
-        qk_rope_cache_kernel<bf16_t><<<grid, block, smem, stream>>>(
-            (bf16_t*)qkv, row_stride, n_heads, n_kv_heads, head_dim, rot, pairing, q_norm_w, k_norm_w, eps,
-            (const float2*)cs, (bf16_t*)k_pool, (bf16_t*)v_pool, cache, tok_seq, tok_pos);
-    else
-        return LLOGOS_BAD_ARGUMENT;
+#define LAUNCH(TI, T_) qk_rope_cache_kernel<TI, T_><<<grid, block, smem, stream>>>( \
+        (const TI*)qkv, parts, (size_t)part_stride, row_stride, bias, (T_*)q_out, n_heads, n_kv_heads, head_dim, \
+        rot, pairing, q_norm_w, k_norm_w, eps, (const float2*)cs, (T_*)k_pool, (T_*)v_pool, cache, tok_seq, tok_pos)
+    if (dtype == DT_F32 && in_dtype == DT_F32) LAUNCH(float, float);
+    else if (dtype == DT_BF16 && in_dtype == DT_BF16) LAUNCH(bf16_t, bf16_t);
+    else if (dtype == DT_BF16 && in_dtype == DT_F32) LAUNCH(float, bf16_t);
+    else return LLOGOS_BAD_ARGUMENT;
+#undef LAUNCH
     return LLOGOS_LAUNCH_CHECK();
 }
 
 // ---------------------------------------------------------------- SwiGLU
 // out[t, i] = silu(gu[t, i]) * gu[t, I + i] from the fused row [gate | up].
 // (reference: split_swiglu, Daisi.Llogos.Cuda/kernels/elementwise.cu:1084-1110; silu(z) = z / (1 + exp(-z)))
-template <typename T>
-__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ gu, int I, size_t n) {
+template <typename TI, typename T>
+__global__ void swiglu_kernel(T* __restrict__ out, const TI* __restrict__ gu, int parts, size_t part_stride,
+                              int I, size_t n) {
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= n) return;
     const size_t t = idx / I;
     const int i = (int)(idx % I);
-    const float g = load_f32(gu + t * 2 * I + i);
-    const float u = load_f32(gu + t * 2 * I + I + i);
+    const float g = sum_parts(gu, t * 2 * I + i, parts, part_stride);
+    const float u = sum_parts(gu, t * 2 * I + I + i, parts, part_stride);
     store_f32(out + idx, g / (1.0f + expf(-g)) * u);
 }
 
-LLOGOS_EXPORT int llogos_swiglu(void* out, const void* gu, int dtype, int T, int I, hipStream_t stream) {
-    if (T <= 0 || I <= 0) return LLOGOS_BAD_ARGUMENT;
+// gu: [parts][T][2 I] in float32 or in the output's type; parts are summed on the way.
+LLOGOS_EXPORT int llogos_swiglu(void* out, int dtype, const void* gu, int in_dtype, int parts,
+                                long long part_stride, int T, int I, hipStream_t stream) {
+    if (T <= 0 || I <= 0 || parts < 1) return LLOGOS_BAD_ARGUMENT;
     const size_t n = (size_t)T * I;
     const unsigned blocks = (unsigned)((n + 255) / 256);
-    if (dtype == DT_F32) swiglu_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)gu, I, n);
-    else if (dtype == DT_BF16) swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, I, n);
+#define LAUNCH(TI, T_) swiglu_kernel<TI, T_><<<blocks, 256, 0, stream>>>( \
+        (T_*)out, (const TI*)gu, parts, (size_t)part_stride, I, n)
+    if (dtype == DT_F32 && in_dtype == DT_F32) LAUNCH(float, float);
+    else if (dtype == DT_BF16 && in_dtype == DT_BF16) LAUNCH(bf16_t, bf16_t);
+    else if (dtype == DT_BF16 && in_dtype == DT_F32) LAUNCH(float, bf16_t);
     else return LLOGOS_BAD_ARGUMENT;
+#undef LAUNCH
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+// out[T, N] = sum of parts (+ bias): for consumers that want one plain tensor.
+template <typename TI, typename TO>
+__global__ void sum_parts_kernel(TO* __restrict__ out, const TI* __restrict__ in, int parts, size_t part_stride,
+                                 const float* __restrict__ bias, int N, size_t n) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n) return;
+    float v = sum_parts(in, idx, parts, part_stride);
+    if (bias) v += bias[idx % N];
+    store_f32(out + idx, v);
+}
+
+LLOGOS_EXPORT int llogos_sum_parts(void* out, int out_dtype, const void* in, int in_dtype, int parts,
+                                   long long part_stride, const float* bias, int T, int N, hipStream_t stream) {
+    if (T <= 0 || N <= 0 || parts < 1) return LLOGOS_BAD_ARGUMENT;
+    const size_t n = (size_t)T * N;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+#define LAUNCH(TI, TO) sum_parts_kernel<TI, TO><<<blocks, 256, 0, stream>>>( \
+        (TO*)out, (const TI*)in, parts, (size_t)part_stride, bias, N, n)
+    if (in_dtype == DT_F32 && out_dtype == DT_F32) LAUNCH(float, float);
+    else if (in_dtype == DT_F32 && out_dtype == DT_BF16) LAUNCH(float, bf16_t);
+    else if (in_dtype == DT_BF16 && out_dtype == DT_F32) LAUNCH(bf16_t, float);
+    else if (in_dtype == DT_BF16 && out_dtype == DT_BF16) LAUNCH(bf16_t, bf16_t);
+    else return LLOGOS_BAD_ARGUMENT;
+#undef LAUNCH
     return LLOGOS_LAUNCH_CHECK();
 }

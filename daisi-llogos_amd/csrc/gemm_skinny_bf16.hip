@@ -1,0 +1,169 @@
+// out[M, N] = a[M, K] . w[N, K]^T (+ bias) for few rows (M <= 64) of bfloat16 activations:
+// the decode step's matrix products, which are bound by streaming w from HBM once.
+//
+// Mapping to the hardware (gfx950, 64-wide waves, v_mfma_f32_16x16x32_bf16):
+//  * a wave owns a strip of RB * 16 rows of w and a range of k.  Each lane loads 16 bytes of
+//    a row straight from global memory into the matrix-core operand layout (lane = row +
+//    16 * k-group), several loads in flight before the first MFMA;
+//  * the activations are the other operand (M padded to MB * 16 columns); they are small,
+//    come from L2, and one activation fragment serves the RB row blocks of the strip;
+//  * the 4 waves of a block split the block's k range and add their sums through LDS;
+//  * when k is split over blocks as well, each block writes its float32 partial sums to
+//    out[split][M][N] and the kernel that consumes the product adds the parts in a fixed
+//    order (a fence between blocks would cost a write-back of the whole L2 on this chip).
+// Every output element sums k in an order that depends on N and K alone, never on M.
+// (reference: one-row dequant_matmul_bf16, Daisi.Llogos.Cuda/kernels/dequant_matmul.cu:593-619,
+//  one row of w per block with FP32 accumulation.)
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kSkinnyWaves = 4;
+constexpr int kStepK = 32;
+
+__device__ __forceinline__ bf16x8 load_frag(const bf16_t* p, bool ok) {
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (ok) v = *reinterpret_cast<const uint4*>(p);
+    return __builtin_bit_cast(bf16x8, v);
+}
+
+template <int RB, int MB, int U, typename TO>
+__global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny_kernel(
+        TO* __restrict__ out, const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
+        const float* __restrict__ bias, int M, int N, int K, int lda, int ldo, size_t part_stride,
+        int k_per_block) {
+    __shared__ float red[kSkinnyWaves][RB * MB][kWave][4];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int r = lane & 15, g = lane >> 4;
+    const int split = blockIdx.y;
+    const int n0 = blockIdx.x * (16 * RB);
+    const int k_per_wave = k_per_block / kSkinnyWaves;
+    const int k_begin = split * k_per_block + wave * k_per_wave;
+    const int k_end = min(K, k_begin + k_per_wave);
+
+    const bf16_t* wrow[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)                        // rows past N read a valid row, never stored
+        wrow[rb] = w + (size_t)min(n0 + rb * 16 + r, N - 1) * K + g * 8;
+    const bf16_t* arow[MB];
+    bool a_ok[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const int m = mb * 16 + r;
+        a_ok[mb] = m < M;
+        arow[mb] = a + (size_t)min(m, M - 1) * lda + g * 8;
+    }
+    f32x4 acc[RB][MB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    for (int k = k_begin; k < k_end; k += kStepK * U) {
+        bf16x8 wf[U][RB], af[U][MB];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int kk = k + u * kStepK;
+            const bool ok = kk + g * 8 < k_end;           // K % 8 == 0: a 16-byte load is in or out as a whole
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) wf[u][rb] = load_frag(wrow[rb] + kk, ok);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) af[u][mb] = load_frag(arow[mb] + kk, ok && a_ok[mb]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+                    acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][rb], af[u][mb], acc[rb][mb], 0, 0, 0);
+    }
+
+    // acc[rb][mb][i] = sum for row n0 + rb * 16 + 4 g + i of w and activation row mb * 16 + r
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[wave][rb * MB + mb][lane][i] = acc[rb][mb][i];
+    __syncthreads();
+
+    const int t_lane = threadIdx.x & (kWave - 1), t_i = threadIdx.x / kWave;   // 256 threads: one (lane, i) each
+    TO* dst = out + (size_t)split * part_stride;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+        const int n = n0 + rb * 16 + 4 * (t_lane >> 4) + t_i;
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            float s = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < kSkinnyWaves; ++wv) s += red[wv][rb * MB + mb][t_lane][t_i];
+            const int m = mb * 16 + (t_lane & 15);
+            if (m < M && n < N) store_f32(dst + (size_t)m * ldo + n, s + (bias ? bias[n] : 0.f));
+        }
+    }
+}
+
+template <int RB, int MB, int U>
+static int launch_skinny(void* out, int out_dtype, const bf16_t* a, const bf16_t* w, const float* bias,
+                         int M, int N, int K, int lda, int ldo, size_t part_stride, int k_per_block,
+                         int k_splits, hipStream_t stream) {
+    dim3 grid((N + 16 * RB - 1) / (16 * RB), k_splits);
+    if (out_dtype == DT_BF16)
+        gemm_skinny_kernel<RB, MB, U, bf16_t><<<grid, kSkinnyWaves * kWave, 0, stream>>>(
+            (bf16_t*)out, a, w, bias, M, N, K, lda, ldo, part_stride, k_per_block);
+    else
+        gemm_skinny_kernel<RB, MB, U, float><<<grid, kSkinnyWaves * kWave, 0, stream>>>(
+            (float*)out, a, w, bias, M, N, K, lda, ldo, part_stride, k_per_block);
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+// k range of one block for `splits` blocks along k: a multiple of 4 waves * 32.
+static int k_per_block_for(int K, int splits) {
+    const int unit = kSkinnyWaves * kStepK;
+    return ((K + splits - 1) / splits + unit - 1) / unit * unit;
+}
+
+// The number of parts the product is written in for `splits` requested blocks along k
+// (rounding k per block up can need fewer blocks than asked for).
+LLOGOS_EXPORT int llogos_gemm_skinny_parts(int K, int splits) {
+    if (K <= 0 || splits <= 1) return 1;
+    const int kpb = k_per_block_for(K, splits);
+    return (K + kpb - 1) / kpb;
+}
+
+// out: [parts][M][ldo] with parts = llogos_gemm_skinny_parts(K, splits); float32 when parts > 1
+// (bias must then be left to the consumer).  row_blocks: 16-row blocks of w per wave (1, 2, 4).
+// Returns LLOGOS_UNSUPPORTED for shapes this kernel does not take.
+LLOGOS_EXPORT int llogos_gemm_skinny_bf16(void* out, int out_dtype, const void* a, const void* w,
+                                          const float* bias, int M, int N, int K, int lda, int ldo,
+                                          long long part_stride, int splits, int row_blocks,
+                                          hipStream_t stream) {
+    if (M <= 0 || N <= 0 || K <= 0 || lda < K || ldo < N || splits < 1) return LLOGOS_BAD_ARGUMENT;
+    if (out_dtype != DT_BF16 && out_dtype != DT_F32) return LLOGOS_BAD_ARGUMENT;
+    if (M > 64 || (K % 8) || (lda % 8) || ((uintptr_t)a % 16) || ((uintptr_t)w % 16)) return LLOGOS_UNSUPPORTED;
+    const int parts = llogos_gemm_skinny_parts(K, splits);
+    if (parts > 1 && (out_dtype != DT_F32 || bias != nullptr || part_stride < (long long)M * ldo))
+        return LLOGOS_BAD_ARGUMENT;
+    const int kpb = k_per_block_for(K, parts);
+    const bf16_t* A = (const bf16_t*)a;
+    const bf16_t* W = (const bf16_t*)w;
+    const int mb = (M + 15) / 16;
+#define GO(RB, MB, U) return launch_skinny<RB, MB, U>(out, out_dtype, A, W, bias, M, N, K, lda, ldo, \
+                                                      (size_t)part_stride, kpb, parts, stream)
+    if (mb == 1) {
+        if (row_blocks >= 4) GO(4, 1, 4);
+        if (row_blocks == 2) GO(2, 1, 8);
+        GO(1, 1, 8);
+    } else if (mb == 2) {
+        if (row_blocks >= 4) GO(4, 2, 2);
+        if (row_blocks == 2) GO(2, 2, 4);
+        GO(1, 2, 4);
+    } else {
+        if (row_blocks >= 4) GO(4, 4, 2);
+        if (row_blocks == 2) GO(2, 4, 2);
+        GO(1, 4, 4);
+    }
+#undef GO
+}

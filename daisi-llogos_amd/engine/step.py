@@ -83,6 +83,37 @@ class Engine:
             ckpt.close()
         return cls(model, rt, max_tokens, n_slots, config)
 
+    @classmethod
+    def from_config(cls, config: dict, seed: int = 0, dtype: Union[str, torch.dtype] = "bfloat16",
+                    max_tokens: int = 4096, n_slots: int = 64, device: Union[str, torch.device] = "cuda:0",
+                    std: float = 0.02, **spec_options) -> "Engine":
+        """A model of the parsed config.json `config` with random weights made on the device
+        (matrices N(0, std), norm weights 1 + U(-0.1, 0.1)), without a model folder."""
+        import hashlib
+        dev = require_gpu(device)
+        arch = architecture_of(config)
+        typed = arch.read_config(config)
+        model = Model(arch.model_spec(typed, **spec_options))
+        specs = {s.name: s for s in model.tensor_specs()}
+        rt = Runtime(dev, resolve_dtype(dtype))
+        gen = torch.Generator(device=dev)
+
+        def get(name: str):
+            spec = specs.get(name)
+            if spec is None:
+                return None
+            digest = hashlib.sha256(f"{seed}:{name}".encode()).digest()
+            gen.manual_seed(int.from_bytes(digest[:8], "little") & ((1 << 63) - 1))
+            if spec.kind == "norm":
+                return 1.0 + (torch.rand(spec.shape, generator=gen, device=dev) * 0.2 - 0.1)
+            t = torch.empty(spec.shape, dtype=rt.dtype if spec.kind in ("matrix", "table") else torch.float32,
+                            device=dev)
+            return t.normal_(0.0, std, generator=gen)
+        with torch.cuda.device(dev):
+            model.bind(get, rt)
+            torch.cuda.synchronize()
+        return cls(model, rt, max_tokens, n_slots, typed)
+
     # ---- slots ---------------------------------------------------------------------
     def alloc_slot(self) -> int:
         return self.cache.alloc_slot()

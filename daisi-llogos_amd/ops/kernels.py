@@ -7,7 +7,7 @@ tensors used as device memory; launches go to torch's current stream.
 from __future__ import annotations
 
 import ctypes
-from typing import Optional, Sequence
+from typing import Optional, Sequence, Tuple
 
 import torch
 
@@ -68,6 +68,22 @@ def _i32(t: Optional[torch.Tensor], name: str) -> None:
         _need(t.dtype == torch.int32, f"{name} must be int32")
 
 
+def _parts(t: Optional[torch.Tensor]) -> Tuple[int, int]:
+    """(number of parts, elements between parts) of a product: [T, N] is one part,
+    [P, T, N] are P partial sums that the consumer adds."""
+    if t is None or t.dim() == 2:
+        return 1, 0
+    _need(t.dim() == 3, "a product must be [T, N] or [parts, T, N]")
+    return t.shape[0], t.stride(0)
+
+
+def _check_pools(k_pool: torch.Tensor, v_pool: torch.Tensor, n_kv_heads: int, head_dim: int, who: str) -> None:
+    _need(tuple(k_pool.shape[1:]) == (n_kv_heads, PAGE_TOKENS, head_dim),
+          f"{who}: key pool must be [pages, kv_heads, {PAGE_TOKENS}, head_dim]")
+    _need(tuple(v_pool.shape) == (k_pool.shape[0], n_kv_heads, head_dim, PAGE_TOKENS),
+          f"{who}: value pool must be [pages, kv_heads, head_dim, {PAGE_TOKENS}] (transposed pages)")
+
+
 # ----------------------------------------------------------------------------
 def embed(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
     """float32 rows of `table` ([V, H], float32 or bfloat16) at int32 `ids`."""
@@ -83,21 +99,23 @@ def embed(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
             delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
             write_back: bool = True) -> torch.Tensor:
-    """RMSNorm of the float32 residual stream `x` [T, H] with the pending `delta` added
-    first (and written back to `x` when `write_back`).  With `rows` only those rows are
-    normed, into a compact output."""
+    """RMSNorm of the float32 residual stream `x` [T, H] with the pending `delta` ([T, H] or
+    partial sums [parts, T, H]) added first (and written back to `x` when `write_back`).
+    With `rows` only those rows are normed, into a compact output."""
     _dev(x, weight, delta, rows)
     _i32(rows, "rows")
     _need(x.dtype == torch.float32 and x.dim() == 2, "rmsnorm: x must be float32 [T, H]")
     T, H = x.shape
     _need(weight.dtype == torch.float32 and weight.shape == (H,), "rmsnorm: weight must be float32 [H]")
+    parts, part_stride = _parts(delta)
     if delta is not None:
-        _need(delta.shape == x.shape, "rmsnorm: delta must have x's shape")
+        _need(tuple(delta.shape[-2:]) == tuple(x.shape), "rmsnorm: delta must have x's shape")
     R = rows.numel() if rows is not None else T
     out = torch.empty((R, H), dtype=out_dtype, device=x.device)
     if R == 0:
         return out
     _check(_lib().llogos_rmsnorm(_p(out), _DT[out_dtype], _p(x), _p(delta), _dt(delta) if delta is not None else F32,
+                                 parts, ctypes.c_longlong(part_stride),
                                  _p(rows), _p(weight), ctypes.c_float(eps), R, H, int(write_back), _stream()),
            "rmsnorm")
     return out
@@ -142,35 +160,43 @@ def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
     return cs
 
 
-def qk_rope_cache(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, rot: int, pairing: int,
+def qk_rope_cache(qkv: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype,
+                  n_heads: int, n_kv_heads: int, head_dim: int, rot: int, pairing: int,
                   q_norm_w: Optional[torch.Tensor], k_norm_w: Optional[torch.Tensor], eps: float,
                   cs: torch.Tensor, k_pool: Optional[torch.Tensor], v_pool: Optional[torch.Tensor],
-                  table: Optional[torch.Tensor], tok_seq: torch.Tensor, tok_pos: torch.Tensor) -> None:
-    """Per-head norm (optional), rotation and cache write on the fused projection rows
-    [q | k | v] in place: q stays in `qkv`, k and v go to their pages."""
-    _dev(qkv, q_norm_w, k_norm_w, cs, k_pool, v_pool, table, tok_seq, tok_pos)
+                  table: Optional[torch.Tensor], tok_seq: torch.Tensor, tok_pos: torch.Tensor) -> torch.Tensor:
+    """From the fused projection rows [q | k | v] ([T, W] or partial sums [parts, T, W], plus
+    `bias` [W]): per-head norm (optional) and rotation of q and k; q is returned
+    [T, n_heads * head_dim] in `out_dtype`, k and v go to their cache pages."""
+    _dev(qkv, bias, q_norm_w, k_norm_w, cs, k_pool, v_pool, table, tok_seq, tok_pos)
     _i32(tok_seq, "tok_seq"); _i32(tok_pos, "tok_pos"); _i32(table, "table")
-    T = qkv.shape[0]
+    parts, part_stride = _parts(qkv)
+    T = qkv.shape[-2]
     width = (n_heads + 2 * n_kv_heads) * head_dim
-    _need(qkv.dim() == 2 and qkv.shape[1] == width, f"qk_rope_cache: qkv must be [T, {width}]")
+    _need(qkv.shape[-1] == width, f"qk_rope_cache: qkv must be [T, {width}]")
+    _need(qkv.dtype == out_dtype or qkv.dtype == torch.float32, "qk_rope_cache: qkv must be float32 or the cache's type")
     _need(0 < head_dim <= MAX_HEAD_DIM, f"qk_rope_cache: head_dim {head_dim} not in 1..{MAX_HEAD_DIM}")
     _need(rot % 2 == 0 and 0 <= rot <= head_dim, "qk_rope_cache: rotary dimension must be even and <= head_dim")
     _need(cs.dtype == torch.float32 and cs.shape == (T, rot // 2, 2), "qk_rope_cache: rotary table shape")
     _need(tok_seq.numel() == T and tok_pos.numel() == T, "qk_rope_cache: per-token arrays must have T entries")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.shape == (width,), f"qk_rope_cache: bias must be float32 [{width}]")
     for wgt in (q_norm_w, k_norm_w):
         if wgt is not None:
             _need(wgt.dtype == torch.float32 and wgt.shape == (head_dim,), "qk_rope_cache: norm weight float32 [head_dim]")
     if n_kv_heads > 0:
         _need(k_pool is not None and v_pool is not None and table is not None, "qk_rope_cache: cache missing")
-        _need(k_pool.dtype == qkv.dtype and v_pool.dtype == qkv.dtype, "qk_rope_cache: cache type differs")
-        _need(tuple(k_pool.shape[1:]) == (n_kv_heads, PAGE_TOKENS, head_dim) and k_pool.shape == v_pool.shape,
-              "qk_rope_cache: pool must be [pages, kv_heads, 64, head_dim]")
+        _need(k_pool.dtype == out_dtype and v_pool.dtype == out_dtype, "qk_rope_cache: cache type differs")
+        _check_pools(k_pool, v_pool, n_kv_heads, head_dim, "qk_rope_cache")
         _need(table.dim() == 2, "qk_rope_cache: page table must be [batch, pages]")
+    q_out = torch.empty((T, n_heads * head_dim), dtype=out_dtype, device=qkv.device)
     _check(_lib().llogos_qk_rope_cache(
-        _p(qkv), _dt(qkv), qkv.stride(0), n_heads, n_kv_heads, head_dim, rot, pairing,
+        _p(qkv), _dt(qkv), parts, ctypes.c_longlong(part_stride), qkv.stride(-2), _p(bias), _p(q_out), _DT[out_dtype],
+        n_heads, n_kv_heads, head_dim, rot, pairing,
         _p(q_norm_w), _p(k_norm_w), ctypes.c_float(eps), _p(cs), _p(k_pool), _p(v_pool),
         _p(table), table.stride(0) if table is not None else 0, _p(tok_seq), _p(tok_pos), T, _stream()),
         "qk_rope_cache")
+    return q_out
 
 
 def attention_generic(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
@@ -185,8 +211,7 @@ def attention_generic(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_po
     _need(q.is_cuda and q.dtype == k_pool.dtype, "attention: q and cache types differ")
     _need(n_heads % n_kv_heads == 0, "attention: heads must be a multiple of kv heads")
     _need(0 < head_dim <= MAX_HEAD_DIM, f"attention: head_dim {head_dim} not in 1..{MAX_HEAD_DIM}")
-    _need(tuple(k_pool.shape[1:]) == (n_kv_heads, PAGE_TOKENS, head_dim) and k_pool.shape == v_pool.shape,
-          "attention: pool must be [pages, kv_heads, 64, head_dim]")
+    _check_pools(k_pool, v_pool, n_kv_heads, head_dim, "attention")
     _need(q_stride >= n_heads * head_dim and q.numel() >= (T - 1) * q_stride + n_heads * head_dim,
           "attention: q too small")
     out = torch.empty((T, n_heads * head_dim), dtype=q.dtype, device=q.device)
@@ -197,13 +222,31 @@ def attention_generic(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_po
     return out
 
 
-def swiglu(gu: torch.Tensor) -> torch.Tensor:
-    """silu(gate) * up from fused rows [gate | up]."""
+def swiglu(gu: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """silu(gate) * up from fused rows [gate | up] ([T, 2 I] or partial sums [parts, T, 2 I])."""
     _dev(gu)
-    _need(gu.dim() == 2 and gu.shape[1] % 2 == 0, "swiglu: rows must be [gate | up]")
-    T, I = gu.shape[0], gu.shape[1] // 2
-    out = torch.empty((T, I), dtype=gu.dtype, device=gu.device)
-    _check(_lib().llogos_swiglu(_p(out), _p(gu), _dt(gu), T, I, _stream()), "swiglu")
+    parts, part_stride = _parts(gu)
+    _need(gu.shape[-1] % 2 == 0, "swiglu: rows must be [gate | up]")
+    out_dtype = out_dtype or gu.dtype
+    _need(gu.dtype == out_dtype or gu.dtype == torch.float32, "swiglu: input must be float32 or the output's type")
+    T, I = gu.shape[-2], gu.shape[-1] // 2
+    out = torch.empty((T, I), dtype=out_dtype, device=gu.device)
+    _check(_lib().llogos_swiglu(_p(out), _DT[out_dtype], _p(gu), _dt(gu), parts, ctypes.c_longlong(part_stride),
+                                T, I, _stream()), "swiglu")
+    return out
+
+
+def sum_parts(product: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype) -> torch.Tensor:
+    """One plain [T, N] tensor of `out_dtype` from a product that may come in parts, plus bias."""
+    _dev(product, bias)
+    parts, part_stride = _parts(product)
+    if parts == 1 and bias is None and product.dtype == out_dtype:
+        return product if product.dim() == 2 else product[0]
+    _need(parts == 1 or product.dtype == torch.float32, "sum_parts: parts must be float32")
+    T, N = product.shape[-2:]
+    out = torch.empty((T, N), dtype=out_dtype, device=product.device)
+    _check(_lib().llogos_sum_parts(_p(out), _DT[out_dtype], _p(product), _dt(product), parts, ctypes.c_longlong(part_stride),
+                                   _p(bias), T, N, _stream()), "sum_parts")
     return out
 
 
@@ -220,8 +263,96 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
 # ----------------------------------------------------------------------------
 # dispatch: which kernel serves a call
 # ----------------------------------------------------------------------------
+SKINNY_MAX_ROWS = 64
+
+
+def skinny_plan(M: int, N: int, K: int) -> Tuple[int, int]:
+    """(blocks along k, 16-row blocks of w per wave) for the few-row product.  The split of k
+    depends on N and K alone, so the order of a row's additions does not depend on how many
+    other rows the batch has; wider strips with more rows re-read the activations less."""
+    strips = -(-N // 16)
+    splits = max(1, min(-(-1024 // strips), K // 1024, 8))
+    if M <= 8:
+        row_blocks = 4 if N >= 65536 and M > 4 else 1
+    elif M <= 16:
+        row_blocks = 4 if N >= 16384 else 2
+    else:
+        row_blocks = 4
+    return splits, row_blocks
+
+
+def gemm_skinny_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype,
+                     splits: int = 1, row_blocks: int = 1) -> Optional[torch.Tensor]:
+    """The few-row bfloat16 product on the matrix cores: [parts, M, N], where parts > 1 are
+    float32 partial sums over ranges of k that the consumer adds (then no bias is applied
+    here).  None when the shape is not one the kernel takes."""
+    M, K = a.shape
+    N = w.shape[0]
+    if not (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and 0 < M <= SKINNY_MAX_ROWS and K % 8 == 0
+            and a.stride(1) == 1 and a.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+            and w.is_contiguous()):
+        return None
+    _dev(w, bias)
+    _need(w.dim() == 2 and w.shape[1] == K, f"gemm: w must be [N, {K}], got {tuple(w.shape)}")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.shape == (N,), "gemm: bias must be float32 [N]")
+    lib = _lib()
+    parts = lib.llogos_gemm_skinny_parts(K, int(splits))
+    if parts > 1:
+        _need(bias is None, "gemm: a product in parts leaves the bias to its consumer")
+        out_dtype = torch.float32
+    out = torch.empty((parts, M, N), dtype=out_dtype, device=a.device)
+    code = lib.llogos_gemm_skinny_bf16(
+        _p(out), _DT[out_dtype], _p(a), _p(w), _p(bias), M, N, K, a.stride(0), N,
+        ctypes.c_longlong(M * N), int(splits), int(row_blocks), _stream())
+    if code == -2:
+        return None
+    _check(code, "gemm_skinny_bf16")
+    return out
+
+
+def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """a [M, K] . w [N, K]^T without bias, as [M, N] of `out_dtype` or as float32 partial sums
+    [parts, M, N] for a consumer that adds them (rmsnorm, qk_rope_cache, swiglu, sum_parts).
+
+    float32 operands: plain FMAs in 32-bit throughout.  bfloat16 operands: up to 64 rows the
+    hand-written weight-streaming kernel; more rows the library product (as the reference
+    uses a library for its prompt products, Daisi.Llogos.Cuda/CudaBackend.cs:158-316)."""
+    if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
+        M = a.shape[0]
+        if M <= SKINNY_MAX_ROWS:
+            splits, row_blocks = skinny_plan(M, w.shape[0], w.shape[1])
+            out = gemm_skinny_bf16(a, w, None, out_dtype, splits, row_blocks)
+            if out is not None:
+                return out
+        elif out_dtype == torch.bfloat16 and a.is_contiguous():
+            return torch.matmul(a, w.t())
+    return gemm_generic(a, w, None, out_dtype)
+
+
 def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype) -> torch.Tensor:
-    """a [M, K] . w [N, K]^T (+ bias [N]) -> [M, N] of `out_dtype`."""
+    """a [M, K] . w [N, K]^T (+ bias [N]) -> one plain [M, N] tensor of `out_dtype`."""
+    if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
+        M = a.shape[0]
+        if M <= SKINNY_MAX_ROWS:
+            _, row_blocks = skinny_plan(M, w.shape[0], w.shape[1])
+            out = gemm_skinny_bf16(a, w, bias, out_dtype, 1, row_blocks)
+            if out is not None:
+                return out[0]
+        elif out_dtype == torch.bfloat16 and a.is_contiguous():
+            out = torch.matmul(a, w.t())
+            if bias is not None:
+                out += bias.to(torch.bfloat16)
+            return out
+        elif out_dtype == torch.float32 and a.is_contiguous() and a.shape[1] % 8 == 0:
+            # float32 results for many rows: row blocks through the hand-written kernel
+            out = torch.empty((M, w.shape[0]), dtype=torch.float32, device=a.device)
+            for r in range(0, M, SKINNY_MAX_ROWS):
+                blk = gemm_skinny_bf16(a[r:r + SKINNY_MAX_ROWS], w, bias, torch.float32, 1, 4)
+                if blk is None:
+                    return gemm_generic(a, w, bias, out_dtype)
+                out[r:r + SKINNY_MAX_ROWS] = blk[0]
+            return out
     return gemm_generic(a, w, bias, out_dtype)
 
 

@@ -64,7 +64,7 @@ class GroupView:
 class LayerCache:
     """What one scheduled layer sees of the cache in a step."""
     k_pool: Optional[torch.Tensor] = None     # [pages, kv_heads, 64, head_dim]
-    v_pool: Optional[torch.Tensor] = None
+    v_pool: Optional[torch.Tensor] = None     # [pages, kv_heads, head_dim, 64] (transposed pages)
     table: Optional[torch.Tensor] = None      # int32 [batch, pages]
     writes: bool = True                       # False: reads the pages another layer wrote
     state: Optional[torch.Tensor] = None      # [slots, *StateSpec.shape]
@@ -105,7 +105,8 @@ class Part:
 
 
 class Mixer(Part):
-    """Token mixer: forward(ctx, h [T, H] in the runtime's type, cache) -> [T, H]."""
+    """Token mixer: forward(ctx, h [T, H] in the runtime's type, cache) -> [T, H], or float32
+    partial sums [parts, T, H] that the residual sum after it adds."""
 
     def kv_spec(self) -> Optional[KVSpec]:
         return None
@@ -118,7 +119,7 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    """forward(ctx, h [T, H]) -> [T, H]."""
+    """forward(ctx, h [T, H]) -> [T, H], or float32 partial sums [parts, T, H]."""
 
     def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
@@ -126,7 +127,8 @@ class FeedForward(Part):
 
 class Norm(Part):
     """forward(x, delta, rows) -> normed rows in the runtime's type.  `x` is the float32
-    residual stream; a pending `delta` is added to it first (in place)."""
+    residual stream; a pending `delta` ([T, H] or partial sums [parts, T, H]) is added to it
+    first (in place)."""
 
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None,
                 rows: Optional[torch.Tensor] = None, write_back: bool = True) -> torch.Tensor:

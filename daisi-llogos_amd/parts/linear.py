@@ -48,6 +48,15 @@ class Linear(Part):
         self.rt = rt
         self.weight = weight
 
+    def product(self, a: torch.Tensor, rows_out: Optional[int] = None) -> torch.Tensor:
+        """a . W^T without the bias, as [M, out] or as float32 partial sums [parts, M, out] for a
+        consumer kernel that adds parts (and the bias, `bias_rows`)."""
+        w = self.weight if rows_out is None else self.weight[:rows_out]
+        return K.gemm_product(a, w, self.rt.dtype)
+
+    def bias_rows(self, rows_out: Optional[int] = None) -> Optional[torch.Tensor]:
+        return self.bias if (self.bias is None or rows_out is None) else self.bias[:rows_out]
+
     def forward(self, a: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
                 rows_out: Optional[int] = None) -> torch.Tensor:
         """a [M, in] -> [M, out]; `rows_out` uses only the first rows of the stacked matrix."""

@@ -29,5 +29,5 @@ class SwiGLU(FeedForward):
         self.down.bind(get, rt)
 
     def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
-        gu = self.gate_up.forward(h)
-        return self.down.forward(K.swiglu(gu))
+        gu = self.gate_up.product(h)
+        return self.down.product(K.swiglu(gu, self.rt.dtype))      # the residual sum that follows adds the parts

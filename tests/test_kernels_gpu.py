@@ -84,6 +84,32 @@ def test_gemm(dtype, M, N, K_):
     assert _np(o).tolist() == [[58, 64], [139, 154]]
 
 
+@pytest.mark.parametrize("M,N,K_", [(1, 4096, 4096), (8, 331, 1000), (16, 100, 72), (17, 4096, 14336), (64, 257, 2048),
+                                    (33, 6144, 4096)])
+def test_gemm_few_rows_on_the_matrix_cores(M, N, K_):
+    rng = np.random.default_rng(7)
+    a = _t(rng.standard_normal((M, K_)), torch.bfloat16)
+    w = _t(rng.standard_normal((N, K_)) * 0.05, torch.bfloat16)
+    b = _t(rng.standard_normal(N))
+    want = pm.linear(_np(a), _np(w))
+    scale = np.abs(want).max()
+    for splits in (1, 2, 5, 8):
+        for rb in (1, 2, 4):
+            out = K.gemm_skinny_bf16(a, w, None, torch.float32, splits, rb)
+            assert out is not None and out.dtype == torch.float32 and out.shape[1:] == (M, N)
+            assert np.abs(_np(out).sum(0) - want).max() <= 2e-6 * scale * math.sqrt(K_)
+    plain = K.gemm(a, w, b, torch.bfloat16)
+    assert np.abs(_np(plain) - (want + _np(b))).max() <= 1e-2 * scale
+    prod = K.gemm_product(a, w, torch.bfloat16)
+    assert np.abs(_np(K.sum_parts(prod, b, torch.float32)) - (want + _np(b))).max() <= (1e-2 if prod.dtype == torch.bfloat16 else 1e-5) * scale
+    # a row's result does not depend on how many rows the batch has
+    if M > 1:
+        alone = K.sum_parts(K.gemm_product(a[:1], w, torch.bfloat16), None, torch.float32)
+        many = K.sum_parts(prod, None, torch.float32)[:1]
+        assert torch.equal(alone, many)
+    assert K.gemm_skinny_bf16(a[:, :K_ - 4], w[:, :K_ - 4].contiguous(), None, torch.float32) is None   # k % 8
+
+
 def test_rope_table_is_double_precision():
     pos = _t([0, 1, 4095, 100000], torch.int32)
     f = pm.rope_frequencies(64, 5e5)
@@ -111,31 +137,38 @@ def test_qk_rope_cache(dtype, nh, nkv, hd, rot, pairing, norm):
     tok_seq = np.repeat(np.arange(2), new).astype(np.int32)
     tok_pos = np.concatenate([np.arange(l - n, l) for l, n in zip(lens, new)]).astype(np.int32)
     table, n_pages = _pages(2, 70, rng)
-    qkv = _t(rng.standard_normal((T, (nh + 2 * nkv) * hd)), DT[dtype])
-    orig = _np(qkv)
+    width = (nh + 2 * nkv) * hd
+    qkv = _t(rng.standard_normal((T, width)), DT[dtype])
+    bias = _t(rng.standard_normal(width)) if norm else None              # bias and norm together: bias first
+    orig = _np(qkv) + (_np(bias) if bias is not None else 0)
     qw = 1 + 0.1 * rng.standard_normal(hd)
     kw = 1 + 0.1 * rng.standard_normal(hd)
     f = pm.rope_frequencies(rot, 1e4)
     cs = K.rope_table(_t(tok_pos, torch.int32), _t(f, torch.float64))
     kp = torch.zeros((n_pages, nkv, 64, hd), dtype=DT[dtype], device=DEV)
-    vp = torch.zeros_like(kp)
-    K.qk_rope_cache(qkv, nh, nkv, hd, rot, pairing, _t(qw) if norm else None, _t(kw) if norm else None, 1e-5,
-                    cs, kp, vp, _t(table, torch.int32), _t(tok_seq, torch.int32), _t(tok_pos, torch.int32))
+    vp = torch.zeros((n_pages, nkv, hd, 64), dtype=DT[dtype], device=DEV)     # value pages are transposed
+    args = (nh, nkv, hd, rot, pairing, _t(qw) if norm else None, _t(kw) if norm else None, 1e-5,
+            cs, kp, vp, _t(table, torch.int32), _t(tok_seq, torch.int32), _t(tok_pos, torch.int32))
+    q_out = K.qk_rope_cache(qkv, bias, DT[dtype], *args)
+    # the same projection as three float32 partial sums gives the same result
+    third = qkv.float() / 4
+    q_parts = K.qk_rope_cache(torch.stack([third, 2 * third, third]), bias, DT[dtype], *args)
+    assert torch.equal(q_parts, q_out)
     q, k, v = orig[:, :nh * hd], orig[:, nh * hd:(nh + nkv) * hd], orig[:, (nh + nkv) * hd:]
     if norm:
         q = pm.per_head_rms_norm(q, qw, nh, hd, 1e-5)
         k = pm.per_head_rms_norm(k, kw, nkv, hd, 1e-5)
     rope = pm.rope_split_half if pairing == 0 else pm.rope_interleaved
     q, k = rope(q, tok_pos, nh, hd, f), rope(k, tok_pos, nkv, hd, f)
-    _close(qkv[:, :nh * hd], q, dtype)
+    _close(q_out, q, dtype)
     kc, vc = _np(kp), _np(vp)
     for t in range(T):
         page = table[tok_seq[t], tok_pos[t] // 64]
         got_k = kc[page, :, tok_pos[t] % 64, :].reshape(-1)
-        got_v = vc[page, :, tok_pos[t] % 64, :].reshape(-1)
+        got_v = vc[page, :, :, tok_pos[t] % 64].reshape(-1)
         assert np.abs(got_k - k[t]).max() <= RT[dtype] * max(1, np.abs(k).max())
         assert np.abs(got_v - v[t]).max() <= RT[dtype] * max(1, np.abs(v).max())
-    assert np.count_nonzero(kc) == T * nkv * hd                         # nothing else was written
+    assert np.count_nonzero(kc) == T * nkv * hd and np.count_nonzero(vc) == T * nkv * hd   # nothing else was written
 
 
 def _attention_case(dtype, nh, nkv, hd, lens, new, window=0, sinks=0, seed=4, scale_q=1.0):
@@ -145,7 +178,7 @@ def _attention_case(dtype, nh, nkv, hd, lens, new, window=0, sinks=0, seed=4, sc
     B, T = len(lens), sum(new)
     table, n_pages = _pages(B, max(lens), rng)
     kp = torch.zeros((n_pages, nkv, 64, hd), dtype=DT[dtype], device=DEV)
-    vp = torch.zeros_like(kp)
+    vp = torch.zeros((n_pages, nkv, hd, 64), dtype=DT[dtype], device=DEV)
     ks = [rng.standard_normal((l, nkv * hd)) for l in lens]
     vs = [rng.standard_normal((l, nkv * hd)) for l in lens]
     for b in range(B):
@@ -153,7 +186,7 @@ def _attention_case(dtype, nh, nkv, hd, lens, new, window=0, sinks=0, seed=4, sc
         ks[b], vs[b] = _np(kb), _np(vb)
         for p in range(lens[b]):
             kp[table[b, p // 64], :, p % 64, :] = kb[p].view(nkv, hd)
-            vp[table[b, p // 64], :, p % 64, :] = vb[p].view(nkv, hd)
+            vp[table[b, p // 64], :, :, p % 64] = vb[p].view(nkv, hd)
     stride = nh * hd + 24                                               # queries sit in a wider row
     qbuf = _t(rng.standard_normal((T, stride)) * scale_q, DT[dtype])
     tok_seq = np.repeat(np.arange(B), new).astype(np.int32)
@@ -241,6 +274,9 @@ def test_swiglu(dtype):
     gu = _t(rng.standard_normal((9, 2 * 137)) * 4, DT[dtype])
     g, u = _np(gu)[:, :137], _np(gu)[:, 137:]
     _close(K.swiglu(gu), pm.silu(g) * u, dtype)
+    parts = torch.stack([gu.float() * 0.25, gu.float() * 0.75])
+    _close(K.swiglu(parts, DT[dtype]), pm.silu(g) * u, dtype)
+    _close(K.sum_parts(parts, None, DT[dtype]), _np(gu), dtype)
 
 
 def test_argmax_first_maximum_wins():
@@ -266,6 +302,6 @@ def test_kernels_refuse_what_they_cannot_do():
     with pytest.raises(K.KernelError, match="not supported"):
         K.gemm(x.half(), torch.zeros(8, 64, device=DEV).half(), None, torch.float16)
     with pytest.raises(K.KernelError, match="head_dim"):
-        K.qk_rope_cache(torch.zeros(1, 3 * 1024, device=DEV), 1, 1, 1024, 2, 0, None, None, 1e-6,
+        K.qk_rope_cache(torch.zeros(1, 3 * 1024, device=DEV), None, torch.float32, 1, 1, 1024, 2, 0, None, None, 1e-6,
                         torch.zeros(1, 1, 2, device=DEV), None, None, None,
                         torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV))

@@ -133,11 +133,12 @@ def test_attention_part_alone(dtype, nh, nkv, hd, bias, qk_norm, window):
     q, k = pm.rope_split_half(q, range(T), nh, hd, f), pm.rope_split_half(k, range(T), nkv, hd, f)
     want = pm.linear(pm.attention(q, k, v, nh, nkv, hd, window=window), plain["a.o_proj.weight"])
     # engine part, with a cache of its own
-    pool = lambda: torch.zeros((3, nkv, 64, hd), dtype=DT[dtype], device=DEV)
-    cache = P.LayerCache(k_pool=pool(), v_pool=pool(), table=torch.tensor([[2, 0]], dtype=torch.int32, device=DEV))
-    outs = [att.forward(_ctx(rt, [68], [68]), x[:68].to(DEV), cache)]
+    pool = lambda *shape: torch.zeros((3, nkv) + shape, dtype=DT[dtype], device=DEV)
+    cache = P.LayerCache(k_pool=pool(64, hd), v_pool=pool(hd, 64), table=torch.tensor([[2, 0]], dtype=torch.int32, device=DEV))
+    plain_out = lambda o: K.sum_parts(o, None, DT[dtype])            # a mixer may hand on partial sums
+    outs = [plain_out(att.forward(_ctx(rt, [68], [68]), x[:68].to(DEV), cache))]
     for t in (68, 69):
-        outs.append(att.forward(_ctx(rt, [t + 1], [1]), x[t:t + 1].to(DEV), cache))
+        outs.append(plain_out(att.forward(_ctx(rt, [t + 1], [1]), x[t:t + 1].to(DEV), cache)))
     got = _np(torch.cat(outs))
     assert np.abs(got - want).max() <= TOL[dtype] * max(1.0, np.abs(want).max())
 
@@ -153,7 +154,8 @@ def test_swiglu_part_alone(dtype):
     ffn.bind(tensors.get, rt)
     x, x_ = _rand(rng, (9, 40), dtype)
     want = pm.swiglu_mlp(x_, plain["m.gate_proj.weight"], plain["m.up_proj.weight"], plain["m.down_proj.weight"])
-    assert np.abs(_np(ffn.forward(None, x.to(DEV))) - want).max() <= TOL[dtype] * max(1.0, np.abs(want).max())
+    got = K.sum_parts(ffn.forward(None, x.to(DEV)), None, DT[dtype])
+    assert np.abs(_np(got) - want).max() <= TOL[dtype] * max(1.0, np.abs(want).max())
 
 
 # ---------------------------------------------------------------------------
