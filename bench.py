@@ -1,0 +1,162 @@
+"""Decode and prefill throughput of the Llama-3.1-8B layer sizes with random bfloat16
+weights on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+
+A step is one decode step of the whole batch.  The line printed at the end is the record:
+value = decoded tokens a second at the default batch of 8 (512-token random prompts, the
+context grows from there), "prefill" = one 2,048-token prompt, "roofline" = bytes the decode
+step has to read (every weight it uses once, the cache of the live requests) / its time
+against 8 TB/s, "points" = decoding at batch 1 and 64."""
+import argparse
+import importlib
+import json
+import sys
+import time
+
+HBM_PEAK = 8.0e12            # bytes/s, MI355X
+MFMA_PEAK = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}   # dense flop/s
+
+LLAMA31_8B = {
+    "architectures": ["LlamaForCausalLM"], "vocab_size": 128256, "hidden_size": 4096, "intermediate_size": 14336,
+    "num_hidden_layers": 32, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+    "rms_norm_eps": 1e-5, "rope_theta": 500000.0, "max_position_embeddings": 131072,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 8192},
+    "attention_bias": False, "tie_word_embeddings": False, "torch_dtype": "bfloat16", "eos_token_id": 128001,
+}
+CONTEXT, PROMPT, PREFILL_TOKENS = 4096, 512, 2048
+
+
+def weight_bytes(cfg, elt=2):
+    """Bytes of every matrix a decode step reads once: the layers' projections and the head
+    (the embedding table is read for a few rows only)."""
+    h, i, v = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    q = cfg["num_attention_heads"] * cfg["head_dim"]
+    kv = cfg["num_key_value_heads"] * cfg["head_dim"]
+    per_layer = h * (q + 2 * kv) + q * h + 3 * h * i + 2 * h        # + the two norm weights
+    return (cfg["num_hidden_layers"] * per_layer + v * h + h) * elt
+
+
+def kv_bytes_per_token(cfg, elt=2):
+    return cfg["num_hidden_layers"] * 2 * cfg["num_key_value_heads"] * cfg["head_dim"] * elt
+
+
+def prefill_flops(cfg, t):
+    """2 * (matrix parameters) per token, causal attention 2 * 2 * heads * head_dim * t^2 / 2 per
+    layer, the head on one row."""
+    h, i, v = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    q = cfg["num_attention_heads"] * cfg["head_dim"]
+    kv = cfg["num_key_value_heads"] * cfg["head_dim"]
+    linear = cfg["num_hidden_layers"] * (h * (q + 2 * kv) + q * h + 3 * h * i)
+    attn = cfg["num_hidden_layers"] * 2 * q * t * t                  # qk^T and pv, half of the square each
+    return 2 * linear * t + attn + 2 * v * h
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration has (0 = all)")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    args = ap.parse_args(argv)
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU library")
+        return 2
+
+    import numpy as np
+    import torch
+    llogos = importlib.import_module("daisi-llogos_amd")
+    K = importlib.import_module("daisi-llogos_amd.ops.kernels")
+
+    cfg = dict(LLAMA31_8B)
+    full_layers = cfg["num_hidden_layers"]
+    if args.layers:
+        cfg["num_hidden_layers"] = args.layers
+    max_batch = max(args.batch, 1 if args.no_points else 64)
+    per_seq = PROMPT + args.steps + args.warmup + 64
+    t0 = time.time()
+    eng = llogos.Engine.from_config(cfg, seed=0, dtype="bfloat16",
+                                    max_tokens=max(max_batch * (per_seq + 64), PREFILL_TOKENS + 128), n_slots=max_batch)
+    print(f"[bench] model ready in {time.time() - t0:.1f} s; weights {weight_bytes(cfg) / 1e9:.2f} GB, "
+          f"cache {eng.cache.bytes() / 1e9:.2f} GB", file=sys.stderr, flush=True)
+    rng = np.random.default_rng(0)
+
+    def decode_run(batch, steps, warmup):
+        """Prompts in one step, then greedy single-token steps: `warmup` untimed, `steps` timed."""
+        slots = [eng.alloc_slot() for _ in range(batch)]
+        prompts = [rng.integers(0, cfg["vocab_size"], size=PROMPT).tolist() for _ in range(batch)]
+        logits = eng.step(list(zip(slots, prompts)), want="last")
+        ids = K.argmax(logits).tolist()
+
+        def run(n):
+            nonlocal ids
+            for _ in range(n):
+                logits = eng.step([(s, [t]) for s, t in zip(slots, ids)], want="last")
+                ids = K.argmax(logits).tolist()       # the tokens come to the host every step, as in generation
+        run(warmup)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        run(steps)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        ctx_mid = PROMPT + warmup + steps / 2.0
+        for s in slots:
+            eng.free_slot(s)
+        return dt, ctx_mid
+
+    dt, ctx_mid = decode_run(args.batch, args.steps, args.warmup)
+    ms_per_step = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+    step_bytes = weight_bytes(cfg) + args.batch * ctx_mid * kv_bytes_per_token(cfg)
+    achieved = step_bytes / (dt / args.steps)
+    record = {
+        "metric": "decode tok/s, Llama-3.1-8B bf16", "value": round(value, 1), "unit": "tok/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"model": "Llama-3.1-8B sizes, random weights", "global_batch": args.batch, "seq_len": CONTEXT,
+                   "parallelism": "single GPU", "prompt_len": PROMPT, "layers": cfg["num_hidden_layers"],
+                   "layers_full": full_layers, "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
+                   "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
+                   "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
+                   "rope_theta": cfg["rope_theta"], "rope_scaling": "llama3 x8", "rms_eps": cfg["rms_norm_eps"],
+                   "sampling": "greedy", "hip_graphs": eng.graphs is not None},
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK, 4)},
+    }
+    print(f"[bench] decode b{args.batch}: {value:.1f} tok/s, {ms_per_step:.3f} ms/step, "
+          f"{achieved / 1e12:.2f} TB/s", file=sys.stderr, flush=True)
+
+    if not args.no_points:
+        points = {}
+        for b in (1, 64):
+            steps = min(args.steps, 64)
+            d, _ = decode_run(b, steps, min(args.warmup, 4))
+            points[f"decode_b{b}"] = round(b * steps / d, 1)
+            print(f"[bench] decode b{b}: {points[f'decode_b{b}']:.1f} tok/s, {d / steps * 1e3:.3f} ms/step",
+                  file=sys.stderr, flush=True)
+        record["points"] = points
+        prompt = rng.integers(0, cfg["vocab_size"], size=PREFILL_TOKENS).tolist()
+        times = []
+        for it in range(3):
+            s = eng.alloc_slot()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            eng.step([(s, prompt)], want="last")
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t)
+            eng.free_slot(s)
+        pt = min(times[1:])
+        flops = prefill_flops(cfg, PREFILL_TOKENS)
+        record["prefill"] = {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS, "ms": round(pt * 1e3, 3),
+                             "frac": round(flops / pt / MFMA_PEAK["bf16"], 4)}
+        print(f"[bench] prefill {PREFILL_TOKENS}: {PREFILL_TOKENS / pt:.0f} tok/s, {pt * 1e3:.2f} ms", file=sys.stderr,
+              flush=True)
+    print(json.dumps(record), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

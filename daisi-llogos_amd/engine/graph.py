@@ -1,0 +1,107 @@
+"""Decode steps as HIP graphs.  A step in which every sequence brings one token launches
+the same kernels with the same shapes as the last one; only token ids, positions and page
+tables change, and those live in device memory.  The step is captured once per batch shape
+and replayed, which removes the launch cost of some three hundred kernels per step.
+
+The reference records its single-token forward pass as a CUDA graph and patches it every
+token (Daisi.Llogos.Cuda/CudaBackend.cs:99-141); here nothing is patched: the graph reads
+what changes from a static buffer that is filled before each replay."""
+from __future__ import annotations
+
+from collections import OrderedDict
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from ..parts.base import StepContext
+
+TABLE_BUCKET = 16          # page-table widths are rounded up to this many pages (1024 positions)
+MAX_GRAPHS = 32
+
+
+def bucket_width(width: int) -> int:
+    return -(-max(1, width) // TABLE_BUCKET) * TABLE_BUCKET
+
+
+class DecodeGraph:
+    def __init__(self, engine, batch: int, widths: Tuple[int, ...]):
+        self.engine, self.batch, self.widths = engine, batch, widths
+        rt = engine.rt
+        B = batch
+        self.sizes = [B, B, B, B, B] + [B * w for w in widths]          # ids, seq, pos, slots, rows, tables
+        total = sum(self.sizes)
+        self.host = torch.empty(total, dtype=torch.int32, pin_memory=True)
+        self.host_np = self.host.numpy()
+        self.dev = torch.zeros(total, dtype=torch.int32, device=rt.device)
+        self.views, o = [], 0
+        for n in self.sizes:
+            self.views.append(self.dev[o:o + n])
+            o += n
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.logits: Optional[torch.Tensor] = None
+        self.copied = torch.cuda.Event()
+
+    def _fill(self, ids, tok_pos, slot_ids, tables: List[np.ndarray]) -> None:
+        B = self.batch
+        h = self.host_np
+        self.copied.synchronize()                  # the last step's copy has left the staging buffer
+        h[0:B] = ids
+        h[B:2 * B] = np.arange(B, dtype=np.int32)
+        h[2 * B:3 * B] = tok_pos
+        h[3 * B:4 * B] = slot_ids
+        h[4 * B:5 * B] = np.arange(B, dtype=np.int32)
+        o = 5 * B
+        for t, w in zip(tables, self.widths):
+            block = h[o:o + B * w].reshape(B, w)
+            block[:, :t.shape[1]] = t
+            block[:, t.shape[1]:] = -1
+            o += B * w
+        self.dev.copy_(self.host, non_blocking=True)
+        self.copied.record()
+
+    def _forward(self, max_context: int) -> Optional[torch.Tensor]:
+        eng, v, B = self.engine, self.views, self.batch
+        ctx = StepContext(runtime=eng.rt, n_tokens=B, batch=B, ids=v[0], tok_seq=v[1], tok_pos=v[2], slots=v[3],
+                          cu_seqlens=list(range(B + 1)), starts=[], slot_ids=[], is_decode=True,
+                          max_context=max_context, in_graph=True)
+        tables = [t.view(B, w) for t, w in zip(v[5:], self.widths)]
+        return eng.model.forward(ctx, eng.cache.layer_caches(tables), v[4])
+
+    def run(self, ids, tok_pos, slot_ids, tables: List[np.ndarray]) -> torch.Tensor:
+        self._fill(ids, tok_pos, slot_ids, tables)
+        if self.graph is None:
+            # the longest context this graph may ever see: what its page tables can hold
+            cap = max(self.widths) * 64 if self.widths else 64
+            self._forward(cap)                          # warm up: lazy workspaces are made outside the capture
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                self.logits = self._forward(cap)
+            self.graph = graph
+        self.graph.replay()
+        return self.logits
+
+
+class GraphCache:
+    """Captured decode steps by (batch size, page-table widths); the least recently used
+    graph is dropped when there are too many."""
+
+    def __init__(self, engine):
+        self.engine = engine
+        self.graphs: "OrderedDict[tuple, DecodeGraph]" = OrderedDict()
+
+    def clear(self) -> None:
+        self.graphs.clear()
+
+    def step(self, ids, tok_pos, slot_ids, tables: List[np.ndarray]) -> torch.Tensor:
+        key = (len(slot_ids), tuple(bucket_width(t.shape[1]) for t in tables))
+        g = self.graphs.get(key)
+        if g is None:
+            while len(self.graphs) >= MAX_GRAPHS:
+                self.graphs.popitem(last=False)
+            g = DecodeGraph(self.engine, key[0], key[1])
+            self.graphs[key] = g
+        else:
+            self.graphs.move_to_end(key)
+        return g.run(ids, tok_pos, slot_ids, tables)

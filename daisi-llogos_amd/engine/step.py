@@ -20,6 +20,7 @@ from ..models.model import Model
 from ..ops import library
 from ..parts.base import Runtime, StepContext
 from ..weights.loader import Checkpoint
+from .graph import GraphCache
 
 _DTYPES = {"float32": torch.float32, "fp32": torch.float32, "f32": torch.float32,
            "bfloat16": torch.bfloat16, "bf16": torch.bfloat16}
@@ -53,8 +54,14 @@ def require_gpu(device: Union[str, torch.device] = "cuda:0") -> torch.device:
 class Engine:
     """A bound model with its cache.  `step` is the only way tokens reach the model."""
 
-    def __init__(self, model: Model, rt: Runtime, max_tokens: int, n_slots: int = 64, config=None):
+    def __init__(self, model: Model, rt: Runtime, max_tokens: int, n_slots: int = 64, config=None,
+                 use_graphs: Optional[bool] = None):
         self.model, self.rt, self.config = model, rt, config
+        # single-token steps are replayed as HIP graphs when every mixer allows it
+        graph_ok = all(layer.mixer.graph_safe for layer in model.layers)
+        if use_graphs is None:
+            use_graphs = os.environ.get("LLOGOS_GRAPHS", "1") != "0"
+        self.graphs = GraphCache(self) if (use_graphs and graph_ok) else None
         reads_from = [e.cache_of for e in model.schedule]
         self.cache = Cache(model.cache_needs(), reads_from, max_tokens, rt, n_slots)
         self.vocab_size = model.spec.vocab_size
@@ -115,6 +122,15 @@ class Engine:
         return cls(model, rt, max_tokens, n_slots, typed)
 
     # ---- slots ---------------------------------------------------------------------
+    def _graph_slots(self) -> int:
+        """Captured graphs hold pointers to the per-slot state tensors, which are made anew
+        when the number of slots grows: drop the graphs then."""
+        n = self.cache.slots.n_slots
+        if getattr(self, "_graphs_for_slots", n) != n and self.graphs is not None:
+            self.graphs.clear()
+        self._graphs_for_slots = n
+        return n
+
     def alloc_slot(self) -> int:
         return self.cache.alloc_slot()
 
@@ -147,6 +163,14 @@ class Engine:
 
         self.cache.reserve(slot_ids, new_lens)
         T, B = int(cu[-1]), len(entries)
+        if self.graphs is not None and T == B and rows == list(range(B)) and self.cache.slots.n_slots == self._graph_slots():
+            with torch.cuda.device(self.rt.device):
+                logits = self.graphs.step(ids.astype(np.int32), np.asarray(starts, dtype=np.int32),
+                                          np.asarray(slot_ids, dtype=np.int32), self.cache.step_tables(slot_ids))
+                logits = logits.clone()          # the graph's own buffer is overwritten by its next replay
+            self.cache.commit(slot_ids, new_lens)
+            self.steps_run += 1
+            return logits
         tok_seq = np.repeat(np.arange(B, dtype=np.int32), counts)
         tok_pos = np.concatenate([np.arange(s, s + c, dtype=np.int32) for s, c in zip(starts, counts)])
         tables = self.cache.step_tables(slot_ids)

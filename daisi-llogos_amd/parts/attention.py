@@ -21,6 +21,8 @@ from .rope import Rotary
 
 @register_mixer("attention")
 class Attention(Mixer):
+    graph_safe = True
+
     def __init__(self, prefix: str, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int,
                  position: Rotary, bias: bool = False, qk_norm: bool = False, eps: float = 1e-6,
                  window: int = 0, sinks: int = 0, scale: Optional[float] = None):

@@ -87,7 +87,8 @@ class StepContext:
     starts: List[int]                   # host: position of each sequence's first token in this step
     slot_ids: List[int]                 # host copy of `slots`
     is_decode: bool                     # every sequence brings exactly one token
-    max_context: int                    # largest position + 1 in the step
+    max_context: int                    # largest position + 1 in the step (in a graph: the most it may become)
+    in_graph: bool = False              # the step is being captured for replay: host lists are not valid
     shared: Dict[object, object] = field(default_factory=dict)   # per-step tables shared by layers
 
 
@@ -113,6 +114,10 @@ class Mixer(Part):
 
     def state_spec(self) -> Optional[StateSpec]:
         return None
+
+    # True when forward reads the step only through device tensors (ids, tok_seq, tok_pos, slots,
+    # page tables), so that a captured single-token step can be replayed with new contents.
+    graph_safe = False
 
     def forward(self, ctx: StepContext, h: torch.Tensor, cache: LayerCache) -> torch.Tensor:
         raise NotImplementedError
