@@ -28,8 +28,8 @@ class KVGroup:
         if rt is not None:
             # keys [.., token in page, head size]; values transposed [.., head size, token in page]
             shape = (len(entries), n_pages, spec.n_kv_heads, PAGE_TOKENS, spec.head_dim)
-            self.k = torch.empty(shape, dtype=rt.dtype, device=rt.device)
-            self.v = torch.empty(shape[:3] + (spec.head_dim, PAGE_TOKENS), dtype=rt.dtype, device=rt.device)
+            self.k = torch.zeros(shape, dtype=rt.dtype, device=rt.device)
+            self.v = torch.zeros(shape[:3] + (spec.head_dim, PAGE_TOKENS), dtype=rt.dtype, device=rt.device)
 
     def bytes(self) -> int:
         return 0 if self.k is None else 2 * self.k.numel() * self.k.element_size()

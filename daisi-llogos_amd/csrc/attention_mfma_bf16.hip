@@ -1,0 +1,345 @@
+// bfloat16 attention over the paged cache on the matrix cores (gfx950,
+// v_mfma_f32_16x16x32_bf16), for head sizes 64 and 128 and up to 16 query heads per
+// key/value head.  Softmax statistics, scores and the output sums are float32.
+//
+// One wave works on 16 "columns" and one page of 64 keys at a time:
+//   decode  (one token per sequence): the columns are the query heads of one kv head;
+//           a block of 4 waves takes 4 consecutive pages of one (sequence, kv head), the
+//           waves' running (max, sum, output) are merged through LDS, blocks along the
+//           context write partial results that a second small kernel merges;
+//   prefill (many tokens per sequence): the columns are 16 consecutive tokens of one
+//           sequence for one query head; each wave walks the pages up to its last row.
+// Scores are computed transposed, S^T[key][column] = K . Q^T, so that the lane that holds
+// the scores of a column for 16 keys is the lane that must supply them as the second
+// operand of O^T[d][column] = V^T[d][key] . P^T[key][column]; no shuffle or LDS pass sits
+// between the two products.  Value pages are stored transposed ([head_dim][64 tokens]), so
+// a lane reads eight consecutive tokens of one dimension with one 16-byte load.  The rows
+// of a key page are visited in the order key = 16 * (i / 4) + 4 * rb + i % 4 (i = operand
+// row, rb = block of 16), which makes lane group g own keys 16 g .. 16 g + 15.
+// (reference: gated_attention / batched_gated_attention, Daisi.Llogos.Cuda/kernels/
+//  composite_ops.cu:275-512: tiles of keys with running maximum and sum, kv head = head /
+//  group, scale after the dot, query m of a prompt sees keys 0 .. start + m.)
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kAttnWaves = 4;
+
+__device__ __forceinline__ bf16x8 ld_frag(const bf16_t* p) {
+    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
+}
+
+__device__ __forceinline__ bf16x8 zero_frag() {
+    return __builtin_bit_cast(bf16x8, make_uint4(0, 0, 0, 0));
+}
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+
+// Keeps the first n (0..8) of a fragment's eight values and zeroes the rest.
+__device__ __forceinline__ bf16x8 keep_first(bf16x8 f, int n) {
+    uint4 u = __builtin_bit_cast(uint4, f);
+    uint32_t* w = reinterpret_cast<uint32_t*>(&u);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t mask = (2 * j + 1 < n) ? 0xffffffffu : ((2 * j < n) ? 0x0000ffffu : 0u);
+        w[j] &= mask;
+    }
+    return __builtin_bit_cast(bf16x8, u);
+}
+
+// Running softmax state of one wave: per column (lane & 15) the maximum and the sum, and
+// the output sums O^T[d][column] with d = 16 db + 4 g + r in acc[db][r].
+template <int HD>
+struct WaveState {
+    float m, l;
+    f32x4 acc[HD / 16];
+    __device__ void init() {
+        m = -INFINITY;
+        l = 0.f;
+#pragma unroll
+        for (int db = 0; db < HD / 16; ++db) acc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+};
+
+// One page of 64 keys.  qf: the columns' queries as second operands (lane (c, g) holds
+// Q[c][32 s + 8 g ..]); kpage [64][HD], vpage [HD][64]; q_pos: position of this lane's column
+// (-1: the column is not in use); key0: position of the page's first key; valid_keys: how
+// many of the page's keys have been written (the rest of the page holds whatever was there
+// before: such scores are masked, and such values are zeroed because 0 * NaN is NaN).
+template <int HD>
+__device__ __forceinline__ void attend_page(WaveState<HD>& st, const bf16x8 (&qf)[HD / 32],
+                                            const bf16_t* __restrict__ kpage, const bf16_t* __restrict__ vpage,
+                                            int q_pos, int key0, int valid_keys, float scale, int window, int sinks) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int i = lane & 15, g = lane >> 4;
+    // S^T = K . Q^T, four blocks of 16 keys
+    f32x4 s[4];
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb) {
+        s[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const bf16_t* krow = kpage + (size_t)(16 * (i >> 2) + 4 * rb + (i & 3)) * HD + 8 * g;
+#pragma unroll
+        for (int sk = 0; sk < HD / 32; ++sk)
+            s[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ld_frag(krow + 32 * sk), qf[sk], s[rb], 0, 0, 0);
+    }
+    // this lane: column i, keys key0 + 16 g + 4 rb + r
+    float tile_max = -INFINITY;
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int key = key0 + 16 * g + 4 * rb + r;
+            const bool vis = q_pos >= 0 && key_visible(q_pos, key, window, sinks);
+            const float v = vis ? s[rb][r] * scale : -INFINITY;
+            s[rb][r] = v;
+            tile_max = fmaxf(tile_max, v);
+        }
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+    const float m_new = fmaxf(st.m, tile_max);
+    const bool any = m_new != -INFINITY;
+    const float corr = (st.m == -INFINITY) ? 0.f : expf(st.m - m_new);
+    float p[16];
+    float sum = 0.f;
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float e = (any && s[rb][r] != -INFINITY) ? expf(s[rb][r] - m_new) : 0.f;
+            p[4 * rb + r] = e;
+            sum += e;
+        }
+    sum += __shfl_xor(sum, 16, kWave);
+    sum += __shfl_xor(sum, 32, kWave);
+    st.l = st.l * corr + sum;
+    st.m = m_new;
+    // P^T as second operand: slot (g, e) of step t is key 16 g + 8 t + e
+    bf16x8 pf[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        uint4 u;
+        u.x = pack_bf16(p[8 * t + 0], p[8 * t + 1]);
+        u.y = pack_bf16(p[8 * t + 2], p[8 * t + 3]);
+        u.z = pack_bf16(p[8 * t + 4], p[8 * t + 5]);
+        u.w = pack_bf16(p[8 * t + 6], p[8 * t + 7]);
+        pf[t] = __builtin_bit_cast(bf16x8, u);
+    }
+    // O^T += V^T . P^T
+#pragma unroll
+    for (int db = 0; db < HD / 16; ++db) {
+        const bf16_t* vrow = vpage + (size_t)(16 * db + i) * kPageTokens + 16 * g;
+        f32x4 a = st.acc[db];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) a[r] *= corr;
+        bf16x8 v0 = ld_frag(vrow), v1 = ld_frag(vrow + 8);
+        if (valid_keys < kPageTokens) {
+            v0 = keep_first(v0, valid_keys - 16 * g);
+            v1 = keep_first(v1, valid_keys - 16 * g - 8);
+        }
+        a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v0, pf[0], a, 0, 0, 0);
+        a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v1, pf[1], a, 0, 0, 0);
+        st.acc[db] = a;
+    }
+}
+
+// Whether any key of the page [key0, key0 + 63] can be visible to a query at q_pos.
+__device__ __forceinline__ bool page_may_be_visible(int q_pos, int key0, int window, int sinks) {
+    if (key0 > q_pos) return false;
+    if (window <= 0) return true;
+    return key0 < sinks || key0 + kPageTokens - 1 > q_pos - window;
+}
+
+// ---------------------------------------------------------------- decode
+// grid (batch, kv heads, ceil(table width / 4)); block 4 waves, wave w takes page 4 z + w.
+// partial: [batch][heads][grid.z][HD + 2] floats (max, sum, unnormalised output).
+template <int HD>
+__global__ __launch_bounds__(kAttnWaves * kWave) void attn_decode_kernel(
+        float* __restrict__ partial, const bf16_t* __restrict__ q, int q_stride,
+        const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
+        const int* __restrict__ table, int table_stride, const int* __restrict__ tok_pos,
+        int n_heads, int n_kv_heads, int group, float scale, int window, int sinks) {
+    __shared__ float lds_o[kAttnWaves][16][HD + 1];
+    __shared__ float lds_m[kAttnWaves][16], lds_l[kAttnWaves][16];
+    const int b = blockIdx.x, kvh = blockIdx.y, z = blockIdx.z;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int c = lane & 15, g = lane >> 4;
+    const int pos = tok_pos[b];
+    const int n_pages = pos / kPageTokens + 1;
+    if (z * kAttnWaves >= n_pages) return;                       // nothing of this sequence here
+    const int page_idx = z * kAttnWaves + wave;
+
+    WaveState<HD> st;
+    st.init();
+    if (page_idx < n_pages && page_may_be_visible(pos, page_idx * kPageTokens, window, sinks)) {
+        bf16x8 qf[HD / 32];
+        const bool col_ok = c < group;
+        const bf16_t* qrow = q + (size_t)b * q_stride + (size_t)(kvh * group + (col_ok ? c : 0)) * HD + 8 * g;
+#pragma unroll
+        for (int sk = 0; sk < HD / 32; ++sk) qf[sk] = col_ok ? ld_frag(qrow + 32 * sk) : zero_frag();
+        const int page = table[(size_t)b * table_stride + page_idx];
+        const size_t base = ((size_t)page * n_kv_heads + kvh) * kPageTokens * HD;
+        attend_page<HD>(st, qf, k_pool + base, v_pool + base, col_ok ? pos : -1, page_idx * kPageTokens,
+                        min(kPageTokens, pos - page_idx * kPageTokens + 1), scale, window, sinks);
+    }
+    // merge the four waves
+    if (g == 0) { lds_m[wave][c] = st.m; lds_l[wave][c] = st.l; }
+#pragma unroll
+    for (int db = 0; db < HD / 16; ++db)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) lds_o[wave][c][16 * db + 4 * g + r] = st.acc[db][r];
+    __syncthreads();
+    const int n_z = gridDim.z;
+    for (int idx = threadIdx.x; idx < group * HD; idx += blockDim.x) {
+        const int col = idx / HD, d = idx % HD;
+        float m = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kAttnWaves; ++w) m = fmaxf(m, lds_m[w][col]);
+        float l = 0.f, o = 0.f;
+#pragma unroll
+        for (int w = 0; w < kAttnWaves; ++w) {
+            const float f = (lds_m[w][col] == -INFINITY) ? 0.f : expf(lds_m[w][col] - m);
+            l += lds_l[w][col] * f;
+            o += lds_o[w][col][d] * f;
+        }
+        float* dst = partial + (((size_t)b * n_heads + kvh * group + col) * n_z + z) * (HD + 2);
+        dst[2 + d] = o;
+        if (d == 0) { dst[0] = m; dst[1] = l; }
+    }
+}
+
+// grid (batch, heads); HD threads.  Adds the partial results of the blocks along the context.
+template <int HD>
+__global__ void attn_decode_merge_kernel(bf16_t* __restrict__ out, const float* __restrict__ partial,
+                                         const int* __restrict__ tok_pos, int n_heads, int n_z) {
+    const int b = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
+    const int n_pages = tok_pos[b] / kPageTokens + 1;
+    const int used = min(n_z, (n_pages + kAttnWaves - 1) / kAttnWaves);
+    const float* src = partial + ((size_t)b * n_heads + h) * n_z * (HD + 2);
+    float m = -INFINITY;
+    for (int z = 0; z < used; ++z) m = fmaxf(m, src[(size_t)z * (HD + 2)]);
+    float l = 0.f, o = 0.f;
+    for (int z = 0; z < used; ++z) {
+        const float* p = src + (size_t)z * (HD + 2);
+        const float f = (p[0] == -INFINITY) ? 0.f : expf(p[0] - m);
+        l += p[1] * f;
+        o += p[2 + d] * f;
+    }
+    out[((size_t)b * n_heads + h) * HD + d] = f32_to_bf16(l > 0.f ? o / l : 0.f);
+}
+
+// ---------------------------------------------------------------- prefill
+// grid (tiles of 64 tokens over all sequences, heads); wave w of a block takes rows
+// 16 w .. 16 w + 15 of the tile.  cu: token offsets of the sequences [batch + 1];
+// starts: position of each sequence's first token in this step.
+template <int HD>
+__global__ __launch_bounds__(kAttnWaves * kWave) void attn_prefill_kernel(
+        bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int q_stride,
+        const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
+        const int* __restrict__ table, int table_stride, const int* __restrict__ cu,
+        const int* __restrict__ tok_pos, int batch, int n_heads, int n_kv_heads, int group,
+        float scale, int window, int sinks) {
+    // which sequence does this tile belong to?
+    int tile = blockIdx.x, b = 0, first = 0;
+    for (; b < batch; ++b) {
+        const int len = cu[b + 1] - cu[b];
+        const int tiles = (len + 63) / 64;
+        if (tile < tiles) { first = cu[b] + tile * 64; break; }
+        tile -= tiles;
+    }
+    if (b >= batch) return;
+    const int h = blockIdx.y, kvh = h / group;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int c = lane & 15, g = lane >> 4;
+    const int row0 = first + 16 * wave;                          // this wave's first token row
+    const int seq_end = cu[b + 1];
+    if (row0 >= seq_end) return;
+    const int rows = min(16, seq_end - row0);
+    const bool col_ok = c < rows;
+    const int my_row = row0 + (col_ok ? c : 0);
+    const int q_pos = col_ok ? tok_pos[my_row] : -1;
+    const int last_pos = tok_pos[row0 + rows - 1];
+    const int first_pos = tok_pos[row0];
+    const int written = tok_pos[seq_end - 1] + 1;                // positions of this sequence that hold keys
+
+    bf16x8 qf[HD / 32];
+    const bf16_t* qrow = q + (size_t)my_row * q_stride + (size_t)h * HD + 8 * g;
+#pragma unroll
+    for (int sk = 0; sk < HD / 32; ++sk) qf[sk] = col_ok ? ld_frag(qrow + 32 * sk) : zero_frag();
+
+    WaveState<HD> st;
+    st.init();
+    const int n_pages = last_pos / kPageTokens + 1;
+    for (int pi = 0; pi < n_pages; ++pi) {
+        const int key0 = pi * kPageTokens;
+        // a page is skipped when neither the wave's first nor its last row can see any of it
+        if (!page_may_be_visible(last_pos, key0, window, sinks) && !page_may_be_visible(first_pos, key0, window, sinks))
+            continue;
+        const int page = table[(size_t)b * table_stride + pi];
+        const size_t base = ((size_t)page * n_kv_heads + kvh) * kPageTokens * HD;
+        attend_page<HD>(st, qf, k_pool + base, v_pool + base, q_pos, key0, min(kPageTokens, written - key0),
+                        scale, window, sinks);
+    }
+    if (!col_ok) return;
+    const float inv = st.l > 0.f ? 1.0f / st.l : 0.f;
+    bf16_t* orow = out + ((size_t)my_row * n_heads + h) * HD;
+#pragma unroll
+    for (int db = 0; db < HD / 16; ++db) {
+        uint2 u;
+        u.x = pack_bf16(st.acc[db][0] * inv, st.acc[db][1] * inv);
+        u.y = pack_bf16(st.acc[db][2] * inv, st.acc[db][3] * inv);
+        *reinterpret_cast<uint2*>(orow + 16 * db + 4 * g) = u;
+    }
+}
+
+// ---------------------------------------------------------------- entry points
+static bool mfma_shape_ok(int n_heads, int n_kv_heads, int head_dim) {
+    if (n_kv_heads <= 0 || n_heads % n_kv_heads) return false;
+    return (head_dim == 64 || head_dim == 128) && n_heads / n_kv_heads <= 16;
+}
+
+// floats the decode workspace needs
+LLOGOS_EXPORT long long llogos_attn_decode_workspace(int batch, int n_heads, int head_dim, int table_width) {
+    const int n_z = (table_width + kAttnWaves - 1) / kAttnWaves;
+    return (long long)batch * n_heads * n_z * (head_dim + 2);
+}
+
+LLOGOS_EXPORT int llogos_attn_decode_bf16(void* out, const void* q, int q_stride, const void* k_pool,
+                                          const void* v_pool, const int* table, int table_stride, int table_width,
+                                          const int* tok_pos, int batch, int n_heads, int n_kv_heads, int head_dim,
+                                          float scale, int window, int sinks, float* workspace,
+                                          long long workspace_floats, hipStream_t stream) {
+    if (batch <= 0 || table_width <= 0 || window < 0 || sinks < 0) return LLOGOS_BAD_ARGUMENT;
+    if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || (q_stride % 8) || ((uintptr_t)q % 16)) return LLOGOS_UNSUPPORTED;
+    if (workspace_floats < llogos_attn_decode_workspace(batch, n_heads, head_dim, table_width)) return LLOGOS_BAD_ARGUMENT;
+    const int n_z = (table_width + kAttnWaves - 1) / kAttnWaves;
+    const int group = n_heads / n_kv_heads;
+    dim3 grid(batch, n_kv_heads, n_z), mgrid(batch, n_heads);
+#define GO(HD) \
+    attn_decode_kernel<HD><<<grid, kAttnWaves * kWave, 0, stream>>>( \
+        workspace, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride, \
+        tok_pos, n_heads, n_kv_heads, group, scale, window, sinks); \
+    attn_decode_merge_kernel<HD><<<mgrid, HD, 0, stream>>>((bf16_t*)out, workspace, tok_pos, n_heads, n_z)
+    if (head_dim == 64) { GO(64); } else { GO(128); }
+#undef GO
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+LLOGOS_EXPORT int llogos_attn_prefill_bf16(void* out, const void* q, int q_stride, const void* k_pool,
+                                           const void* v_pool, const int* table, int table_stride,
+                                           const int* cu, const int* tok_pos, int batch, int n_tiles,
+                                           int n_heads, int n_kv_heads, int head_dim,
+                                           float scale, int window, int sinks, hipStream_t stream) {
+    if (batch <= 0 || n_tiles <= 0 || window < 0 || sinks < 0) return LLOGOS_BAD_ARGUMENT;
+    if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || (q_stride % 8) || ((uintptr_t)q % 16)) return LLOGOS_UNSUPPORTED;
+    const int group = n_heads / n_kv_heads;
+    dim3 grid(n_tiles, n_heads);
+#define GO(HD) attn_prefill_kernel<HD><<<grid, kAttnWaves * kWave, 0, stream>>>( \
+        (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride, \
+        cu, tok_pos, batch, n_heads, n_kv_heads, group, scale, window, sinks)
+    if (head_dim == 64) { GO(64); } else { GO(128); }
+#undef GO
+    return LLOGOS_LAUNCH_CHECK();
+}

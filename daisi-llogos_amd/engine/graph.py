@@ -8,6 +8,8 @@ token (Daisi.Llogos.Cuda/CudaBackend.cs:99-141); here nothing is patched: the gr
 what changes from a static buffer that is filled before each replay."""
 from __future__ import annotations
 
+import gc
+import weakref
 from collections import OrderedDict
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -26,7 +28,10 @@ def bucket_width(width: int) -> int:
 
 class DecodeGraph:
     def __init__(self, engine, batch: int, widths: Tuple[int, ...]):
-        self.engine, self.batch, self.widths = engine, batch, widths
+        # no strong reference back to the engine: a graph must die with its engine at once and
+        # not later in a collection of reference cycles, which could fall into another capture
+        self._engine = weakref.ref(engine)
+        self.batch, self.widths = batch, widths
         rt = engine.rt
         B = batch
         self.sizes = [B, B, B, B, B] + [B * w for w in widths]          # ids, seq, pos, slots, rows, tables
@@ -61,7 +66,7 @@ class DecodeGraph:
         self.copied.record()
 
     def _forward(self, max_context: int) -> Optional[torch.Tensor]:
-        eng, v, B = self.engine, self.views, self.batch
+        eng, v, B = self._engine(), self.views, self.batch
         ctx = StepContext(runtime=eng.rt, n_tokens=B, batch=B, ids=v[0], tok_seq=v[1], tok_pos=v[2], slots=v[3],
                           cu_seqlens=list(range(B + 1)), starts=[], slot_ids=[], is_decode=True,
                           max_context=max_context, in_graph=True)
@@ -76,8 +81,16 @@ class DecodeGraph:
             self._forward(cap)                          # warm up: lazy workspaces are made outside the capture
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                self.logits = self._forward(cap)
+            # freeing device memory or another graph is not allowed while a stream captures:
+            # keep the collector of reference cycles out of the capture
+            gc_was_on = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(graph):
+                    self.logits = self._forward(cap)
+            finally:
+                if gc_was_on:
+                    gc.enable()
             self.graph = graph
         self.graph.replay()
         return self.logits
@@ -88,7 +101,7 @@ class GraphCache:
     graph is dropped when there are too many."""
 
     def __init__(self, engine):
-        self.engine = engine
+        self._engine = weakref.ref(engine)
         self.graphs: "OrderedDict[tuple, DecodeGraph]" = OrderedDict()
 
     def clear(self) -> None:
@@ -100,7 +113,7 @@ class GraphCache:
         if g is None:
             while len(self.graphs) >= MAX_GRAPHS:
                 self.graphs.popitem(last=False)
-            g = DecodeGraph(self.engine, key[0], key[1])
+            g = DecodeGraph(self._engine(), key[0], key[1])
             self.graphs[key] = g
         else:
             self.graphs.move_to_end(key)

@@ -175,13 +175,13 @@ class Engine:
         tok_pos = np.concatenate([np.arange(s, s + c, dtype=np.int32) for s, c in zip(starts, counts)])
         tables = self.cache.step_tables(slot_ids)
         parts = [ids.astype(np.int32), tok_seq, tok_pos, np.asarray(slot_ids, dtype=np.int32),
-                 np.asarray(rows, dtype=np.int32)] + [t.reshape(-1) for t in tables]
+                 np.asarray(rows, dtype=np.int32), cu.astype(np.int32)] + [t.reshape(-1) for t in tables]
         dev = self._upload(parts)
         with torch.cuda.device(self.rt.device):
             ctx = StepContext(runtime=self.rt, n_tokens=T, batch=B, ids=dev[0], tok_seq=dev[1], tok_pos=dev[2],
                               slots=dev[3], cu_seqlens=[int(c) for c in cu], starts=starts, slot_ids=slot_ids,
-                              is_decode=max(counts) == 1, max_context=max(new_lens))
-            dev_tables = [d.view(t.shape) for d, t in zip(dev[5:], tables)]
+                              is_decode=max(counts) == 1, max_context=max(new_lens), cu_dev=dev[5])
+            dev_tables = [d.view(t.shape) for d, t in zip(dev[6:], tables)]
             caches = self.cache.layer_caches(dev_tables)
             logits = self.model.forward(ctx, caches, dev[4] if len(rows) else None)
         self.cache.commit(slot_ids, new_lens)

@@ -356,10 +356,67 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dty
     return gemm_generic(a, w, bias, out_dtype)
 
 
+_attn_workspaces = {}
+
+
+def _attn_workspace(device: torch.device, floats: int) -> torch.Tensor:
+    key = (device.type, device.index)
+    ws = _attn_workspaces.get(key)
+    if ws is None or ws.numel() < floats:
+        if torch.cuda.is_current_stream_capturing():
+            raise KernelError("attention workspace must be made before a step is captured")
+        ws = torch.empty(max(floats, 1 << 20), dtype=torch.float32, device=device)
+        _attn_workspaces[key] = ws
+    return ws
+
+
+def attention_mfma_bf16(ctx, q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                        table: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
+                        window: int = 0, sinks: int = 0) -> Optional[torch.Tensor]:
+    """bfloat16 attention on the matrix cores; None for shapes it does not take (head sizes
+    other than 64 and 128, more than 16 query heads per kv head)."""
+    if q.dtype != torch.bfloat16 or head_dim not in (64, 128) or n_heads // n_kv_heads > 16:
+        return None
+    if q_stride % 8 or q.data_ptr() % 16:
+        return None
+    _dev(k_pool, v_pool, table)
+    _i32(table, "table")
+    _check_pools(k_pool, v_pool, n_kv_heads, head_dim, "attention")
+    _need(k_pool.dtype == torch.bfloat16, "attention: q and cache types differ")
+    T = ctx.n_tokens
+    _need(q.numel() >= (T - 1) * q_stride + n_heads * head_dim, "attention: q too small")
+    out = torch.empty((T, n_heads * head_dim), dtype=torch.bfloat16, device=q.device)
+    lib = _lib()
+    if ctx.is_decode:
+        width = table.shape[1]
+        floats = lib.llogos_attn_decode_workspace(T, n_heads, head_dim, width)
+        ws = _attn_workspace(q.device, floats)
+        code = lib.llogos_attn_decode_bf16(
+            _p(out), _p(q), q_stride, _p(k_pool), _p(v_pool), _p(table), table.stride(0), width, _p(ctx.tok_pos),
+            T, n_heads, n_kv_heads, head_dim, ctypes.c_float(scale), window, sinks, _p(ws),
+            ctypes.c_longlong(ws.numel()), _stream())
+    else:
+        cu = ctx.cu_dev
+        _need(cu is not None and cu.numel() == ctx.batch + 1, "attention: the step's token offsets are missing")
+        n_tiles = sum(-(-(ctx.cu_seqlens[i + 1] - ctx.cu_seqlens[i]) // 64) for i in range(ctx.batch))
+        code = lib.llogos_attn_prefill_bf16(
+            _p(out), _p(q), q_stride, _p(k_pool), _p(v_pool), _p(table), table.stride(0), _p(cu), _p(ctx.tok_pos),
+            ctx.batch, n_tiles, n_heads, n_kv_heads, head_dim, ctypes.c_float(scale), window, sinks, _stream())
+    if code == -2:
+        return None
+    _check(code, "attention_mfma_bf16")
+    return out
+
+
 def attention(ctx, q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
               table: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
               window: int = 0, sinks: int = 0) -> torch.Tensor:
     """Attention of the step's query rows over the cache pages of their sequences."""
+    if q.dtype == torch.bfloat16:
+        out = attention_mfma_bf16(ctx, q, q_stride, k_pool, v_pool, table, n_heads, n_kv_heads, head_dim, scale,
+                                  window, sinks)
+        if out is not None:
+            return out
     return attention_generic(q, q_stride, k_pool, v_pool, table, ctx.tok_seq, ctx.tok_pos,
                              n_heads, n_kv_heads, head_dim, scale, window, sinks)
 

@@ -88,6 +88,7 @@ class StepContext:
     slot_ids: List[int]                 # host copy of `slots`
     is_decode: bool                     # every sequence brings exactly one token
     max_context: int                    # largest position + 1 in the step (in a graph: the most it may become)
+    cu_dev: Optional[torch.Tensor] = None   # int32 [B + 1] token offsets on the device (None in a captured step)
     in_graph: bool = False              # the step is being captured for replay: host lists are not valid
     shared: Dict[object, object] = field(default_factory=dict)   # per-step tables shared by layers
 

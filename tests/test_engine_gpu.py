@@ -11,7 +11,7 @@ import plain_model as pm
 import tiny_configs as tc
 
 pytestmark = pytest.mark.gpu
-CONFIGS = ["tiny_a", "tiny_b", "tiny_c", "tiny_w"]
+CONFIGS = ["tiny_a", "tiny_b", "tiny_c", "tiny_w", "tiny_d"]
 
 
 def _np(t):
@@ -121,7 +121,7 @@ def test_batch_composition_and_slot_do_not_change_float_results(dtype):
 
 
 @pytest.mark.parametrize("dtype", H.DTYPES)
-@pytest.mark.parametrize("name", ["tiny_c", "tiny_w"])
+@pytest.mark.parametrize("name", ["tiny_c", "tiny_w", "tiny_d"])
 def test_long_decoding(name, dtype):
     """300 positions, most of them decoded one by one: crosses page borders, and in the
     windowed configuration pages leave the window and are given back meanwhile."""
@@ -152,9 +152,9 @@ def test_first_tokens(name, dtype):
     H.close(got, want[[5, 2]], dtype, f"{name} wanted places")
 
 
+@pytest.mark.parametrize("name", ["tiny_a", "tiny_d"])
 @pytest.mark.parametrize("dtype", H.DTYPES)
-def test_window_and_sinks_as_run_time_strategy(dtype):
-    name = "tiny_a"
+def test_window_and_sinks_as_run_time_strategy(name, dtype):
     cfg, w = H.plain(name)
     toks = H.tokens(name, 100, 17)
     want = pm.forward(cfg, w, list(toks), window=24, sinks=3)

@@ -222,6 +222,7 @@ def test_attention_whole_prompts_and_single_tokens(dtype, nh, nkv, hd):
         ctx = type("Ctx", (), dict(tok_seq=_t(c["tok_seq"], torch.int32), tok_pos=_t(c["tok_pos"], torch.int32),
                                    is_decode=max(new) == 1, max_context=max(lens), batch=len(lens),
                                    n_tokens=sum(new), cu_seqlens=np.concatenate([[0], np.cumsum(new)]).tolist(),
+                                   cu_dev=_t(np.concatenate([[0], np.cumsum(new)]), torch.int32),
                                    starts=[l - n for l, n in zip(lens, new)], shared={}))()
         out = K.attention(ctx, c["q"], c["stride"], c["kp"], c["vp"], c["table"], nh, nkv, hd, 1 / math.sqrt(hd))
         _close(out, _plain_attention(c, nh, nkv, hd), dtype)
@@ -239,7 +240,7 @@ def test_attention_finds_a_far_key_among_hundreds(dtype):
     c["kp"][page, :, off, :] = key.to(c["kp"].dtype)
     q[0, :nh * hd] = (key.repeat(nh) * 2).to(q.dtype)                   # score 40 * 80 / 8 = 400 for that key
     ctx = type("Ctx", (), dict(tok_seq=_t(c["tok_seq"], torch.int32), tok_pos=_t(c["tok_pos"], torch.int32),
-                               is_decode=True, max_context=L, batch=1, n_tokens=1, cu_seqlens=[0, 1],
+                               is_decode=True, max_context=L, batch=1, n_tokens=1, cu_seqlens=[0, 1], cu_dev=None,
                                starts=[L - 1], shared={}))()
     out = _np(K.attention(ctx, q, c["stride"], c["kp"], c["vp"], c["table"], nh, nkv, hd, 1 / math.sqrt(hd)))
     want = np.concatenate([c["vs"][0][far].reshape(nkv, hd)[h // 2] for h in range(nh)])
@@ -247,9 +248,10 @@ def test_attention_finds_a_far_key_among_hundreds(dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("hd", [32, 64, 128])
 @pytest.mark.parametrize("window,sinks", [(64, 0), (70, 0), (5, 2), (128, 64), (1, 0)])
-def test_attention_window_edges(dtype, window, sinks):
-    nh, nkv, hd = 4, 2, 32
+def test_attention_window_edges(dtype, window, sinks, hd):
+    nh, nkv = 4, 2
     for lens, new in (([300, 66], [1, 1]), ([200, 10], [200, 10]), ([257], [100])):
         c = _attention_case(dtype, nh, nkv, hd, lens, new, seed=9)
         # keys just outside and just inside the window stand out, so an off-by-one shows
@@ -262,6 +264,7 @@ def test_attention_window_edges(dtype, window, sinks):
         ctx = type("Ctx", (), dict(tok_seq=_t(c["tok_seq"], torch.int32), tok_pos=_t(c["tok_pos"], torch.int32),
                                    is_decode=max(new) == 1, max_context=max(lens), batch=len(lens),
                                    n_tokens=sum(new), cu_seqlens=np.concatenate([[0], np.cumsum(new)]).tolist(),
+                                   cu_dev=_t(np.concatenate([[0], np.cumsum(new)]), torch.int32),
                                    starts=[l - n for l, n in zip(lens, new)], shared={}))()
         out = K.attention(ctx, c["q"], c["stride"], c["kp"], c["vp"], c["table"], nh, nkv, hd, 1 / math.sqrt(hd),
                           window, sinks)

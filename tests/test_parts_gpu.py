@@ -41,7 +41,8 @@ def _ctx(rt, lens, new, slots=None):
                          tok_pos=i32(tok_pos), slots=i32(slots or list(range(B))),
                          cu_seqlens=np.concatenate([[0], np.cumsum(new)]).tolist(),
                          starts=[l - n for l, n in zip(lens, new)], slot_ids=slots or list(range(B)),
-                         is_decode=max(new) == 1, max_context=max(lens))
+                         is_decode=max(new) == 1, max_context=max(lens),
+                         cu_dev=i32(np.concatenate([[0], np.cumsum(new)])))
 
 
 @pytest.mark.parametrize("dtype", H.DTYPES)

@@ -33,4 +33,11 @@ TINY_W = {   # Qwen2 style with a sliding window in the upper layers
     "tie_word_embeddings": False, "torch_dtype": "bfloat16", "eos_token_id": 199,
 }
 
-ALL = {"tiny_a": TINY_A, "tiny_b": TINY_B, "tiny_c": TINY_C, "tiny_w": TINY_W}
+TINY_D = {   # Llama style with head size 64 and window: the matrix-core attention path
+    "architectures": ["LlamaForCausalLM"], "vocab_size": 300, "hidden_size": 120, "intermediate_size": 200,
+    "num_hidden_layers": 2, "num_attention_heads": 6, "num_key_value_heads": 2, "head_dim": 64,
+    "rms_norm_eps": 1e-5, "rope_theta": 10000.0, "max_position_embeddings": 512,
+    "tie_word_embeddings": False, "torch_dtype": "bfloat16", "eos_token_id": 1,
+}
+
+ALL = {"tiny_a": TINY_A, "tiny_b": TINY_B, "tiny_c": TINY_C, "tiny_w": TINY_W, "tiny_d": TINY_D}
