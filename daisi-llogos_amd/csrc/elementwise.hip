@@ -73,6 +73,74 @@ __global__ void rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ x, cons
     }
 }
 
+// The same with the row held in registers: each thread owns ITEMS groups of 4 consecutive
+// values, all loads (the row and every part of delta) are issued before the first sum, and
+// the row is read from memory once.  For H % 4 == 0 and H <= 4 * ITEMS * blockDim.
+__device__ __forceinline__ float4 load4_f32(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 load4_f32(const bf16_t* p) {
+    const uint2 u = *reinterpret_cast<const uint2*>(p);
+    return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u),
+                       __uint_as_float(u.y << 16), __uint_as_float(u.y & 0xffff0000u));
+}
+__device__ __forceinline__ void store4_f32(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void store4_f32(bf16_t* p, float4 v) {
+    uint2 u;
+    u.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
+    u.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
+    *reinterpret_cast<uint2*>(p) = u;
+}
+
+constexpr int kMaxNormParts = 8;
+
+template <typename TO, typename TD, int ITEMS>
+__global__ void rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ x, const TD* __restrict__ delta,
+                                   int parts, size_t part_stride,
+                                   const int* __restrict__ rows, const float* __restrict__ w,
+                                   float eps, int H, int write_back) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const size_t s = rows ? (size_t)rows[r] : (size_t)r;
+    float* xr = x + s * H;
+    const TD* dr = delta ? delta + s * H : nullptr;
+    float4 v[ITEMS], wv[ITEMS];
+    float4 dv[ITEMS][kMaxNormParts];
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+        const int i = 4 * (it * blockDim.x + threadIdx.x);
+        const bool ok = i < H;
+        v[it] = ok ? load4_f32(xr + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+        wv[it] = ok ? load4_f32(w + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int q = 0; q < kMaxNormParts; ++q)
+            dv[it][q] = (ok && dr && q < parts) ? load4_f32(dr + q * part_stride + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+        if (dr) {
+            float4 d = dv[it][0];
+#pragma unroll
+            for (int q = 1; q < kMaxNormParts; ++q) {       // ascending order, as sum_parts
+                d.x += dv[it][q].x; d.y += dv[it][q].y; d.z += dv[it][q].z; d.w += dv[it][q].w;
+            }
+            v[it].x += d.x; v[it].y += d.y; v[it].z += d.z; v[it].w += d.w;
+            const int i = 4 * (it * blockDim.x + threadIdx.x);
+            if (write_back && i < H) store4_f32(xr + i, v[it]);
+        }
+        ss += v[it].x * v[it].x + v[it].y * v[it].y + v[it].z * v[it].z + v[it].w * v[it].w;
+    }
+    const float total = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(total / (float)H + eps);
+    TO* o = out + (size_t)r * H;
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+        const int i = 4 * (it * blockDim.x + threadIdx.x);
+        if (i < H)
+            store4_f32(o + i, make_float4(v[it].x * inv * wv[it].x, v[it].y * inv * wv[it].y,
+                                          v[it].z * inv * wv[it].z, v[it].w * inv * wv[it].w));
+    }
+}
+
 // delta: `parts` partial products [parts][T][H] (part_stride elements apart) that are summed
 // on the way; parts = 1 for a plain delta.
 LLOGOS_EXPORT int llogos_rmsnorm(void* out, int out_dtype, float* x, const void* delta, int delta_dtype,
@@ -80,6 +148,25 @@ LLOGOS_EXPORT int llogos_rmsnorm(void* out, int out_dtype, float* x, const void*
                                  const int* rows, const float* w, float eps, int R, int H,
                                  int write_back, hipStream_t stream) {
     if (R <= 0 || H <= 0 || parts < 1) return LLOGOS_BAD_ARGUMENT;
+    const bool aligned = (H % 4 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0) &&
+                         ((uintptr_t)out % 16 == 0) && (!delta || ((uintptr_t)delta % 16 == 0 && part_stride % 4 == 0));
+    if (aligned && parts <= kMaxNormParts && H <= 4 * 4 * 1024) {
+        const int groups = H / 4;
+        const int items = groups <= 1024 ? 1 : (groups <= 2048 ? 2 : 4);
+        int threads = (groups + items - 1) / items;
+        threads = (threads + kWave - 1) / kWave * kWave;
+#define LAUNCHV(TO, TD, IT) rmsnorm_vec_kernel<TO, TD, IT><<<R, threads, 0, stream>>>( \
+        (TO*)out, x, (const TD*)delta, parts, (size_t)part_stride, rows, w, eps, H, write_back)
+#define PICK(TO, TD) do { if (items == 1) LAUNCHV(TO, TD, 1); else if (items == 2) LAUNCHV(TO, TD, 2); else LAUNCHV(TO, TD, 4); } while (0)
+        if (out_dtype == DT_F32 && delta_dtype == DT_F32) PICK(float, float);
+        else if (out_dtype == DT_BF16 && delta_dtype == DT_BF16) PICK(bf16_t, bf16_t);
+        else if (out_dtype == DT_BF16 && delta_dtype == DT_F32) PICK(bf16_t, float);
+        else if (out_dtype == DT_F32 && delta_dtype == DT_BF16) PICK(float, bf16_t);
+        else return LLOGOS_BAD_ARGUMENT;
+#undef PICK
+#undef LAUNCHV
+        return LLOGOS_LAUNCH_CHECK();
+    }
     const int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
 #define LAUNCH(TO, TD) rmsnorm_kernel<TO, TD><<<R, threads, 0, stream>>>( \
         (TO*)out, x, (const TD*)delta, parts, (size_t)part_stride, rows, w, eps, H, write_back)

@@ -60,8 +60,10 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny_kernel(
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) acc[rb][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    for (int k = k_begin; k < k_end; k += kStepK * U) {
-        bf16x8 wf[U][RB], af[U][MB];
+    // two register buffers of U steps each: the loads of the next U steps are in flight while
+    // the matrix cores work on the current ones
+    bf16x8 wf0[U][RB], af0[U][MB], wf1[U][RB], af1[U][MB];
+    auto load = [&](bf16x8 (&wf)[U][RB], bf16x8 (&af)[U][MB], int k) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int kk = k + u * kStepK;
@@ -71,6 +73,8 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny_kernel(
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) af[u][mb] = load_frag(arow[mb] + kk, ok && a_ok[mb]);
         }
+    };
+    auto multiply = [&](const bf16x8 (&wf)[U][RB], const bf16x8 (&af)[U][MB]) {
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -78,6 +82,15 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny_kernel(
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb)
                     acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][rb], af[u][mb], acc[rb][mb], 0, 0, 0);
+    };
+    constexpr int kChunk = kStepK * U;
+    if (k_begin < k_end) load(wf0, af0, k_begin);
+    for (int k = k_begin; k < k_end; k += 2 * kChunk) {
+        const bool second = k + kChunk < k_end;
+        if (second) load(wf1, af1, k + kChunk);
+        multiply(wf0, af0);
+        if (k + 2 * kChunk < k_end) load(wf0, af0, k + 2 * kChunk);
+        if (second) multiply(wf1, af1);
     }
 
     // acc[rb][mb][i] = sum for row n0 + rb * 16 + 4 g + i of w and activation row mb * 16 + r
@@ -153,17 +166,17 @@ LLOGOS_EXPORT int llogos_gemm_skinny_bf16(void* out, int out_dtype, const void* 
 #define GO(RB, MB, U) return launch_skinny<RB, MB, U>(out, out_dtype, A, W, bias, M, N, K, lda, ldo, \
                                                       (size_t)part_stride, kpb, parts, stream)
     if (mb == 1) {
-        if (row_blocks >= 4) GO(4, 1, 4);
-        if (row_blocks == 2) GO(2, 1, 8);
-        GO(1, 1, 8);
+        if (row_blocks >= 4) GO(4, 1, 2);
+        if (row_blocks == 2) GO(2, 1, 4);
+        GO(1, 1, 4);
     } else if (mb == 2) {
         if (row_blocks >= 4) GO(4, 2, 2);
-        if (row_blocks == 2) GO(2, 2, 4);
+        if (row_blocks == 2) GO(2, 2, 2);
         GO(1, 2, 4);
     } else {
-        if (row_blocks >= 4) GO(4, 4, 2);
+        if (row_blocks >= 4) GO(4, 4, 1);
         if (row_blocks == 2) GO(2, 4, 2);
-        GO(1, 4, 4);
+        GO(1, 4, 2);
     }
 #undef GO
 }

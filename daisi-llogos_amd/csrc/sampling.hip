@@ -17,9 +17,24 @@ __global__ __launch_bounds__(kSampleThreads) void argmax_kernel(int* __restrict_
     const float* row = logits + (size_t)blockIdx.x * V;
     float best = -INFINITY;
     int best_i = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += blockDim.x) {
-        const float v = row[i];
-        if (v > best || best_i == 0x7fffffff) { best = v; best_i = i; }
+    if ((V & 3) == 0 && ((uintptr_t)row & 15) == 0) {
+        // four values per load, several loads in flight; a thread visits its indices in
+        // ascending order, so the strict comparison keeps the first maximum
+        const float4* row4 = reinterpret_cast<const float4*>(row);
+        const int n4 = V >> 2;
+#pragma unroll 4
+        for (int i = threadIdx.x; i < n4; i += blockDim.x) {
+            const float4 v = row4[i];
+            const float e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (e[j] > best || best_i == 0x7fffffff) { best = e[j]; best_i = 4 * i + j; }
+        }
+    } else {
+        for (int i = threadIdx.x; i < V; i += blockDim.x) {
+            const float v = row[i];
+            if (v > best || best_i == 0x7fffffff) { best = v; best_i = i; }
+        }
     }
 #pragma unroll
     for (int o = kWave / 2; o > 0; o >>= 1) {
