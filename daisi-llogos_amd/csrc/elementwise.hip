@@ -152,7 +152,10 @@ LLOGOS_EXPORT int llogos_rmsnorm(void* out, int out_dtype, float* x, const void*
                          ((uintptr_t)out % 16 == 0) && (!delta || ((uintptr_t)delta % 16 == 0 && part_stride % 4 == 0));
     if (aligned && parts <= kMaxNormParts && H <= 4 * 4 * 1024) {
         const int groups = H / 4;
-        const int items = groups <= 1024 ? 1 : (groups <= 2048 ? 2 : 4);
+        // few rows: one group per thread, so that the row's loads are all in flight at once;
+        // many rows: four groups per thread, fewer and fuller waves
+        int items = groups <= 1024 ? 1 : (groups <= 2048 ? 2 : 4);
+        if (R >= 256 && groups >= 256) items = 4;
         int threads = (groups + items - 1) / items;
         threads = (threads + kWave - 1) / kWave * kWave;
 #define LAUNCHV(TO, TD, IT) rmsnorm_vec_kernel<TO, TD, IT><<<R, threads, 0, stream>>>( \
@@ -297,6 +300,53 @@ __global__ void qk_rope_cache_kernel(const TI* __restrict__ qkv, int parts, size
     }
 }
 
+// The same for head_dim = rot = 128 with split-half pairing, without LDS or block barriers:
+// lane l of a wave holds dimensions 2 l and 2 l + 1 of its head, and the rotation partner
+// (64 dimensions away) sits in lane l ^ 32.
+template <typename TI, typename T>
+__global__ void qk_rope_cache_hd128_kernel(const TI* __restrict__ qkv, int parts, size_t part_stride, int row_stride,
+                                           const float* __restrict__ bias, T* __restrict__ q_out,
+                                           int n_heads, int n_kv_heads,
+                                           const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w,
+                                           float eps, const float2* __restrict__ cs,
+                                           T* __restrict__ k_pool, T* __restrict__ v_pool, PagedKV cache,
+                                           const int* __restrict__ tok_seq, const int* __restrict__ tok_pos) {
+    constexpr int HD = 128;
+    const int t = blockIdx.x;
+    const int head = blockIdx.y * kHeadsPerBlock + threadIdx.y;
+    const int lane = threadIdx.x;
+    if (head >= n_heads + 2 * n_kv_heads) return;
+    const int d = 2 * lane;
+    const size_t col = (size_t)head * HD + d;
+    const TI* src = qkv + (size_t)t * row_stride + col;
+    float x0 = sum_parts(src, 0, parts, part_stride), x1 = sum_parts(src, 1, parts, part_stride);
+    if (bias) { x0 += bias[col]; x1 += bias[col + 1]; }
+    const bool is_q = head < n_heads;
+    const bool is_k = !is_q && head < n_heads + n_kv_heads;
+    if (!is_q && !is_k) {
+        T* vdst = v_pool + paged_v_offset(cache, tok_seq[t], head - n_heads - n_kv_heads, tok_pos[t]);
+        store_f32(vdst + (size_t)d * kPageTokens, x0);
+        store_f32(vdst + (size_t)(d + 1) * kPageTokens, x1);
+        return;
+    }
+    const float* norm_w = is_q ? q_norm_w : k_norm_w;
+    if (norm_w) {
+        const float ss = wave_sum(x0 * x0 + x1 * x1);
+        const float inv = 1.0f / sqrtf(ss / (float)HD + eps);
+        x0 = x0 * inv * norm_w[d];
+        x1 = x1 * inv * norm_w[d + 1];
+    }
+    const float p0 = __shfl_xor(x0, 32, kWave), p1 = __shfl_xor(x1, 32, kWave);
+    const float2 c0 = cs[(size_t)t * 64 + (d & 63)], c1 = cs[(size_t)t * 64 + (d & 63) + 1];
+    float y0, y1;
+    if (lane < 32) { y0 = x0 * c0.x - p0 * c0.y; y1 = x1 * c1.x - p1 * c1.y; }
+    else           { y0 = p0 * c0.y + x0 * c0.x; y1 = p1 * c1.y + x1 * c1.x; }
+    T* dst = is_q ? q_out + ((size_t)t * n_heads + head) * HD
+                  : k_pool + paged_offset(cache, tok_seq[t], head - n_heads, tok_pos[t]);
+    store_f32(dst + d, y0);
+    store_f32(dst + d + 1, y1);
+}
+
 // qkv: the fused projection [parts][T][row_stride] in float32 or in the cache's type (parts are
 // summed, then `bias` [width] is added); q_out [T, n_heads * head_dim] and the pools have the
 // cache's type `dtype`.
@@ -315,9 +365,16 @@ LLOGOS_EXPORT int llogos_qk_rope_cache(const void* qkv, int in_dtype, int parts,
     const int total_heads = n_heads + 2 * n_kv_heads;
     dim3 grid(T, (total_heads + kHeadsPerBlock - 1) / kHeadsPerBlock), block(kWave, kHeadsPerBlock);
     const size_t smem = (size_t)kHeadsPerBlock * head_dim * sizeof(float);
-#define LAUNCH(TI, T_) qk_rope_cache_kernel<TI, T_><<<grid, block, smem, stream>>>( \
-        (const TI*)qkv, parts, (size_t)part_stride, row_stride, bias, (T_*)q_out, n_heads, n_kv_heads, head_dim, \
-        rot, pairing, q_norm_w, k_norm_w, eps, (const float2*)cs, (T_*)k_pool, (T_*)v_pool, cache, tok_seq, tok_pos)
+#define LAUNCH(TI, T_) do { \
+        if (head_dim == 128 && rot == 128 && pairing == 0) \
+            qk_rope_cache_hd128_kernel<TI, T_><<<grid, block, 0, stream>>>( \
+                (const TI*)qkv, parts, (size_t)part_stride, row_stride, bias, (T_*)q_out, n_heads, n_kv_heads, \
+                q_norm_w, k_norm_w, eps, (const float2*)cs, (T_*)k_pool, (T_*)v_pool, cache, tok_seq, tok_pos); \
+        else \
+            qk_rope_cache_kernel<TI, T_><<<grid, block, smem, stream>>>( \
+                (const TI*)qkv, parts, (size_t)part_stride, row_stride, bias, (T_*)q_out, n_heads, n_kv_heads, head_dim, \
+                rot, pairing, q_norm_w, k_norm_w, eps, (const float2*)cs, (T_*)k_pool, (T_*)v_pool, cache, tok_seq, tok_pos); \
+    } while (0)
     if (dtype == DT_F32 && in_dtype == DT_F32) LAUNCH(float, float);
     else if (dtype == DT_BF16 && in_dtype == DT_BF16) LAUNCH(bf16_t, bf16_t);
     else if (dtype == DT_BF16 && in_dtype == DT_F32) LAUNCH(float, bf16_t);
@@ -341,11 +398,38 @@ __global__ void swiglu_kernel(T* __restrict__ out, const TI* __restrict__ gu, in
     store_f32(out + idx, g / (1.0f + expf(-g)) * u);
 }
 
+// the same for one bfloat16 part and I % 8 == 0: eight values per thread, 16-byte loads and stores
+__global__ void swiglu_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ gu, int I, size_t n8) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n8) return;
+    const int per_row = I / 8;
+    const size_t t = idx / per_row;
+    const int i = (int)(idx % per_row) * 8;
+    const uint4 gv = *reinterpret_cast<const uint4*>(gu + t * 2 * I + i);
+    const uint4 uv = *reinterpret_cast<const uint4*>(gu + t * 2 * I + I + i);
+    const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
+        const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
+        o[j] = (uint32_t)f32_to_bf16(g0 / (1.0f + expf(-g0)) * u0) |
+               ((uint32_t)f32_to_bf16(g1 / (1.0f + expf(-g1)) * u1) << 16);
+    }
+    *reinterpret_cast<uint4*>(out + t * I + i) = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
 // gu: [parts][T][2 I] in float32 or in the output's type; parts are summed on the way.
 LLOGOS_EXPORT int llogos_swiglu(void* out, int dtype, const void* gu, int in_dtype, int parts,
                                 long long part_stride, int T, int I, hipStream_t stream) {
     if (T <= 0 || I <= 0 || parts < 1) return LLOGOS_BAD_ARGUMENT;
     const size_t n = (size_t)T * I;
+    if (dtype == DT_BF16 && in_dtype == DT_BF16 && parts == 1 && I % 8 == 0 &&
+        (uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0) {
+        const size_t n8 = n / 8;
+        swiglu_bf16x8_kernel<<<(unsigned)((n8 + 255) / 256), 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, I, n8);
+        return LLOGOS_LAUNCH_CHECK();
+    }
     const unsigned blocks = (unsigned)((n + 255) / 256);
 #define LAUNCH(TI, T_) swiglu_kernel<TI, T_><<<blocks, 256, 0, stream>>>( \
         (T_*)out, (const TI*)gu, parts, (size_t)part_stride, I, n)

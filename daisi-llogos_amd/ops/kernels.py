@@ -266,19 +266,19 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
 SKINNY_MAX_ROWS = 64
 
 
-def skinny_plan(M: int, N: int, K: int) -> Tuple[int, int]:
-    """(blocks along k, 16-row blocks of w per wave) for the few-row product.  The split of k
-    depends on N and K alone, so the order of a row's additions does not depend on how many
-    other rows the batch has; wider strips with more rows re-read the activations less."""
-    strips = -(-N // 16)
-    splits = max(1, min(-(-1024 // strips), K // 1024, 8))
-    if M <= 8:
-        row_blocks = 4 if N >= 65536 and M > 4 else 1
-    elif M <= 16:
-        row_blocks = 4 if N >= 16384 else 2
-    else:
-        row_blocks = 4
-    return splits, row_blocks
+def skinny_plan(M: int, N: int, K: int) -> Tuple[str, int, int]:
+    """(kernel, blocks along k, 16-row blocks of w per wave) for the few-row product.
+    'regs': every wave fetches its own activation fragments; best for up to 4 rows and many
+    rows of w.  'lds': the block shares the activations through LDS; its speed hardly depends
+    on the number of rows.  The split of k depends on N and K alone within a kernel, so the
+    order of a row's additions does not depend on how many other rows the batch has."""
+    if M <= 4 and N >= 16384:
+        strips = -(-N // 16)
+        return "regs", max(1, min(-(-1024 // strips), K // 1024, 8)), 1
+    blocks = -(-N // 64)
+    if blocks >= 256:
+        return "lds", 1, 1
+    return "lds", max(1, min(-(-512 // blocks), K // 512, 8)), 1
 
 
 def gemm_skinny_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype,
@@ -311,22 +311,82 @@ def gemm_skinny_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tens
     return out
 
 
-def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+def gemm_skinny_lds_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype,
+                         splits: int = 1, row_blocks: int = 1, swiglu: bool = False) -> Optional[torch.Tensor]:
+    """The few-row bfloat16 product with the activations shared through LDS: [parts, M, N].
+    With `swiglu`, `a` is the fused gate/up product ([M, 2 K] bfloat16 or float32 partial sums
+    [parts, M, 2 K]) and silu(gate) * up is made on the way.  None for shapes it does not take."""
+    if swiglu:
+        a_parts, a_stride = _parts(a)
+        M, K2 = a.shape[-2:]
+        K = K2 // 2
+        if a.dtype == torch.float32:
+            mode = 1
+        elif a.dtype == torch.bfloat16 and a_parts == 1:
+            mode = 2
+        else:
+            return None
+        lda = a.stride(-2)
+    else:
+        if a.dtype != torch.bfloat16 or a.dim() != 2:
+            return None
+        a_parts, a_stride, mode = 1, 0, 0
+        M, K = a.shape
+        lda = a.stride(0)
+    N = w.shape[0]
+    if not (w.dtype == torch.bfloat16 and 0 < M <= SKINNY_MAX_ROWS and K % 8 == 0 and a.stride(-1) == 1
+            and lda % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and w.is_contiguous()
+            and a_stride % 4 == 0):
+        return None
+    _dev(w, bias)
+    _need(w.dim() == 2 and w.shape[1] == K, f"gemm: w must be [N, {K}], got {tuple(w.shape)}")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.shape == (N,), "gemm: bias must be float32 [N]")
+    lib = _lib()
+    parts = lib.llogos_gemm_skinny_lds_parts(K, int(splits))
+    if parts > 1:
+        _need(bias is None, "gemm: a product in parts leaves the bias to its consumer")
+        out_dtype = torch.float32
+    out = torch.empty((parts, M, N), dtype=out_dtype, device=a.device)
+    code = lib.llogos_gemm_skinny_lds_bf16(
+        _p(out), _DT[out_dtype], _p(a), mode, lda, a_parts, ctypes.c_longlong(a_stride), _p(w), _p(bias),
+        M, N, K, N, ctypes.c_longlong(M * N), int(splits), int(row_blocks), _stream())
+    if code == -2:
+        return None
+    _check(code, "gemm_skinny_lds_bf16")
+    return out
+
+
+def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swiglu_input: bool = False) -> torch.Tensor:
     """a [M, K] . w [N, K]^T without bias, as [M, N] of `out_dtype` or as float32 partial sums
     [parts, M, N] for a consumer that adds them (rmsnorm, qk_rope_cache, swiglu, sum_parts).
+    With `swiglu_input`, `a` is a fused gate/up product ([M, 2 K] or parts of it) and the
+    product is taken of silu(gate) * up.
 
     float32 operands: plain FMAs in 32-bit throughout.  bfloat16 operands: up to 64 rows the
-    hand-written weight-streaming kernel; more rows the library product (as the reference
+    hand-written weight-streaming kernels; more rows the library product (as the reference
     uses a library for its prompt products, Daisi.Llogos.Cuda/CudaBackend.cs:158-316)."""
-    if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
-        M = a.shape[0]
-        if M <= SKINNY_MAX_ROWS:
-            splits, row_blocks = skinny_plan(M, w.shape[0], w.shape[1])
-            out = gemm_skinny_bf16(a, w, None, out_dtype, splits, row_blocks)
+    M = a.shape[-2]
+    if w.dtype == torch.bfloat16 and M <= SKINNY_MAX_ROWS and out_dtype == torch.bfloat16:
+        kernel, splits, row_blocks = skinny_plan(M, w.shape[0], w.shape[1])
+        # silu(gate) * up inside the product costs every block of rows of w a second read of the
+        # gate/up row: worth it for few rows in bfloat16, not for partial sums or many rows
+        if swiglu_input and not (M <= 16 and a.dtype == torch.bfloat16 and (a.dim() == 2 or a.shape[0] == 1)):
+            a, swiglu_input = swiglu(a, out_dtype), False
+        if swiglu_input or kernel == "lds":
+            out = gemm_skinny_lds_bf16(a, w, None, out_dtype, splits if kernel == "lds" else 1, row_blocks,
+                                       swiglu_input)
             if out is not None:
                 return out
-        elif out_dtype == torch.bfloat16 and a.is_contiguous():
-            return torch.matmul(a, w.t())
+        if not swiglu_input and a.dtype == torch.bfloat16:
+            out = gemm_skinny_bf16(a, w, None, out_dtype, splits if kernel == "regs" else 1, row_blocks)
+            if out is not None:
+                return out
+    if swiglu_input:
+        a = swiglu(a, out_dtype)
+    if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out_dtype == torch.bfloat16 and a.is_contiguous() \
+            and M > SKINNY_MAX_ROWS:
+        return torch.matmul(a, w.t())
     return gemm_generic(a, w, None, out_dtype)
 
 
@@ -335,8 +395,9 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dty
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
         M = a.shape[0]
         if M <= SKINNY_MAX_ROWS:
-            _, row_blocks = skinny_plan(M, w.shape[0], w.shape[1])
-            out = gemm_skinny_bf16(a, w, bias, out_dtype, 1, row_blocks)
+            kernel, _, row_blocks = skinny_plan(M, w.shape[0], w.shape[1])
+            fn = gemm_skinny_lds_bf16 if kernel == "lds" else gemm_skinny_bf16
+            out = fn(a, w, bias, out_dtype, 1, row_blocks)
             if out is not None:
                 return out[0]
         elif out_dtype == torch.bfloat16 and a.is_contiguous():
@@ -348,7 +409,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dty
             # float32 results for many rows: row blocks through the hand-written kernel
             out = torch.empty((M, w.shape[0]), dtype=torch.float32, device=a.device)
             for r in range(0, M, SKINNY_MAX_ROWS):
-                blk = gemm_skinny_bf16(a[r:r + SKINNY_MAX_ROWS], w, bias, torch.float32, 1, 4)
+                blk = gemm_skinny_lds_bf16(a[r:r + SKINNY_MAX_ROWS], w, bias, torch.float32, 1, 1)
                 if blk is None:
                     return gemm_generic(a, w, bias, out_dtype)
                 out[r:r + SKINNY_MAX_ROWS] = blk[0]

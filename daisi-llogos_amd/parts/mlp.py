@@ -7,7 +7,6 @@ from typing import Callable, List, Optional
 
 import torch
 
-from ..ops import kernels as K
 from .base import FeedForward, Runtime, StepContext, TensorSpec, register_feed_forward
 from .linear import Linear
 
@@ -30,4 +29,6 @@ class SwiGLU(FeedForward):
 
     def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
         gu = self.gate_up.product(h)
-        return self.down.product(K.swiglu(gu, self.rt.dtype))      # the residual sum that follows adds the parts
+        # silu(gate) * up is made inside the down product where its kernel can (few rows), by a
+        # kernel of its own otherwise; the residual sum that follows adds the product's parts
+        return self.down.product(gu, swiglu_input=True)

@@ -93,11 +93,22 @@ def test_gemm_few_rows_on_the_matrix_cores(M, N, K_):
     b = _t(rng.standard_normal(N))
     want = pm.linear(_np(a), _np(w))
     scale = np.abs(want).max()
-    for splits in (1, 2, 5, 8):
-        for rb in (1, 2, 4):
-            out = K.gemm_skinny_bf16(a, w, None, torch.float32, splits, rb)
-            assert out is not None and out.dtype == torch.float32 and out.shape[1:] == (M, N)
-            assert np.abs(_np(out).sum(0) - want).max() <= 2e-6 * scale * math.sqrt(K_)
+    for kernel, rbs in ((K.gemm_skinny_bf16, (1, 2, 4)), (K.gemm_skinny_lds_bf16, (1, 2))):
+        for splits in (1, 2, 5, 8):
+            for rb in rbs:
+                out = kernel(a, w, None, torch.float32, splits, rb)
+                assert out is not None and out.dtype == torch.float32 and out.shape[1:] == (M, N)
+                assert np.abs(_np(out).sum(0) - want).max() <= 2e-6 * scale * math.sqrt(K_)
+    # silu(gate) * up made inside the product, from a bfloat16 row or from float32 partial sums
+    if K_ % 16 == 0:
+        I = K_ // 2
+        act = pm.silu(_np(a)[:, :I]) * _np(a)[:, I:]
+        act = _np(_t(act, torch.bfloat16))                              # the kernel rounds it to bfloat16
+        want_sw = pm.linear(act, _np(w)[:, :I])
+        w_half = w[:, :I].contiguous()
+        for src in (a, torch.stack([a.float() * 0.25, a.float() * 0.75])):
+            out = K.gemm_skinny_lds_bf16(src, w_half, None, torch.float32, 2, 1, swiglu=True)
+            assert np.abs(_np(out).sum(0) - want_sw).max() <= 2e-2 * max(1.0, np.abs(want_sw).max())
     plain = K.gemm(a, w, b, torch.bfloat16)
     assert np.abs(_np(plain) - (want + _np(b))).max() <= 1e-2 * scale
     prod = K.gemm_product(a, w, torch.bfloat16)
@@ -128,7 +139,7 @@ def _pages(n_seqs, max_len, rng):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("nh,nkv,hd,rot,pairing,norm", [
     (4, 2, 16, 16, 0, False), (6, 1, 32, 32, 0, True), (5, 5, 48, 24, 0, True), (8, 2, 80, 80, 1, False),
-    (3, 3, 128, 64, 1, True), (2, 1, 256, 256, 0, False)])
+    (3, 3, 128, 64, 1, True), (2, 1, 256, 256, 0, False), (8, 2, 128, 128, 0, True), (5, 5, 128, 128, 0, False)])
 def test_qk_rope_cache(dtype, nh, nkv, hd, rot, pairing, norm):
     rng = np.random.default_rng(3)
     lens = [70, 3]                                      # two sequences; this step brings the last 5 and 3 tokens
