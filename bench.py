@@ -61,6 +61,7 @@ def main(argv=None) -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration has (0 = all)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    ap.add_argument("--only-prefill", action="store_true", help="time the 2,048-token prompt alone (for profiling)")
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU library")
@@ -75,7 +76,7 @@ def main(argv=None) -> int:
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
-    max_batch = max(args.batch, 1 if args.no_points else 64)
+    max_batch = max(args.batch, 1 if (args.no_points or args.only_prefill) else 64)
     per_seq = PROMPT + args.steps + args.warmup + 64
     t0 = time.time()
     eng = llogos.Engine.from_config(cfg, seed=0, dtype="bfloat16",
@@ -106,6 +107,19 @@ def main(argv=None) -> int:
         for s in slots:
             eng.free_slot(s)
         return dt, ctx_mid
+
+    if args.only_prefill:
+        prompt = rng.integers(0, cfg["vocab_size"], size=PREFILL_TOKENS).tolist()
+        for it in range(4):
+            s = eng.alloc_slot()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            eng.step([(s, prompt)], want="last")
+            torch.cuda.synchronize()
+            print(f"[bench] prefill {PREFILL_TOKENS} tokens, {cfg['num_hidden_layers']} layers: "
+                  f"{(time.perf_counter() - t) * 1e3:.2f} ms", file=sys.stderr, flush=True)
+            eng.free_slot(s)
+        return 0
 
     dt, ctx_mid = decode_run(args.batch, args.steps, args.warmup)
     ms_per_step = dt / args.steps * 1e3
