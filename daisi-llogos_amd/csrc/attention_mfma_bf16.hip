@@ -152,6 +152,15 @@ __device__ __forceinline__ bool page_may_be_visible(int q_pos, int key0, int win
     return key0 < sinks || key0 + kPageTokens - 1 > q_pos - window;
 }
 
+// The same for queries at positions first_pos .. last_pos: the causal bound is loosest for the
+// last of them, the window's for the first.
+__device__ __forceinline__ bool page_may_be_visible_to_range(int first_pos, int last_pos, int key0,
+                                                             int window, int sinks) {
+    if (key0 > last_pos) return false;
+    if (window <= 0) return true;
+    return key0 < sinks || key0 + kPageTokens - 1 > first_pos - window;
+}
+
 // ---------------------------------------------------------------- decode
 // grid (batch, kv heads, ceil(table width / 4)); block 4 waves, wave w takes page 4 z + w.
 // partial: [batch][heads][grid.z][HD + 2] floats (max, sum, unnormalised output).
@@ -274,9 +283,7 @@ __global__ __launch_bounds__(kAttnWaves * kWave) void attn_prefill_kernel(
     const int n_pages = last_pos / kPageTokens + 1;
     for (int pi = 0; pi < n_pages; ++pi) {
         const int key0 = pi * kPageTokens;
-        // a page is skipped when neither the wave's first nor its last row can see any of it
-        if (!page_may_be_visible(last_pos, key0, window, sinks) && !page_may_be_visible(first_pos, key0, window, sinks))
-            continue;
+        if (!page_may_be_visible_to_range(first_pos, last_pos, key0, window, sinks)) continue;
         const int page = table[(size_t)b * table_stride + pi];
         const size_t base = ((size_t)page * n_kv_heads + kvh) * kPageTokens * HD;
         attend_page<HD>(st, qf, k_pool + base, v_pool + base, q_pos, key0, min(kPageTokens, written - key0),
@@ -291,6 +298,215 @@ __global__ __launch_bounds__(kAttnWaves * kWave) void attn_prefill_kernel(
         u.x = pack_bf16(st.acc[db][0] * inv, st.acc[db][1] * inv);
         u.y = pack_bf16(st.acc[db][2] * inv, st.acc[db][3] * inv);
         *reinterpret_cast<uint2*>(orow + 16 * db + 4 * g) = u;
+    }
+}
+
+// ---------------------------------------------------------------- prefill, pages shared through LDS
+// grid (tiles of 128 tokens over all sequences, heads); the 4 waves of a block take 32 rows
+// each (two blocks of 16 columns) and walk the same pages: a page's keys and transposed
+// values are copied to LDS once per block (two buffers, the copy of the next page is in
+// flight while the current one is used), and every key fragment a wave reads serves both of
+// its column blocks.  Keys are visited in natural order here (operand row i of block rb is key
+// 16 rb + i, conflict-free in LDS with rows padded by 16 bytes), so lane group g owns keys
+// 16 rb + 4 g .. + 3 of each block, and the value operand of a step of 32 keys is two runs of
+// four tokens.
+constexpr int kTileRows = 128;
+constexpr int kKPad = 8, kVPad = 8;
+
+template <int HD>
+struct PageLds {
+    bf16_t k[kPageTokens][HD + kKPad];
+    bf16_t v[HD][kPageTokens + kVPad];
+};
+
+template <int HD>
+__global__ __launch_bounds__(kAttnWaves * kWave) void attn_prefill_lds_kernel(
+        bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int q_stride,
+        const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
+        const int* __restrict__ table, int table_stride, const int* __restrict__ cu,
+        const int* __restrict__ tok_pos, int batch, int n_heads, int n_kv_heads, int group,
+        float scale, int window, int sinks) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    PageLds<HD>* lds = reinterpret_cast<PageLds<HD>*>(smem_raw);      // two buffers
+    int tile = blockIdx.x, b = 0, first = 0;
+    for (; b < batch; ++b) {
+        const int len = cu[b + 1] - cu[b];
+        const int tiles = (len + kTileRows - 1) / kTileRows;
+        if (tile < tiles) { first = cu[b] + tile * kTileRows; break; }
+        tile -= tiles;
+    }
+    if (b >= batch) return;
+    const int h = blockIdx.y, kvh = h / group;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int c = lane & 15, g = lane >> 4;
+    const int seq_end = cu[b + 1];
+    const int tile_rows = min(kTileRows, seq_end - first);
+    const int tile_last_pos = tok_pos[first + tile_rows - 1];
+    const int tile_first_pos = tok_pos[first];
+    const int written = tok_pos[seq_end - 1] + 1;
+    // this wave: rows first + 32 wave .. + 31, column block cb holds rows + 16 cb
+    const int row0 = first + 32 * wave;
+    const int wave_rows = max(0, min(32, seq_end - row0));
+    int q_pos[2];
+    bf16x8 qf[2][HD / 32];
+    WaveState<HD> st[2];
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb) {
+        const int rr = 16 * cb + c;
+        const bool ok = rr < wave_rows;
+        q_pos[cb] = ok ? tok_pos[row0 + rr] : -1;
+        const bf16_t* qrow = q + (size_t)(row0 + (ok ? rr : 0)) * q_stride + (size_t)h * HD + 8 * g;
+#pragma unroll
+        for (int sk = 0; sk < HD / 32; ++sk) qf[cb][sk] = ok ? ld_frag(qrow + 32 * sk) : zero_frag();
+        st[cb].init();
+    }
+    const int wave_first_pos = wave_rows > 0 ? tok_pos[row0] : 0;
+    const int wave_last_pos = wave_rows > 0 ? tok_pos[row0 + wave_rows - 1] : -1;
+
+    // the pages the tile needs, in order
+    const int n_pages = tile_last_pos / kPageTokens + 1;
+    auto page_needed = [&](int pi) {
+        return page_may_be_visible_to_range(tile_first_pos, tile_last_pos, pi * kPageTokens, window, sinks);
+    };
+    constexpr int kPieces = kPageTokens * HD / 8;                         // 16-byte pieces of a page (keys or values)
+    constexpr int kPerThread = kPieces / (kAttnWaves * kWave);
+    uint4 kreg[kPerThread], vreg[kPerThread];
+    auto fetch = [&](int pi) {
+        const int page = table[(size_t)b * table_stride + pi];
+        const size_t base = ((size_t)page * n_kv_heads + kvh) * kPageTokens * HD;
+#pragma unroll
+        for (int i = 0; i < kPerThread; ++i) {
+            const int piece = i * (kAttnWaves * kWave) + threadIdx.x;
+            kreg[i] = *reinterpret_cast<const uint4*>(k_pool + base + (size_t)piece * 8);
+            vreg[i] = *reinterpret_cast<const uint4*>(v_pool + base + (size_t)piece * 8);
+        }
+    };
+    auto stash = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < kPerThread; ++i) {
+            const int piece = i * (kAttnWaves * kWave) + threadIdx.x;
+            *reinterpret_cast<uint4*>(&lds[buf].k[piece / (HD / 8)][(piece % (HD / 8)) * 8]) = kreg[i];
+            *reinterpret_cast<uint4*>(&lds[buf].v[piece / (kPageTokens / 8)][(piece % (kPageTokens / 8)) * 8]) = vreg[i];
+        }
+    };
+    auto compute = [&](int pi, int buf) {
+        const int key0 = pi * kPageTokens;
+        if (wave_rows <= 0 || key0 > wave_last_pos) return;               // nothing of this page for this wave
+        if (!page_may_be_visible_to_range(wave_first_pos, wave_last_pos, key0, window, sinks)) return;
+        const int valid_keys = min(kPageTokens, written - key0);
+        const PageLds<HD>& pg = lds[buf];
+        // S^T for both column blocks; operand row c of block rb is key 16 rb + c
+        f32x4 s[2][4];
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb) {
+            s[0][rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+            s[1][rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int sk = 0; sk < HD / 32; ++sk) {
+                const bf16x8 kf = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&pg.k[16 * rb + c][32 * sk + 8 * g]));
+                s[0][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[0][sk], s[0][rb], 0, 0, 0);
+                s[1][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[1][sk], s[1][rb], 0, 0, 0);
+            }
+        }
+        // lane (c, g) of block cb: column c, keys key0 + 16 rb + 4 g + r
+        bf16x8 pf[2][2];
+        float corr[2];
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb) {
+            float tile_max = -INFINITY;
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int key = key0 + 16 * rb + 4 * g + r;
+                    const bool vis = q_pos[cb] >= 0 && key_visible(q_pos[cb], key, window, sinks);
+                    const float v = vis ? s[cb][rb][r] * scale : -INFINITY;
+                    s[cb][rb][r] = v;
+                    tile_max = fmaxf(tile_max, v);
+                }
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
+            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+            const float m_new = fmaxf(st[cb].m, tile_max);
+            const bool any = m_new != -INFINITY;
+            corr[cb] = (st[cb].m == -INFINITY) ? 0.f : expf(st[cb].m - m_new);
+            float p[16], sum = 0.f;
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float e = (any && s[cb][rb][r] != -INFINITY) ? expf(s[cb][rb][r] - m_new) : 0.f;
+                    p[4 * rb + r] = e;
+                    sum += e;
+                }
+            sum += __shfl_xor(sum, 16, kWave);
+            sum += __shfl_xor(sum, 32, kWave);
+            st[cb].l = st[cb].l * corr[cb] + sum;
+            st[cb].m = m_new;
+            // step t covers blocks 2 t and 2 t + 1: slots 0..3 keys 32 t + 4 g + e, slots 4..7 keys 32 t + 16 + 4 g + e
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                uint4 u;
+                u.x = pack_bf16(p[8 * t + 0], p[8 * t + 1]);
+                u.y = pack_bf16(p[8 * t + 2], p[8 * t + 3]);
+                u.z = pack_bf16(p[8 * t + 4], p[8 * t + 5]);
+                u.w = pack_bf16(p[8 * t + 6], p[8 * t + 7]);
+                pf[cb][t] = __builtin_bit_cast(bf16x8, u);
+            }
+        }
+#pragma unroll
+        for (int db = 0; db < HD / 16; ++db) {
+            f32x4 a0 = st[0].acc[db], a1 = st[1].acc[db];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) { a0[r] *= corr[0]; a1[r] *= corr[1]; }
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const bf16_t* vrow = &pg.v[16 * db + c][32 * t + 4 * g];
+                uint2 lo = *reinterpret_cast<const uint2*>(vrow), hi = *reinterpret_cast<const uint2*>(vrow + 16);
+                if (valid_keys < kPageTokens) {                           // zero the tokens that were never written
+                    const int n_lo = valid_keys - (32 * t + 4 * g), n_hi = n_lo - 16;
+                    lo.x &= (1 < n_lo) ? 0xffffffffu : ((0 < n_lo) ? 0x0000ffffu : 0u);
+                    lo.y &= (3 < n_lo) ? 0xffffffffu : ((2 < n_lo) ? 0x0000ffffu : 0u);
+                    hi.x &= (1 < n_hi) ? 0xffffffffu : ((0 < n_hi) ? 0x0000ffffu : 0u);
+                    hi.y &= (3 < n_hi) ? 0xffffffffu : ((2 < n_hi) ? 0x0000ffffu : 0u);
+                }
+                const bf16x8 vf = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
+                a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[0][t], a0, 0, 0, 0);
+                a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[1][t], a1, 0, 0, 0);
+            }
+            st[0].acc[db] = a0;
+            st[1].acc[db] = a1;
+        }
+    };
+
+    // walk the needed pages with one page of look-ahead
+    int cur = 0;
+    while (cur < n_pages && !page_needed(cur)) ++cur;
+    if (cur < n_pages) { fetch(cur); stash(0); }
+    __syncthreads();
+    int buf = 0;
+    while (cur < n_pages) {
+        int nxt = cur + 1;
+        while (nxt < n_pages && !page_needed(nxt)) ++nxt;
+        if (nxt < n_pages) fetch(nxt);
+        compute(cur, buf);
+        if (nxt < n_pages) stash(buf ^ 1);
+        __syncthreads();
+        cur = nxt;
+        buf ^= 1;
+    }
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb) {
+        const int rr = 16 * cb + c;
+        if (rr >= wave_rows) continue;
+        const float inv = st[cb].l > 0.f ? 1.0f / st[cb].l : 0.f;
+        bf16_t* orow = out + ((size_t)(row0 + rr) * n_heads + h) * HD;
+#pragma unroll
+        for (int db = 0; db < HD / 16; ++db) {
+            uint2 u;
+            u.x = pack_bf16(st[cb].acc[db][0] * inv, st[cb].acc[db][1] * inv);
+            u.y = pack_bf16(st[cb].acc[db][2] * inv, st[cb].acc[db][3] * inv);
+            *reinterpret_cast<uint2*>(orow + 16 * db + 4 * g) = u;
+        }
     }
 }
 
@@ -327,15 +543,31 @@ LLOGOS_EXPORT int llogos_attn_decode_bf16(void* out, const void* q, int q_stride
     return LLOGOS_LAUNCH_CHECK();
 }
 
+// tile_rows: 64 for the kernel whose waves read pages from global memory, 128 for the kernel
+// that shares pages through LDS (n_tiles counts tiles of that many tokens per sequence).
 LLOGOS_EXPORT int llogos_attn_prefill_bf16(void* out, const void* q, int q_stride, const void* k_pool,
                                            const void* v_pool, const int* table, int table_stride,
-                                           const int* cu, const int* tok_pos, int batch, int n_tiles,
+                                           const int* cu, const int* tok_pos, int batch, int n_tiles, int tile_rows,
                                            int n_heads, int n_kv_heads, int head_dim,
                                            float scale, int window, int sinks, hipStream_t stream) {
     if (batch <= 0 || n_tiles <= 0 || window < 0 || sinks < 0) return LLOGOS_BAD_ARGUMENT;
+    if (tile_rows != 64 && tile_rows != kTileRows) return LLOGOS_BAD_ARGUMENT;
     if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || (q_stride % 8) || ((uintptr_t)q % 16)) return LLOGOS_UNSUPPORTED;
     const int group = n_heads / n_kv_heads;
     dim3 grid(n_tiles, n_heads);
+    if (tile_rows == kTileRows) {
+#define GOL(HD) do { \
+        const size_t smem = 2 * sizeof(PageLds<HD>); \
+        hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<HD>, \
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
+        if (e != hipSuccess) return (int)e; \
+        attn_prefill_lds_kernel<HD><<<grid, kAttnWaves * kWave, smem, stream>>>( \
+            (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride, \
+            cu, tok_pos, batch, n_heads, n_kv_heads, group, scale, window, sinks); } while (0)
+        if (head_dim == 64) GOL(64); else GOL(128);
+#undef GOL
+        return LLOGOS_LAUNCH_CHECK();
+    }
 #define GO(HD) attn_prefill_kernel<HD><<<grid, kAttnWaves * kWave, 0, stream>>>( \
         (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride, \
         cu, tok_pos, batch, n_heads, n_kv_heads, group, scale, window, sinks)

@@ -418,6 +418,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dty
 
 
 _attn_workspaces = {}
+PREFILL_TILE_ROWS = 0        # 0: chosen by the step; 64 or 128 force a prefill attention kernel (tests)
 
 
 def _attn_workspace(device: torch.device, floats: int) -> torch.Tensor:
@@ -459,10 +460,15 @@ def attention_mfma_bf16(ctx, q: torch.Tensor, q_stride: int, k_pool: torch.Tenso
     else:
         cu = ctx.cu_dev
         _need(cu is not None and cu.numel() == ctx.batch + 1, "attention: the step's token offsets are missing")
-        n_tiles = sum(-(-(ctx.cu_seqlens[i + 1] - ctx.cu_seqlens[i]) // 64) for i in range(ctx.batch))
+        # long sequences: tiles of 128 tokens whose waves share each page through LDS; short
+        # ones: tiles of 64 whose waves read the pages themselves
+        lens = [ctx.cu_seqlens[i + 1] - ctx.cu_seqlens[i] for i in range(ctx.batch)]
+        tile_rows = PREFILL_TILE_ROWS or (128 if max(lens) > 64 else 64)
+        n_tiles = sum(-(-n // tile_rows) for n in lens)
         code = lib.llogos_attn_prefill_bf16(
             _p(out), _p(q), q_stride, _p(k_pool), _p(v_pool), _p(table), table.stride(0), _p(cu), _p(ctx.tok_pos),
-            ctx.batch, n_tiles, n_heads, n_kv_heads, head_dim, ctypes.c_float(scale), window, sinks, _stream())
+            ctx.batch, n_tiles, tile_rows, n_heads, n_kv_heads, head_dim, ctypes.c_float(scale), window, sinks,
+            _stream())
     if code == -2:
         return None
     _check(code, "attention_mfma_bf16")

@@ -239,6 +239,35 @@ def test_attention_whole_prompts_and_single_tokens(dtype, nh, nkv, hd):
         _close(out, _plain_attention(c, nh, nkv, hd), dtype)
 
 
+@pytest.mark.parametrize("tile_rows", [64, 128])
+@pytest.mark.parametrize("nh,nkv,hd", [(6, 2, 64), (8, 2, 128), (3, 3, 128)])
+@pytest.mark.parametrize("window,sinks", [(0, 0), (100, 0), (70, 5)])
+def test_prompt_attention_on_the_matrix_cores(tile_rows, nh, nkv, hd, window, sinks):
+    """Both prompt kernels (pages read by each wave; pages shared through LDS) on long and
+    short sequences, whole and continued, with pages half written."""
+    K.PREFILL_TILE_ROWS = tile_rows
+    try:
+        for lens, new in (([300, 129, 5, 64], [300, 129, 5, 64]), ([400, 90, 257], [200, 33, 129])):
+            c = _attention_case("bfloat16", nh, nkv, hd, lens, new, seed=11)
+            ctx = type("Ctx", (), dict(tok_seq=_t(c["tok_seq"], torch.int32), tok_pos=_t(c["tok_pos"], torch.int32),
+                                       is_decode=False, max_context=max(lens), batch=len(lens), n_tokens=sum(new),
+                                       cu_seqlens=np.concatenate([[0], np.cumsum(new)]).tolist(),
+                                       cu_dev=_t(np.concatenate([[0], np.cumsum(new)]), torch.int32),
+                                       starts=[l - n for l, n in zip(lens, new)], shared={}))()
+            # what lies behind the written part of a page must not matter: poison it
+            for b, l in enumerate(lens):
+                if l % 64:
+                    page = int(c["table"][b, l // 64])
+                    c["kp"][page, :, l % 64:, :] = float("nan")
+                    c["vp"][page, :, :, l % 64:] = float("nan")
+            out = K.attention_mfma_bf16(ctx, c["q"], c["stride"], c["kp"], c["vp"], c["table"], nh, nkv, hd,
+                                        1 / math.sqrt(hd), window, sinks)
+            assert out is not None
+            _close(out, _plain_attention(c, nh, nkv, hd, window, sinks), "bfloat16")
+    finally:
+        K.PREFILL_TILE_ROWS = 0
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_attention_finds_a_far_key_among_hundreds(dtype):
     """One early key matches the query strongly; the output must be its value."""
