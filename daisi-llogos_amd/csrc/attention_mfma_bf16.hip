@@ -34,9 +34,16 @@ __device__ __forceinline__ bf16x8 zero_frag() {
     return __builtin_bit_cast(bf16x8, make_uint4(0, 0, 0, 0));
 }
 
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+// two floats to packed bfloat16, round to nearest even (one v_cvt_pk_bf16_f32)
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-    return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
+
+constexpr float kLog2e = 1.4426950408889634f;
 
 // Keeps the first n (0..8) of a fragment's eight values and zeroes the rest.
 __device__ __forceinline__ bf16x8 keep_first(bf16x8 f, int n) {
@@ -51,7 +58,9 @@ __device__ __forceinline__ bf16x8 keep_first(bf16x8 f, int n) {
 }
 
 // Running softmax state of one wave: per column (lane & 15) the maximum and the sum, and
-// the output sums O^T[d][column] with d = 16 db + 4 g + r in acc[db][r].
+// the output sums O^T[d][column] with d = 16 db + 4 g + r in acc[db][r].  The maximum is kept
+// in units of log2: m = max(score * scale) * log2(e), so that exp(x - max) is one
+// multiply-add and one v_exp_f32.
 template <int HD>
 struct WaveState {
     float m, l;
@@ -64,51 +73,38 @@ struct WaveState {
     }
 };
 
-// One page of 64 keys.  qf: the columns' queries as second operands (lane (c, g) holds
-// Q[c][32 s + 8 g ..]); kpage [64][HD], vpage [HD][64]; q_pos: position of this lane's column
-// (-1: the column is not in use); key0: position of the page's first key; valid_keys: how
-// many of the page's keys have been written (the rest of the page holds whatever was there
-// before: such scores are masked, and such values are zeroed because 0 * NaN is NaN).
-template <int HD>
-__device__ __forceinline__ void attend_page(WaveState<HD>& st, const bf16x8 (&qf)[HD / 32],
-                                            const bf16_t* __restrict__ kpage, const bf16_t* __restrict__ vpage,
-                                            int q_pos, int key0, int valid_keys, float scale, int window, int sinks) {
-    const int lane = threadIdx.x & (kWave - 1);
-    const int i = lane & 15, g = lane >> 4;
-    // S^T = K . Q^T, four blocks of 16 keys
-    f32x4 s[4];
-#pragma unroll
-    for (int rb = 0; rb < 4; ++rb) {
-        s[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
-        const bf16_t* krow = kpage + (size_t)(16 * (i >> 2) + 4 * rb + (i & 3)) * HD + 8 * g;
-#pragma unroll
-        for (int sk = 0; sk < HD / 32; ++sk)
-            s[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ld_frag(krow + 32 * sk), qf[sk], s[rb], 0, 0, 0);
-    }
-    // this lane: column i, keys key0 + 16 g + 4 rb + r
+// Softmax of one page for one block of 16 columns.  s[rb][r]: raw dot products of this lane's
+// column with key key0 + g * GS + rb * RS + r.  Returns the probabilities as the two second
+// operands of O^T += V^T . P^T (step t, slot e <-> s[2 t + e / 4][e % 4]) and the factor by
+// which the running sums shrink.  MASKED = false when every key of the page is visible to
+// every column of the wave.
+template <bool MASKED, int GS, int RS, int HD>
+__device__ __forceinline__ void softmax_page(f32x4 (&s)[4], WaveState<HD>& st, float scale_log2, int q_pos,
+                                             int key0, int window, int sinks, bf16x8 (&pf)[2], float& corr) {
+    const int g = (threadIdx.x & (kWave - 1)) >> 4;
     float tile_max = -INFINITY;
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int key = key0 + 16 * g + 4 * rb + r;
-            const bool vis = q_pos >= 0 && key_visible(q_pos, key, window, sinks);
-            const float v = vis ? s[rb][r] * scale : -INFINITY;
-            s[rb][r] = v;
-            tile_max = fmaxf(tile_max, v);
+            if (MASKED) {
+                const int key = key0 + g * GS + rb * RS + r;
+                if (!(q_pos >= 0 && key_visible(q_pos, key, window, sinks))) s[rb][r] = -INFINITY;
+            }
+            tile_max = fmaxf(tile_max, s[rb][r]);
         }
     tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
     tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
-    const float m_new = fmaxf(st.m, tile_max);
-    const bool any = m_new != -INFINITY;
-    const float corr = (st.m == -INFINITY) ? 0.f : expf(st.m - m_new);
-    float p[16];
-    float sum = 0.f;
+    const float m_new = fmaxf(st.m, tile_max * scale_log2);              // scale > 0: the maximum commutes
+    // a column that has seen no key yet keeps m = -inf; exp2(-inf - (-inf)) must not be taken
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    corr = __builtin_amdgcn_exp2f(st.m - m_use);                          // exp2(-inf) = 0 for the first page
+    float p[16], sum = 0.f;
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const float e = (any && s[rb][r] != -INFINITY) ? expf(s[rb][r] - m_new) : 0.f;
+            const float e = __builtin_amdgcn_exp2f(fmaf(s[rb][r], scale_log2, -m_use));   // masked: exp2(-inf) = 0
             p[4 * rb + r] = e;
             sum += e;
         }
@@ -116,8 +112,6 @@ __device__ __forceinline__ void attend_page(WaveState<HD>& st, const bf16x8 (&qf
     sum += __shfl_xor(sum, 32, kWave);
     st.l = st.l * corr + sum;
     st.m = m_new;
-    // P^T as second operand: slot (g, e) of step t is key 16 g + 8 t + e
-    bf16x8 pf[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
         uint4 u;
@@ -127,14 +121,64 @@ __device__ __forceinline__ void attend_page(WaveState<HD>& st, const bf16x8 (&qf
         u.w = pack_bf16(p[8 * t + 6], p[8 * t + 7]);
         pf[t] = __builtin_bit_cast(bf16x8, u);
     }
-    // O^T += V^T . P^T
+}
+
+// Whether every key of the page [key0, key0 + 63] is visible to every query at first_pos .. last_pos.
+__device__ __forceinline__ bool page_fully_visible(int first_pos, int last_pos, int key0, int window, int sinks) {
+    if (key0 + kPageTokens - 1 > first_pos) return false;
+    if (window <= 0) return true;
+    return key0 + kPageTokens - 1 < sinks || key0 > last_pos - window;
+}
+
+// One page of 64 keys.  qf: the columns' queries as second operands (lane (c, g) holds
+// Q[c][32 s + 8 g ..]); kpage [64][HD], vpage [HD][64]; q_pos: position of this lane's column
+// (-1: the column is not in use); key0: position of the page's first key; valid_keys: how
+// many of the page's keys have been written (the rest of the page holds whatever was there
+// before: such scores are masked, and such values are zeroed because 0 * NaN is NaN).
+template <int HD>
+__device__ __forceinline__ void attend_page(WaveState<HD>& st, const bf16x8 (&qf)[HD / 32],
+                                            const bf16_t* __restrict__ kpage, const bf16_t* __restrict__ vpage,
+                                            int q_pos, int key0, int valid_keys, bool all_visible,
+                                            float scale_log2, int window, int sinks) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int i = lane & 15, g = lane >> 4;
+    // all of the page's loads are issued before the first product
+    bf16x8 kf[4][HD / 32], vf[HD / 16][2];
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb) {
+        const bf16_t* krow = kpage + (size_t)(16 * (i >> 2) + 4 * rb + (i & 3)) * HD + 8 * g;
+#pragma unroll
+        for (int sk = 0; sk < HD / 32; ++sk) kf[rb][sk] = ld_frag(krow + 32 * sk);
+    }
 #pragma unroll
     for (int db = 0; db < HD / 16; ++db) {
         const bf16_t* vrow = vpage + (size_t)(16 * db + i) * kPageTokens + 16 * g;
-        f32x4 a = st.acc[db];
+        vf[db][0] = ld_frag(vrow);
+        vf[db][1] = ld_frag(vrow + 8);
+    }
+    // S^T = K . Q^T, four blocks of 16 keys; this lane: column i, keys key0 + 16 g + 4 rb + r
+    f32x4 s[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) a[r] *= corr;
-        bf16x8 v0 = ld_frag(vrow), v1 = ld_frag(vrow + 8);
+    for (int rb = 0; rb < 4; ++rb) {
+        s[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int sk = 0; sk < HD / 32; ++sk)
+            s[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[rb][sk], qf[sk], s[rb], 0, 0, 0);
+    }
+    bf16x8 pf[2];
+    float corr;
+    if (all_visible) softmax_page<false, 16, 4, HD>(s, st, scale_log2, q_pos, key0, window, sinks, pf, corr);
+    else             softmax_page<true, 16, 4, HD>(s, st, scale_log2, q_pos, key0, window, sinks, pf, corr);
+    // O^T = O^T * corr + V^T . P^T; slot (g, e) of step t is key 16 g + 8 t + e
+    const bool rescale = __ballot(corr != 1.0f) != 0;
+#pragma unroll
+    for (int db = 0; db < HD / 16; ++db) {
+        f32x4 a = st.acc[db];
+        if (rescale) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) a[r] *= corr;
+        }
+        bf16x8 v0 = vf[db][0], v1 = vf[db][1];
         if (valid_keys < kPageTokens) {
             v0 = keep_first(v0, valid_keys - 16 * g);
             v1 = keep_first(v1, valid_keys - 16 * g - 8);
@@ -190,8 +234,11 @@ __global__ __launch_bounds__(kAttnWaves * kWave) void attn_decode_kernel(
         for (int sk = 0; sk < HD / 32; ++sk) qf[sk] = col_ok ? ld_frag(qrow + 32 * sk) : zero_frag();
         const int page = table[(size_t)b * table_stride + page_idx];
         const size_t base = ((size_t)page * n_kv_heads + kvh) * kPageTokens * HD;
-        attend_page<HD>(st, qf, k_pool + base, v_pool + base, col_ok ? pos : -1, page_idx * kPageTokens,
-                        min(kPageTokens, pos - page_idx * kPageTokens + 1), scale, window, sinks);
+        const int key0 = page_idx * kPageTokens;
+        // unused columns (c >= group) have zero queries and are never stored: they may run unmasked
+        attend_page<HD>(st, qf, k_pool + base, v_pool + base, col_ok ? pos : -1, key0,
+                        min(kPageTokens, pos - key0 + 1), page_fully_visible(pos, pos, key0, window, sinks),
+                        scale * kLog2e, window, sinks);
     }
     // merge the four waves
     if (g == 0) { lds_m[wave][c] = st.m; lds_l[wave][c] = st.l; }
@@ -209,7 +256,7 @@ __global__ __launch_bounds__(kAttnWaves * kWave) void attn_decode_kernel(
         float l = 0.f, o = 0.f;
 #pragma unroll
         for (int w = 0; w < kAttnWaves; ++w) {
-            const float f = (lds_m[w][col] == -INFINITY) ? 0.f : expf(lds_m[w][col] - m);
+            const float f = (lds_m[w][col] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(lds_m[w][col] - m);
             l += lds_l[w][col] * f;
             o += lds_o[w][col][d] * f;
         }
@@ -232,7 +279,7 @@ __global__ void attn_decode_merge_kernel(bf16_t* __restrict__ out, const float* 
     float l = 0.f, o = 0.f;
     for (int z = 0; z < used; ++z) {
         const float* p = src + (size_t)z * (HD + 2);
-        const float f = (p[0] == -INFINITY) ? 0.f : expf(p[0] - m);
+        const float f = (p[0] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(p[0] - m);
         l += p[1] * f;
         o += p[2 + d] * f;
     }
@@ -287,7 +334,8 @@ __global__ __launch_bounds__(kAttnWaves * kWave) void attn_prefill_kernel(
         const int page = table[(size_t)b * table_stride + pi];
         const size_t base = ((size_t)page * n_kv_heads + kvh) * kPageTokens * HD;
         attend_page<HD>(st, qf, k_pool + base, v_pool + base, q_pos, key0, min(kPageTokens, written - key0),
-                        scale, window, sinks);
+                        rows == 16 && page_fully_visible(first_pos, last_pos, key0, window, sinks),
+                        scale * kLog2e, window, sinks);
     }
     if (!col_ok) return;
     const float inv = st.l > 0.f ? 1.0f / st.l : 0.f;
@@ -319,15 +367,45 @@ struct PageLds {
     bf16_t v[HD][kPageTokens + kVPad];
 };
 
+// the tile's queries, kept in LDS so that their fragments need no registers between pages
 template <int HD>
-__global__ __launch_bounds__(kAttnWaves * kWave) void attn_prefill_lds_kernel(
+struct TileLds {
+    PageLds<HD> page[2];
+    bf16_t q[kTileRows][HD + kKPad];
+};
+
+template <int HD, int N>
+__device__ __forceinline__ void fetch_page(uint4 (&kreg)[N], uint4 (&vreg)[N], const bf16_t* __restrict__ kpage,
+                                           const bf16_t* __restrict__ vpage) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        const int piece = i * (kAttnWaves * kWave) + threadIdx.x;
+        kreg[i] = *reinterpret_cast<const uint4*>(kpage + (size_t)piece * 8);
+        vreg[i] = *reinterpret_cast<const uint4*>(vpage + (size_t)piece * 8);
+    }
+}
+
+template <int HD, int N>
+__device__ __forceinline__ void stash_page(PageLds<HD>& pg, const uint4 (&kreg)[N], const uint4 (&vreg)[N]) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        const int piece = i * (kAttnWaves * kWave) + threadIdx.x;
+        *reinterpret_cast<uint4*>(&pg.k[piece / (HD / 8)][(piece % (HD / 8)) * 8]) = kreg[i];
+        *reinterpret_cast<uint4*>(&pg.v[piece / (kPageTokens / 8)][(piece % (kPageTokens / 8)) * 8]) = vreg[i];
+    }
+}
+
+template <int HD>
+__global__ __launch_bounds__(kAttnWaves * kWave) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void attn_prefill_lds_kernel(
         bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int q_stride,
         const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
         const int* __restrict__ table, int table_stride, const int* __restrict__ cu,
         const int* __restrict__ tok_pos, int batch, int n_heads, int n_kv_heads, int group,
         float scale, int window, int sinks) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    PageLds<HD>* lds = reinterpret_cast<PageLds<HD>*>(smem_raw);      // two buffers
+    TileLds<HD>& tl = *reinterpret_cast<TileLds<HD>*>(smem_raw);
+    PageLds<HD>* lds = tl.page;                                       // two buffers
     int tile = blockIdx.x, b = 0, first = 0;
     for (; b < batch; ++b) {
         const int len = cu[b + 1] - cu[b];
@@ -347,117 +425,104 @@ __global__ __launch_bounds__(kAttnWaves * kWave) void attn_prefill_lds_kernel(
     // this wave: rows first + 32 wave .. + 31, column block cb holds rows + 16 cb
     const int row0 = first + 32 * wave;
     const int wave_rows = max(0, min(32, seq_end - row0));
-    int q_pos[2];
-    bf16x8 qf[2][HD / 32];
-    WaveState<HD> st[2];
-#pragma unroll
-    for (int cb = 0; cb < 2; ++cb) {
-        const int rr = 16 * cb + c;
-        const bool ok = rr < wave_rows;
-        q_pos[cb] = ok ? tok_pos[row0 + rr] : -1;
-        const bf16_t* qrow = q + (size_t)(row0 + (ok ? rr : 0)) * q_stride + (size_t)h * HD + 8 * g;
-#pragma unroll
-        for (int sk = 0; sk < HD / 32; ++sk) qf[cb][sk] = ok ? ld_frag(qrow + 32 * sk) : zero_frag();
-        st[cb].init();
+    const bool ok0 = c < wave_rows, ok1 = 16 + c < wave_rows;
+    const int q_pos0 = ok0 ? tok_pos[row0 + c] : -1, q_pos1 = ok1 ? tok_pos[row0 + 16 + c] : -1;
+    // the wave's 32 query rows go to LDS (rows past the sequence as zeros)
+    for (int piece = lane; piece < 32 * (HD / 8); piece += kWave) {
+        const int rr = piece / (HD / 8), col = (piece % (HD / 8)) * 8;
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (rr < wave_rows) v = *reinterpret_cast<const uint4*>(q + (size_t)(row0 + rr) * q_stride + (size_t)h * HD + col);
+        *reinterpret_cast<uint4*>(&tl.q[32 * wave + rr][col]) = v;
     }
+    WaveState<HD> st0, st1;
+    st0.init();
+    st1.init();
     const int wave_first_pos = wave_rows > 0 ? tok_pos[row0] : 0;
     const int wave_last_pos = wave_rows > 0 ? tok_pos[row0 + wave_rows - 1] : -1;
+    const float scale_log2 = scale * kLog2e;
 
     // the pages the tile needs, in order
     const int n_pages = tile_last_pos / kPageTokens + 1;
     auto page_needed = [&](int pi) {
         return page_may_be_visible_to_range(tile_first_pos, tile_last_pos, pi * kPageTokens, window, sinks);
     };
-    constexpr int kPieces = kPageTokens * HD / 8;                         // 16-byte pieces of a page (keys or values)
-    constexpr int kPerThread = kPieces / (kAttnWaves * kWave);
+    constexpr int kPerThread = kPageTokens * HD / 8 / (kAttnWaves * kWave);   // 16-byte pieces of a page per thread
     uint4 kreg[kPerThread], vreg[kPerThread];
-    auto fetch = [&](int pi) {
-        const int page = table[(size_t)b * table_stride + pi];
-        const size_t base = ((size_t)page * n_kv_heads + kvh) * kPageTokens * HD;
-#pragma unroll
-        for (int i = 0; i < kPerThread; ++i) {
-            const int piece = i * (kAttnWaves * kWave) + threadIdx.x;
-            kreg[i] = *reinterpret_cast<const uint4*>(k_pool + base + (size_t)piece * 8);
-            vreg[i] = *reinterpret_cast<const uint4*>(v_pool + base + (size_t)piece * 8);
-        }
+    // walk the needed pages with one page of look-ahead; the page id of the page after next is
+    // read one iteration early, so that no iteration waits for the table and then for the page
+    auto next_needed = [&](int pi) {
+        ++pi;
+        while (pi < n_pages && !page_needed(pi)) ++pi;
+        return pi;
     };
-    auto stash = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < kPerThread; ++i) {
-            const int piece = i * (kAttnWaves * kWave) + threadIdx.x;
-            *reinterpret_cast<uint4*>(&lds[buf].k[piece / (HD / 8)][(piece % (HD / 8)) * 8]) = kreg[i];
-            *reinterpret_cast<uint4*>(&lds[buf].v[piece / (kPageTokens / 8)][(piece % (kPageTokens / 8)) * 8]) = vreg[i];
+    auto page_id = [&](int pi) { return table[(size_t)b * table_stride + pi]; };
+    auto page_base = [&](int id) { return ((size_t)id * n_kv_heads + kvh) * kPageTokens * HD; };
+    int cur = next_needed(-1);
+    if (cur >= n_pages) return;                                          // cannot happen: a row sees itself
+    int nxt = next_needed(cur);
+    int cur_id = page_id(cur);
+    int nxt_id = nxt < n_pages ? page_id(nxt) : cur_id;
+    {
+        const size_t base = page_base(cur_id);
+        fetch_page<HD, kPerThread>(kreg, vreg, k_pool + base, v_pool + base);
+        stash_page<HD, kPerThread>(lds[0], kreg, vreg);
+    }
+    __syncthreads();
+    int buf = 0;
+    while (cur < n_pages) {
+        const int nxt2 = next_needed(nxt);
+        {   // always fetched and stashed (past the end: the current page once more, never used)
+            const size_t base = page_base(nxt_id);
+            fetch_page<HD, kPerThread>(kreg, vreg, k_pool + base, v_pool + base);
         }
-    };
-    auto compute = [&](int pi, int buf) {
+        const int nxt2_id = nxt2 < n_pages ? page_id(nxt2) : nxt_id;
+        const int pi = cur;
+        do {
         const int key0 = pi * kPageTokens;
-        if (wave_rows <= 0 || key0 > wave_last_pos) return;               // nothing of this page for this wave
-        if (!page_may_be_visible_to_range(wave_first_pos, wave_last_pos, key0, window, sinks)) return;
+        if (wave_rows <= 0 || key0 > wave_last_pos) break;                // nothing of this page for this wave
+        if (!page_may_be_visible_to_range(wave_first_pos, wave_last_pos, key0, window, sinks)) break;
         const int valid_keys = min(kPageTokens, written - key0);
         const PageLds<HD>& pg = lds[buf];
         // S^T for both column blocks; operand row c of block rb is key 16 rb + c
-        f32x4 s[2][4];
+        f32x4 s0[4], s1[4];
 #pragma unroll
         for (int rb = 0; rb < 4; ++rb) {
-            s[0][rb] = f32x4{0.f, 0.f, 0.f, 0.f};
-            s[1][rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+            s0[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+            s1[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
 #pragma unroll
-            for (int sk = 0; sk < HD / 32; ++sk) {
+        for (int sk = 0; sk < HD / 32; ++sk) {
+            const bf16x8 qf0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&tl.q[32 * wave + c][32 * sk + 8 * g]));
+            const bf16x8 qf1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&tl.q[32 * wave + 16 + c][32 * sk + 8 * g]));
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb) {
                 const bf16x8 kf = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&pg.k[16 * rb + c][32 * sk + 8 * g]));
-                s[0][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[0][sk], s[0][rb], 0, 0, 0);
-                s[1][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[1][sk], s[1][rb], 0, 0, 0);
+                s0[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf0, s0[rb], 0, 0, 0);
+                s1[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf1, s1[rb], 0, 0, 0);
             }
         }
-        // lane (c, g) of block cb: column c, keys key0 + 16 rb + 4 g + r
-        bf16x8 pf[2][2];
-        float corr[2];
-#pragma unroll
-        for (int cb = 0; cb < 2; ++cb) {
-            float tile_max = -INFINITY;
-#pragma unroll
-            for (int rb = 0; rb < 4; ++rb)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int key = key0 + 16 * rb + 4 * g + r;
-                    const bool vis = q_pos[cb] >= 0 && key_visible(q_pos[cb], key, window, sinks);
-                    const float v = vis ? s[cb][rb][r] * scale : -INFINITY;
-                    s[cb][rb][r] = v;
-                    tile_max = fmaxf(tile_max, v);
-                }
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
-            tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
-            const float m_new = fmaxf(st[cb].m, tile_max);
-            const bool any = m_new != -INFINITY;
-            corr[cb] = (st[cb].m == -INFINITY) ? 0.f : expf(st[cb].m - m_new);
-            float p[16], sum = 0.f;
-#pragma unroll
-            for (int rb = 0; rb < 4; ++rb)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const float e = (any && s[cb][rb][r] != -INFINITY) ? expf(s[cb][rb][r] - m_new) : 0.f;
-                    p[4 * rb + r] = e;
-                    sum += e;
-                }
-            sum += __shfl_xor(sum, 16, kWave);
-            sum += __shfl_xor(sum, 32, kWave);
-            st[cb].l = st[cb].l * corr[cb] + sum;
-            st[cb].m = m_new;
-            // step t covers blocks 2 t and 2 t + 1: slots 0..3 keys 32 t + 4 g + e, slots 4..7 keys 32 t + 16 + 4 g + e
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                uint4 u;
-                u.x = pack_bf16(p[8 * t + 0], p[8 * t + 1]);
-                u.y = pack_bf16(p[8 * t + 2], p[8 * t + 3]);
-                u.z = pack_bf16(p[8 * t + 4], p[8 * t + 5]);
-                u.w = pack_bf16(p[8 * t + 6], p[8 * t + 7]);
-                pf[cb][t] = __builtin_bit_cast(bf16x8, u);
-            }
+        // lane (c, g) of block cb: column c, keys key0 + 16 rb + 4 g + r; step t of the value
+        // product covers blocks 2 t and 2 t + 1: slots 0..3 keys 32 t + 4 g + e, slots 4..7 keys
+        // 32 t + 16 + 4 g + e
+        bf16x8 pf0[2], pf1[2];
+        float corr0, corr1;
+        const bool all_visible = wave_rows == 32 &&
+                                 page_fully_visible(wave_first_pos, wave_last_pos, key0, window, sinks);
+        if (all_visible) {
+            softmax_page<false, 4, 16, HD>(s0, st0, scale_log2, q_pos0, key0, window, sinks, pf0, corr0);
+            softmax_page<false, 4, 16, HD>(s1, st1, scale_log2, q_pos1, key0, window, sinks, pf1, corr1);
+        } else {
+            softmax_page<true, 4, 16, HD>(s0, st0, scale_log2, q_pos0, key0, window, sinks, pf0, corr0);
+            softmax_page<true, 4, 16, HD>(s1, st1, scale_log2, q_pos1, key0, window, sinks, pf1, corr1);
         }
+        const bool rescale = __ballot(corr0 != 1.0f || corr1 != 1.0f) != 0;
 #pragma unroll
         for (int db = 0; db < HD / 16; ++db) {
-            f32x4 a0 = st[0].acc[db], a1 = st[1].acc[db];
+            f32x4 a0 = st0.acc[db], a1 = st1.acc[db];
+            if (rescale) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) { a0[r] *= corr[0]; a1[r] *= corr[1]; }
+                for (int r = 0; r < 4; ++r) { a0[r] *= corr0; a1[r] *= corr1; }
+            }
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
                 const bf16_t* vrow = &pg.v[16 * db + c][32 * t + 4 * g];
@@ -470,44 +535,34 @@ __global__ __launch_bounds__(kAttnWaves * kWave) void attn_prefill_lds_kernel(
                     hi.y &= (3 < n_hi) ? 0xffffffffu : ((2 < n_hi) ? 0x0000ffffu : 0u);
                 }
                 const bf16x8 vf = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
-                a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[0][t], a0, 0, 0, 0);
-                a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[1][t], a1, 0, 0, 0);
+                a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf0[t], a0, 0, 0, 0);
+                a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf1[t], a1, 0, 0, 0);
             }
-            st[0].acc[db] = a0;
-            st[1].acc[db] = a1;
+            st0.acc[db] = a0;
+            st1.acc[db] = a1;
         }
-    };
-
-    // walk the needed pages with one page of look-ahead
-    int cur = 0;
-    while (cur < n_pages && !page_needed(cur)) ++cur;
-    if (cur < n_pages) { fetch(cur); stash(0); }
-    __syncthreads();
-    int buf = 0;
-    while (cur < n_pages) {
-        int nxt = cur + 1;
-        while (nxt < n_pages && !page_needed(nxt)) ++nxt;
-        if (nxt < n_pages) fetch(nxt);
-        compute(cur, buf);
-        if (nxt < n_pages) stash(buf ^ 1);
+        } while (0);
+        stash_page<HD, kPerThread>(lds[buf ^ 1], kreg, vreg);
         __syncthreads();
         cur = nxt;
+        nxt = nxt2;
+        nxt_id = nxt2_id;
         buf ^= 1;
     }
-#pragma unroll
-    for (int cb = 0; cb < 2; ++cb) {
-        const int rr = 16 * cb + c;
-        if (rr >= wave_rows) continue;
-        const float inv = st[cb].l > 0.f ? 1.0f / st[cb].l : 0.f;
+    auto write_out = [&](const WaveState<HD>& st, int rr) {
+        if (rr >= wave_rows) return;
+        const float inv = st.l > 0.f ? 1.0f / st.l : 0.f;
         bf16_t* orow = out + ((size_t)(row0 + rr) * n_heads + h) * HD;
 #pragma unroll
         for (int db = 0; db < HD / 16; ++db) {
             uint2 u;
-            u.x = pack_bf16(st[cb].acc[db][0] * inv, st[cb].acc[db][1] * inv);
-            u.y = pack_bf16(st[cb].acc[db][2] * inv, st[cb].acc[db][3] * inv);
+            u.x = pack_bf16(st.acc[db][0] * inv, st.acc[db][1] * inv);
+            u.y = pack_bf16(st.acc[db][2] * inv, st.acc[db][3] * inv);
             *reinterpret_cast<uint2*>(orow + 16 * db + 4 * g) = u;
         }
-    }
+    };
+    write_out(st0, c);
+    write_out(st1, 16 + c);
 }
 
 // ---------------------------------------------------------------- entry points
@@ -557,7 +612,7 @@ LLOGOS_EXPORT int llogos_attn_prefill_bf16(void* out, const void* q, int q_strid
     dim3 grid(n_tiles, n_heads);
     if (tile_rows == kTileRows) {
 #define GOL(HD) do { \
-        const size_t smem = 2 * sizeof(PageLds<HD>); \
+        const size_t smem = sizeof(TileLds<HD>); \
         hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<HD>, \
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
         if (e != hipSuccess) return (int)e; \
