@@ -92,8 +92,8 @@ __device__ __forceinline__ void store4_f32(bf16_t* p, float4 v) {
 
 constexpr int kMaxNormParts = 8;
 
-template <typename TO, typename TD, int ITEMS>
-__global__ void rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ x, const TD* __restrict__ delta,
+template <typename TO, typename TD, int ITEMS, int MAXP>
+__global__ __launch_bounds__(1024) void rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ x, const TD* __restrict__ delta,
                                    int parts, size_t part_stride,
                                    const int* __restrict__ rows, const float* __restrict__ w,
                                    float eps, int H, int write_back) {
@@ -103,7 +103,7 @@ __global__ void rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ x, 
     float* xr = x + s * H;
     const TD* dr = delta ? delta + s * H : nullptr;
     float4 v[ITEMS], wv[ITEMS];
-    float4 dv[ITEMS][kMaxNormParts];
+    float4 dv[ITEMS][MAXP];
 #pragma unroll
     for (int it = 0; it < ITEMS; ++it) {
         const int i = 4 * (it * blockDim.x + threadIdx.x);
@@ -111,7 +111,7 @@ __global__ void rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ x, 
         v[it] = ok ? load4_f32(xr + i) : make_float4(0.f, 0.f, 0.f, 0.f);
         wv[it] = ok ? load4_f32(w + i) : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-        for (int q = 0; q < kMaxNormParts; ++q)
+        for (int q = 0; q < MAXP; ++q)
             dv[it][q] = (ok && dr && q < parts) ? load4_f32(dr + q * part_stride + i) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
     float ss = 0.f;
@@ -120,7 +120,7 @@ __global__ void rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ x, 
         if (dr) {
             float4 d = dv[it][0];
 #pragma unroll
-            for (int q = 1; q < kMaxNormParts; ++q) {       // ascending order, as sum_parts
+            for (int q = 1; q < MAXP; ++q) {                // ascending order, as sum_parts
                 d.x += dv[it][q].x; d.y += dv[it][q].y; d.z += dv[it][q].z; d.w += dv[it][q].w;
             }
             v[it].x += d.x; v[it].y += d.y; v[it].z += d.z; v[it].w += d.w;
@@ -150,17 +150,19 @@ LLOGOS_EXPORT int llogos_rmsnorm(void* out, int out_dtype, float* x, const void*
     if (R <= 0 || H <= 0 || parts < 1) return LLOGOS_BAD_ARGUMENT;
     const bool aligned = (H % 4 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0) &&
                          ((uintptr_t)out % 16 == 0) && (!delta || ((uintptr_t)delta % 16 == 0 && part_stride % 4 == 0));
-    if (aligned && parts <= kMaxNormParts && H <= 4 * 4 * 1024) {
+    if (aligned && parts <= kMaxNormParts && H <= (parts == 1 ? 4 : 2) * 4 * 1024) {
         const int groups = H / 4;
         // few rows: one group per thread, so that the row's loads are all in flight at once;
         // many rows: four groups per thread, fewer and fuller waves
         int items = groups <= 1024 ? 1 : (groups <= 2048 ? 2 : 4);
-        if (R >= 256 && groups >= 256) items = 4;
+        if (R >= 256 && groups >= 256 && parts == 1) items = 4;
         int threads = (groups + items - 1) / items;
         threads = (threads + kWave - 1) / kWave * kWave;
-#define LAUNCHV(TO, TD, IT) rmsnorm_vec_kernel<TO, TD, IT><<<R, threads, 0, stream>>>( \
+#define LAUNCHV(TO, TD, IT, MP) rmsnorm_vec_kernel<TO, TD, IT, MP><<<R, threads, 0, stream>>>( \
         (TO*)out, x, (const TD*)delta, parts, (size_t)part_stride, rows, w, eps, H, write_back)
-#define PICK(TO, TD) do { if (items == 1) LAUNCHV(TO, TD, 1); else if (items == 2) LAUNCHV(TO, TD, 2); else LAUNCHV(TO, TD, 4); } while (0)
+#define PICK(TO, TD) do { \
+        if (parts == 1) { if (items == 1) LAUNCHV(TO, TD, 1, 1); else if (items == 2) LAUNCHV(TO, TD, 2, 1); else LAUNCHV(TO, TD, 4, 1); } \
+        else { if (items == 1) LAUNCHV(TO, TD, 1, kMaxNormParts); else LAUNCHV(TO, TD, 2, kMaxNormParts); } } while (0)
         if (out_dtype == DT_F32 && delta_dtype == DT_F32) PICK(float, float);
         else if (out_dtype == DT_BF16 && delta_dtype == DT_BF16) PICK(bf16_t, bf16_t);
         else if (out_dtype == DT_BF16 && delta_dtype == DT_F32) PICK(bf16_t, float);

@@ -165,6 +165,28 @@ def test_window_and_sinks_as_run_time_strategy(name, dtype):
     assert np.abs(want - H.plain_logits(name, toks)).max() > 1e-3              # the window matters here
 
 
+@pytest.mark.parametrize("dtype", H.DTYPES)
+def test_llama_8b_layer_sizes(dtype):
+    """Two layers of the 8B layer sizes (hidden 4096, 32/8 heads of 128, feed-forward 14336):
+    whole, the last tokens one by one, and an unequal batch, against the plain implementation."""
+    name = "layer_8b"
+    eng = H.engine(name, dtype, max_tokens=64 * 12, n_slots=3)
+    a, b, c = H.tokens(name, 150, 1), H.tokens(name, 70, 2), H.tokens(name, 3, 3)
+    pa, pb, pc = (H.plain_logits(name, t) for t in (a, b, c))
+    s = eng.alloc_slot()
+    rows = [_np(eng.step([(s, a[:140])], want="all"))] + [_np(eng.step([(s, [t])])) for t in a[140:]]
+    H.close(np.concatenate(rows), pa, dtype, "8B sizes: prompt then tokens")
+    eng.free_slot(s)
+    slots = [eng.alloc_slot() for _ in range(3)]
+    out = _np(eng.step([(slots[0], a[:100]), (slots[1], b[:66]), (slots[2], c[:2])], want="all"))
+    H.close(out, np.concatenate([pa[:100], pb[:66], pc[:2]]), dtype, "8B sizes: unequal batch")
+    out = _np(eng.step([(slots[0], [a[100]]), (slots[1], [b[66]]), (slots[2], [c[2]])], want="last"))
+    H.close(out, np.stack([pa[100], pb[66], pc[2]]), dtype, "8B sizes: one token each")
+    eng.free_slot(slots[2])
+    out = _np(eng.step([(slots[0], a[101:150]), (slots[1], [b[67]])], want=[[48], [0]]))
+    H.close(out, np.stack([pa[149], pb[67]]), dtype, "8B sizes: a continued prompt beside a single token")
+
+
 def test_step_errors():
     eng = H.engine("tiny_a", "float32", max_tokens=128, n_slots=2)
     s = eng.alloc_slot()

@@ -56,3 +56,32 @@ def test_replay_refuses_more_than_the_cache_holds(tmp_path):
            "--dtype", "float32", "--out", str(tmp_path / "o"), "--max-tokens", "64"]
     p = subprocess.run(cmd, input=json.dumps(steps[0]) + "\n", capture_output=True, text=True, timeout=600)
     assert p.returncode != 0 and "pages" in p.stderr
+
+
+def test_command_line_generates_and_benchmarks():
+    """The command line as a subprocess: greedy generation prints token ids, --bench the
+    reference's block (Daisi.Llogos.Cli/Program.cs:292-296)."""
+    import plain_model as pm
+    name = "tiny_b"
+    cfg, w = H.plain(name)
+    prompt = list(H.tokens(name, 12, 77))
+    cmd = [sys.executable, "-m", "daisi-llogos_amd", "--model", H.folder(name), "--prompt", " ".join(map(str, prompt)),
+           "-n", "6", "-t", "0", "--repeat-penalty", "1.0", "--dtype", "float32", "--max-context", "64"]
+    p = subprocess.run(cmd, capture_output=True, text=True, timeout=600, cwd=ROOT)
+    assert p.returncode == 0, p.stderr[-2000:]
+    got = [int(t) for t in p.stdout.split()]
+    want = pm.generate_greedy(cfg, w, prompt, 6, stop=set(cfg_eos(name)))
+    assert got == want
+    assert "prefill: 12 tokens" in p.stderr and "decode:" in p.stderr
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "llogos"), "-m", H.folder(name), "--bench", "-n", "8",
+                        "--prompt-len", "20", "--batch", "2", "--max-context", "64"],
+                       capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert "=== Benchmark Results ===" in p.stderr and "Prefill:" in p.stderr and "Decode:" in p.stderr
+    assert "40 tokens" in p.stderr.split("Prefill:")[1].split("\n")[0].replace("    ", " ")
+
+
+def cfg_eos(name):
+    import tiny_configs as tc
+    e = tc.ALL[name]["eos_token_id"]
+    return e if isinstance(e, list) else [e]

@@ -40,4 +40,13 @@ TINY_D = {   # Llama style with head size 64 and window: the matrix-core attenti
     "tie_word_embeddings": False, "torch_dtype": "bfloat16", "eos_token_id": 1,
 }
 
-ALL = {"tiny_a": TINY_A, "tiny_b": TINY_B, "tiny_c": TINY_C, "tiny_w": TINY_W, "tiny_d": TINY_D}
+LAYER_8B = {   # two layers of the Llama-3.1-8B layer sizes with a small vocabulary: the kernels at real widths
+    "architectures": ["LlamaForCausalLM"], "vocab_size": 1031, "hidden_size": 4096, "intermediate_size": 14336,
+    "num_hidden_layers": 2, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+    "rms_norm_eps": 1e-5, "rope_theta": 500000.0, "max_position_embeddings": 131072,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 8192},
+    "tie_word_embeddings": False, "torch_dtype": "bfloat16", "eos_token_id": 2,
+}
+
+ALL = {"tiny_a": TINY_A, "tiny_b": TINY_B, "tiny_c": TINY_C, "tiny_w": TINY_W, "tiny_d": TINY_D, "layer_8b": LAYER_8B}
