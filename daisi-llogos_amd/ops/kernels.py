@@ -359,11 +359,13 @@ def gemm_skinny_lds_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.
     return out
 
 
-def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swiglu_input: bool = False) -> torch.Tensor:
+def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swiglu_input: bool = False,
+                 f32_ok: bool = False) -> torch.Tensor:
     """a [M, K] . w [N, K]^T without bias, as [M, N] of `out_dtype` or as float32 partial sums
     [parts, M, N] for a consumer that adds them (rmsnorm, qk_rope_cache, swiglu, sum_parts).
     With `swiglu_input`, `a` is a fused gate/up product ([M, 2 K] or parts of it) and the
-    product is taken of silu(gate) * up.
+    product is taken of silu(gate) * up.  With `f32_ok` the consumer also takes one float32
+    [M, N], which spares the result a rounding to bfloat16.
 
     float32 operands: plain FMAs in 32-bit throughout.  bfloat16 operands: up to 64 rows the
     hand-written weight-streaming kernels; more rows the library product (as the reference
@@ -388,6 +390,8 @@ def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swigl
         a = swiglu(a, out_dtype)
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out_dtype == torch.bfloat16 and a.is_contiguous() \
             and M > SKINNY_MAX_ROWS:
+        if f32_ok:
+            return torch.mm(a, w.t(), out_dtype=torch.float32)
         return torch.matmul(a, w.t())
     return gemm_generic(a, w, None, out_dtype)
 

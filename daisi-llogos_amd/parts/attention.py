@@ -69,16 +69,16 @@ class Attention(Mixer):
         nh, nkv, hd = self.n_heads, self.n_kv_heads, self.head_dim
         cs = self.position.prepare(ctx)
         if cache.writes:
-            qkv = self.qkv.product(h)                                   # [(parts,) T, (nh + 2 nkv) hd]
+            qkv = self.qkv.product(h, f32_ok=True)                      # [(parts,) T, (nh + 2 nkv) hd]
             q = K.qk_rope_cache(qkv, self.qkv.bias_rows(), self.rt.dtype, nh, nkv, hd, self.position.rot,
                                 self.position.pairing, self.q_norm_w, self.k_norm_w, self.eps, cs,
                                 cache.k_pool, cache.v_pool, cache.table, ctx.tok_seq, ctx.tok_pos)
         else:
             # the keys and values of these positions are another layer's: project q alone
-            qkv = self.qkv.product(h, rows_out=nh * hd)
+            qkv = self.qkv.product(h, rows_out=nh * hd, f32_ok=True)
             q = K.qk_rope_cache(qkv, self.qkv.bias_rows(nh * hd), self.rt.dtype, nh, 0, hd, self.position.rot,
                                 self.position.pairing, self.q_norm_w, None, self.eps, cs, None, None, None,
                                 ctx.tok_seq, ctx.tok_pos)
         a = K.attention(ctx, q, q.stride(0), cache.k_pool, cache.v_pool, cache.table,
                         nh, nkv, hd, self.scale, self.window, self.sinks)
-        return self.o.product(a)                # the residual sum that follows adds the parts
+        return self.o.product(a, f32_ok=True)   # the residual sum that follows adds the parts

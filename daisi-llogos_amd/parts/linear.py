@@ -48,12 +48,14 @@ class Linear(Part):
         self.rt = rt
         self.weight = weight
 
-    def product(self, a: torch.Tensor, rows_out: Optional[int] = None, swiglu_input: bool = False) -> torch.Tensor:
+    def product(self, a: torch.Tensor, rows_out: Optional[int] = None, swiglu_input: bool = False,
+                f32_ok: bool = False) -> torch.Tensor:
         """a . W^T without the bias, as [M, out] or as float32 partial sums [parts, M, out] for a
         consumer kernel that adds parts (and the bias, `bias_rows`).  With `swiglu_input`, `a` is a
-        fused gate/up product (maybe in parts) and W is applied to silu(gate) * up."""
+        fused gate/up product (maybe in parts) and W is applied to silu(gate) * up; with `f32_ok`
+        the consumer also takes a float32 result."""
         w = self.weight if rows_out is None else self.weight[:rows_out]
-        return K.gemm_product(a, w, self.rt.dtype, swiglu_input=swiglu_input)
+        return K.gemm_product(a, w, self.rt.dtype, swiglu_input=swiglu_input, f32_ok=f32_ok)
 
     def bias_rows(self, rows_out: Optional[int] = None) -> Optional[torch.Tensor]:
         return self.bias if (self.bias is None or rows_out is None) else self.bias[:rows_out]

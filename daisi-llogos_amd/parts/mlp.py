@@ -31,4 +31,4 @@ class SwiGLU(FeedForward):
         gu = self.gate_up.product(h)
         # silu(gate) * up is made inside the down product where its kernel can (few rows), by a
         # kernel of its own otherwise; the residual sum that follows adds the product's parts
-        return self.down.product(gu, swiglu_input=True)
+        return self.down.product(gu, swiglu_input=True, f32_ok=True)
