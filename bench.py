@@ -56,7 +56,7 @@ def prefill_flops(cfg, t):
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--steps", type=int, default=248)   # + 8 warm-up = 256 new tokens
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration has (0 = all)")
@@ -146,8 +146,8 @@ def main(argv=None) -> int:
     if not args.no_points:
         points = {}
         for b in (1, 64):
-            steps = min(args.steps, 64)
-            d, _ = decode_run(b, steps, min(args.warmup, 4))
+            steps = args.steps
+            d, _ = decode_run(b, steps, args.warmup)
             points[f"decode_b{b}"] = round(b * steps / d, 1)
             print(f"[bench] decode b{b}: {points[f'decode_b{b}']:.1f} tok/s, {d / steps * 1e3:.3f} ms/step",
                   file=sys.stderr, flush=True)

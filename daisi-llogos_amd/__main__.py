@@ -30,6 +30,9 @@ Options:
   --batch <n>              Sequences generated together (default: number of prompts; bench: 1)
   --prompt-len <n>         Bench without --prompt: random prompt of this length (default: 512)
   --help, -h               Show this help
+
+Random weights (a model folder from a configuration and a seed):
+  python -m daisi-llogos_amd random --config <config.json> --output-dir <folder> [--seed <n>]
 """
 
 
@@ -110,8 +113,43 @@ def parse_prompts(text: str, model_dir: str):
     return prompts
 
 
+def run_random(argv) -> int:
+    """`random --config FILE --output-dir DIR [--seed N]`: config.json + model.safetensors with
+    random weights for the configuration's architecture (the reference has no such mode; its
+    sub-commands are `split` and `train`, Daisi.Llogos.Cli/Program.cs:25-31)."""
+    import json
+    config = out = None
+    seed = 0
+    i = 0
+    try:
+        while i < len(argv):
+            if argv[i] == "--config": config = argv[i + 1]; i += 1
+            elif argv[i] in ("--output-dir", "-o"): out = argv[i + 1]; i += 1
+            elif argv[i] == "--seed": seed = int(argv[i + 1]); i += 1
+            else:
+                raise ValueError(f"unknown option {argv[i]}")
+            i += 1
+    except (IndexError, ValueError) as e:
+        print(f"Error: {e if isinstance(e, ValueError) else 'missing value'}", file=sys.stderr)
+        return 1
+    if not config or not out:
+        print("Error: random needs --config and --output-dir", file=sys.stderr)
+        return 1
+    if not os.path.isfile(config):
+        print(f"Error: configuration not found: {config}", file=sys.stderr)
+        return 1
+    from .weights.random_init import write_random_model
+    with open(config) as fh:
+        data = json.load(fh)
+    write_random_model(out, data, seed=seed)
+    print(f"wrote {out}/config.json and {out}/model.safetensors (seed {seed})", file=sys.stderr)
+    return 0
+
+
 def main(argv=None) -> int:
     argv = list(sys.argv[1:] if argv is None else argv)
+    if argv and argv[0] == "random":
+        return run_random(argv[1:])
     try:
         args = parse_args(argv)
     except ValueError as e:

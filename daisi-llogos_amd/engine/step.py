@@ -26,6 +26,9 @@ _DTYPES = {"float32": torch.float32, "fp32": torch.float32, "f32": torch.float32
            "bfloat16": torch.bfloat16, "bf16": torch.bfloat16}
 
 
+GRAPH_MAX_BATCH = 64
+
+
 class StepError(ValueError):
     """A step that cannot run: empty token list, token out of range, slot used twice."""
 
@@ -163,7 +166,9 @@ class Engine:
 
         self.cache.reserve(slot_ids, new_lens)
         T, B = int(cu[-1]), len(entries)
-        if self.graphs is not None and T == B and rows == list(range(B)) and self.cache.slots.n_slots == self._graph_slots():
+        # (more rows than the hand-written products take would put a library call into the graph)
+        if self.graphs is not None and T == B and B <= GRAPH_MAX_BATCH and rows == list(range(B)) \
+                and self.cache.slots.n_slots == self._graph_slots():
             with torch.cuda.device(self.rt.device):
                 logits = self.graphs.step(ids.astype(np.int32), np.asarray(starts, dtype=np.int32),
                                           np.asarray(slot_ids, dtype=np.int32), self.cache.step_tables(slot_ids))

@@ -53,3 +53,18 @@ def test_attention_strategy_strings():
     for bad in ("window:0", "sinks:4", "ring", "sinks:-1,5"):
         with pytest.raises(ValueError):
             api.parse_attention(bad)
+
+
+def test_random_subcommand_writes_a_model_folder(tmp_path, llogos):
+    import json
+    import tiny_configs as tc
+    cfg = tmp_path / "c.json"
+    cfg.write_text(json.dumps(tc.TINY_A))
+    out = tmp_path / "model"
+    assert cli.main(["random", "--config", str(cfg), "--output-dir", str(out), "--seed", "4"]) == 0
+    ck = llogos.Checkpoint(str(out))
+    arch = llogos.architecture_of(tc.TINY_A)
+    ck.check(llogos.Model(arch.model_spec(arch.read_config(tc.TINY_A))).tensor_specs())
+    assert json.load(open(out / "config.json")) == tc.TINY_A
+    assert cli.main(["random", "--config", str(tmp_path / "nope.json"), "--output-dir", str(out)]) == 1
+    assert cli.main(["random", "--output-dir", str(out)]) == 1
