@@ -118,6 +118,112 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny_kernel(
     }
 }
 
+// Third form, for up to 16 activation rows, K <= 4096 and very many rows of w (gate/up, the
+// output head): the activations stay in registers.  The 4 waves of a block split k; each
+// wave loads its quarter of the activation fragments once (up to 32 steps = 128 registers)
+// and then streams `strips` strips of 16 rows of w past them, so that the activations cost
+// 1 / strips of what they cost when every strip fetches its own.  The waves' sums of a strip
+// are added through LDS in wave order, as in the first form.
+constexpr int kStatSteps = 32;          // MFMA steps of 32 values of k per wave at most
+constexpr int kStatU = 4;               // steps per prefetched chunk
+
+template <typename TO>
+__global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny_stationary_kernel(
+        TO* __restrict__ out, const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
+        const float* __restrict__ bias, int M, int N, int K, int lda, int ldo, int strips_per_block) {
+    __shared__ float red[kSkinnyWaves][kWave][4];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int r = lane & 15, g = lane >> 4;
+    const int k_per_wave = (((K + 31) / 32 + kSkinnyWaves - 1) / kSkinnyWaves) * 32;     // <= 32 * kStatSteps
+    const int k_begin = wave * k_per_wave;
+    const int k_end = min(K, k_begin + k_per_wave);
+    constexpr int kChunks = kStatSteps / kStatU;
+
+    // this wave's activation fragments, once
+    bf16x8 af[kStatSteps];
+    {
+        const bool row_ok = r < M;
+        const bf16_t* arow = a + (size_t)min(r, M - 1) * lda + g * 8;
+#pragma unroll
+        for (int s = 0; s < kStatSteps; ++s) {
+            const int kk = k_begin + s * kStepK;
+            af[s] = load_frag(arow + kk, row_ok && kk + g * 8 < k_end);
+        }
+    }
+    const int n_strips = (N + 15) / 16;
+    const int strip0 = blockIdx.x * strips_per_block;
+    const int my_strips = min(strips_per_block, n_strips - strip0);
+    if (my_strips <= 0) return;
+    const int total = my_strips * kChunks;                               // chunks of kStatU steps to stream
+
+    auto load_chunk = [&](bf16x8 (&wf)[kStatU], int gc) {
+        const int strip = strip0 + gc / kChunks, c = gc % kChunks;
+        const bf16_t* wrow = w + (size_t)min(strip * 16 + r, N - 1) * K + g * 8;
+#pragma unroll
+        for (int u = 0; u < kStatU; ++u) {
+            const int kk = k_begin + (c * kStatU + u) * kStepK;
+            wf[u] = load_frag(wrow + kk, gc < total && kk + g * 8 < k_end);
+        }
+    };
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    auto multiply = [&](const bf16x8 (&wf)[kStatU], int c) {
+        // the fragment index must be a constant for the registers: one case per chunk of the strip
+#pragma unroll
+        for (int cc = 0; cc < kChunks; ++cc)
+            if (cc == c) {
+#pragma unroll
+                for (int u = 0; u < kStatU; ++u)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u], af[cc * kStatU + u], acc, 0, 0, 0);
+            }
+    };
+    auto finish_strip = [&](int strip) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red[wave][lane][i] = acc[i];
+        acc = f32x4{0.f, 0.f, 0.f, 0.f};
+        __syncthreads();
+        const int t_lane = threadIdx.x & (kWave - 1), t_i = threadIdx.x / kWave;
+        float sum = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < kSkinnyWaves; ++wv) sum += red[wv][t_lane][t_i];
+        const int n = strip * 16 + 4 * (t_lane >> 4) + t_i, m = t_lane & 15;
+        if (m < M && n < N) store_f32(out + (size_t)m * ldo + n, sum + (bias ? bias[n] : 0.f));
+        __syncthreads();
+    };
+
+    bf16x8 wf0[kStatU], wf1[kStatU];
+    load_chunk(wf0, 0);
+    for (int gc = 0; gc < total; gc += 2) {
+        load_chunk(wf1, gc + 1);
+        multiply(wf0, gc % kChunks);
+        if ((gc + 1) % kChunks == 0) finish_strip(strip0 + gc / kChunks);
+        load_chunk(wf0, gc + 2);
+        if (gc + 1 < total) {
+            multiply(wf1, (gc + 1) % kChunks);
+            if ((gc + 2) % kChunks == 0) finish_strip(strip0 + (gc + 1) / kChunks);
+        }
+    }
+}
+
+// The few-row product with stationary activations: M <= 16, K <= 4096.  One part, bias allowed.
+LLOGOS_EXPORT int llogos_gemm_skinny_stationary_bf16(void* out, int out_dtype, const void* a, const void* w,
+                                                     const float* bias, int M, int N, int K, int lda, int ldo,
+                                                     int strips_per_block, hipStream_t stream) {
+    if (M <= 0 || N <= 0 || K <= 0 || lda < K || ldo < N || strips_per_block < 1) return LLOGOS_BAD_ARGUMENT;
+    if (out_dtype != DT_BF16 && out_dtype != DT_F32) return LLOGOS_BAD_ARGUMENT;
+    if (M > 16 || K > 32 * kStatSteps * kSkinnyWaves || (K % 8) || (lda % 8) || ((uintptr_t)a % 16) ||
+        ((uintptr_t)w % 16))
+        return LLOGOS_UNSUPPORTED;
+    const int n_strips = (N + 15) / 16;
+    const int blocks = (n_strips + strips_per_block - 1) / strips_per_block;
+    if (out_dtype == DT_BF16)
+        gemm_skinny_stationary_kernel<bf16_t><<<blocks, kSkinnyWaves * kWave, 0, stream>>>(
+            (bf16_t*)out, (const bf16_t*)a, (const bf16_t*)w, bias, M, N, K, lda, ldo, strips_per_block);
+    else
+        gemm_skinny_stationary_kernel<float><<<blocks, kSkinnyWaves * kWave, 0, stream>>>(
+            (float*)out, (const bf16_t*)a, (const bf16_t*)w, bias, M, N, K, lda, ldo, strips_per_block);
+    return LLOGOS_LAUNCH_CHECK();
+}
+
 template <int RB, int MB, int U>
 static int launch_skinny(void* out, int out_dtype, const bf16_t* a, const bf16_t* w, const float* bias,
                          int M, int N, int K, int lda, int ldo, size_t part_stride, int k_per_block,

@@ -268,10 +268,13 @@ SKINNY_MAX_ROWS = 64
 
 def skinny_plan(M: int, N: int, K: int) -> Tuple[str, int, int]:
     """(kernel, blocks along k, 16-row blocks of w per wave) for the few-row product.
-    'regs': every wave fetches its own activation fragments; best for up to 4 rows and many
-    rows of w.  'lds': the block shares the activations through LDS; its speed hardly depends
-    on the number of rows.  The split of k depends on N and K alone within a kernel, so the
+    'stationary': activations held in registers while strips of w stream past; best for few
+    rows and very many rows of w (gate/up, the head).  'regs': every wave fetches its own
+    activation fragments; for up to 4 rows where k is too long for 'stationary'.  'lds': the
+    block shares the activations through LDS; its speed hardly depends on the number of rows.  The split of k depends on N and K alone within a kernel, so the
     order of a row's additions does not depend on how many other rows the batch has."""
+    if N >= 16384 and K <= 4096 and (M <= 8 or (M <= 16 and N >= 65536)):
+        return "stationary", 1, (8 if N >= 65536 else 4)      # third value: strips per block
     if M <= 4 and N >= 16384:
         strips = -(-N // 16)
         return "regs", max(1, min(-(-1024 // strips), K // 1024, 8)), 1
@@ -308,6 +311,31 @@ def gemm_skinny_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tens
     if code == -2:
         return None
     _check(code, "gemm_skinny_bf16")
+    return out
+
+
+def gemm_skinny_stationary_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
+                                out_dtype: torch.dtype, strips: int = 4) -> Optional[torch.Tensor]:
+    """The few-row bfloat16 product with the activations held in registers while `strips` strips
+    of 16 rows of w stream past: up to 16 rows, K <= 4096.  [1, M, N]; None for other shapes."""
+    if a.dim() != 2:
+        return None
+    M, K = a.shape
+    N = w.shape[0]
+    if not (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and 0 < M <= 16 and K <= 4096 and K % 8 == 0
+            and a.stride(1) == 1 and a.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+            and w.is_contiguous()):
+        return None
+    _dev(w, bias)
+    _need(w.dim() == 2 and w.shape[1] == K, f"gemm: w must be [N, {K}], got {tuple(w.shape)}")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.shape == (N,), "gemm: bias must be float32 [N]")
+    out = torch.empty((1, M, N), dtype=out_dtype, device=a.device)
+    code = _lib().llogos_gemm_skinny_stationary_bf16(
+        _p(out), _DT[out_dtype], _p(a), _p(w), _p(bias), M, N, K, a.stride(0), N, int(strips), _stream())
+    if code == -2:
+        return None
+    _check(code, "gemm_skinny_stationary_bf16")
     return out
 
 
@@ -373,6 +401,13 @@ def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swigl
     M = a.shape[-2]
     if w.dtype == torch.bfloat16 and M <= SKINNY_MAX_ROWS and out_dtype == torch.bfloat16:
         kernel, splits, row_blocks = skinny_plan(M, w.shape[0], w.shape[1])
+        if kernel == "stationary" and not swiglu_input and a.dim() == 2:
+            out = gemm_skinny_stationary_bf16(a, w, None, out_dtype, row_blocks)
+            if out is not None:
+                return out
+            kernel, splits, row_blocks = "lds", 1, 1
+        elif kernel == "stationary":
+            kernel, splits, row_blocks = "lds", 1, 1
         # silu(gate) * up inside the product costs every block of rows of w a second read of the
         # gate/up row: worth it for few rows in bfloat16, not for partial sums or many rows
         if swiglu_input and not (M <= 16 and a.dtype == torch.bfloat16 and (a.dim() == 2 or a.shape[0] == 1)):
@@ -402,8 +437,14 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dty
         M = a.shape[0]
         if M <= SKINNY_MAX_ROWS:
             kernel, _, row_blocks = skinny_plan(M, w.shape[0], w.shape[1])
-            fn = gemm_skinny_lds_bf16 if kernel == "lds" else gemm_skinny_bf16
-            out = fn(a, w, bias, out_dtype, 1, row_blocks)
+            if kernel == "stationary":
+                out = gemm_skinny_stationary_bf16(a, w, bias, out_dtype, row_blocks)
+                kernel, row_blocks = "lds", 1
+            else:
+                out = None
+            if out is None:
+                fn = gemm_skinny_lds_bf16 if kernel == "lds" else gemm_skinny_bf16
+                out = fn(a, w, bias, out_dtype, 1, row_blocks)
             if out is not None:
                 return out[0]
         elif out_dtype == torch.bfloat16 and a.is_contiguous():
