@@ -271,8 +271,9 @@ def skinny_plan(M: int, N: int, K: int) -> Tuple[str, int, int]:
     'stationary': activations held in registers while strips of w stream past; best for few
     rows and very many rows of w (gate/up, the head).  'regs': every wave fetches its own
     activation fragments; for up to 4 rows where k is too long for 'stationary'.  'lds': the
-    block shares the activations through LDS; its speed hardly depends on the number of rows.  The split of k depends on N and K alone within a kernel, so the
-    order of a row's additions does not depend on how many other rows the batch has."""
+    block shares the activations through LDS; its speed hardly depends on the number of rows.
+    Within a kernel the split of k depends on N and K alone, so the order of a row's additions
+    does not depend on how many other rows the batch has."""
     if N >= 16384 and K <= 4096 and (M <= 8 or (M <= 16 and N >= 65536)):
         return "stationary", 1, (8 if N >= 65536 else 4)      # third value: strips per block
     if M <= 4 and N >= 16384:
