@@ -206,23 +206,31 @@ __device__ __forceinline__ bool page_may_be_visible_to_range(int first_pos, int 
 }
 
 // ---------------------------------------------------------------- decode
-// grid (batch, kv heads, ceil(table width / 4)); block 4 waves, wave w takes page 4 z + w.
-// partial: [batch][heads][grid.z][HD + 2] floats (max, sum, unnormalised output).
-template <int HD>
-__global__ __launch_bounds__(kAttnWaves * kWave) void attn_decode_kernel(
-        float* __restrict__ partial, const bf16_t* __restrict__ q, int q_stride,
+// grid (batch, kv heads, ceil(table width / WAVES)); block of WAVES waves, wave w takes page
+// WAVES z + w.  With one block along the context (gridDim.z == 1) the block writes the
+// attention output itself; otherwise partial: [batch][heads][grid.z][HD + 2] floats (max, sum,
+// unnormalised output) for the merge kernel.  Dynamic LDS: decode_lds_bytes(WAVES, group, HD).
+__host__ __device__ constexpr size_t decode_lds_bytes(int waves, int group, int hd) {
+    return (size_t)waves * (group * (hd + 1) + 32) * sizeof(float);
+}
+
+template <int HD, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void attn_decode_kernel(
+        bf16_t* __restrict__ out, float* __restrict__ partial, const bf16_t* __restrict__ q, int q_stride,
         const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
         const int* __restrict__ table, int table_stride, const int* __restrict__ tok_pos,
         int n_heads, int n_kv_heads, int group, float scale, int window, int sinks) {
-    __shared__ float lds_o[kAttnWaves][16][HD + 1];
-    __shared__ float lds_m[kAttnWaves][16], lds_l[kAttnWaves][16];
+    extern __shared__ float lds[];
+    float* lds_m = lds;                                   // [WAVES][16]
+    float* lds_l = lds + WAVES * 16;                      // [WAVES][16]
+    float* lds_o = lds + WAVES * 32;                      // [WAVES][group][HD + 1]
     const int b = blockIdx.x, kvh = blockIdx.y, z = blockIdx.z;
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int c = lane & 15, g = lane >> 4;
     const int pos = tok_pos[b];
     const int n_pages = pos / kPageTokens + 1;
-    if (z * kAttnWaves >= n_pages) return;                       // nothing of this sequence here
-    const int page_idx = z * kAttnWaves + wave;
+    if (z * WAVES >= n_pages) return;                            // nothing of this sequence here
+    const int page_idx = z * WAVES + wave;
 
     WaveState<HD> st;
     st.init();
@@ -240,39 +248,48 @@ __global__ __launch_bounds__(kAttnWaves * kWave) void attn_decode_kernel(
                         min(kPageTokens, pos - key0 + 1), page_fully_visible(pos, pos, key0, window, sinks),
                         scale * kLog2e, window, sinks);
     }
-    // merge the four waves
-    if (g == 0) { lds_m[wave][c] = st.m; lds_l[wave][c] = st.l; }
+    // merge the waves
+    if (g == 0) { lds_m[wave * 16 + c] = st.m; lds_l[wave * 16 + c] = st.l; }
+    if (c < group) {
+        float* dst = lds_o + ((size_t)wave * group + c) * (HD + 1);
 #pragma unroll
-    for (int db = 0; db < HD / 16; ++db)
+        for (int db = 0; db < HD / 16; ++db)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) lds_o[wave][c][16 * db + 4 * g + r] = st.acc[db][r];
+            for (int r = 0; r < 4; ++r) dst[16 * db + 4 * g + r] = st.acc[db][r];
+    }
     __syncthreads();
     const int n_z = gridDim.z;
     for (int idx = threadIdx.x; idx < group * HD; idx += blockDim.x) {
         const int col = idx / HD, d = idx % HD;
         float m = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < kAttnWaves; ++w) m = fmaxf(m, lds_m[w][col]);
+        for (int w = 0; w < WAVES; ++w) m = fmaxf(m, lds_m[w * 16 + col]);
         float l = 0.f, o = 0.f;
 #pragma unroll
-        for (int w = 0; w < kAttnWaves; ++w) {
-            const float f = (lds_m[w][col] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(lds_m[w][col] - m);
-            l += lds_l[w][col] * f;
-            o += lds_o[w][col][d] * f;
+        for (int w = 0; w < WAVES; ++w) {
+            const float mw = lds_m[w * 16 + col];
+            const float f = (mw == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw - m);
+            l += lds_l[w * 16 + col] * f;
+            o += lds_o[((size_t)w * group + col) * (HD + 1) + d] * f;
         }
-        float* dst = partial + (((size_t)b * n_heads + kvh * group + col) * n_z + z) * (HD + 2);
-        dst[2 + d] = o;
-        if (d == 0) { dst[0] = m; dst[1] = l; }
+        if (n_z == 1) {
+            out[((size_t)b * n_heads + kvh * group + col) * HD + d] = f32_to_bf16(l > 0.f ? o / l : 0.f);
+        } else {
+            float* dst = partial + (((size_t)b * n_heads + kvh * group + col) * n_z + z) * (HD + 2);
+            dst[2 + d] = o;
+            if (d == 0) { dst[0] = m; dst[1] = l; }
+        }
     }
 }
 
-// grid (batch, heads); HD threads.  Adds the partial results of the blocks along the context.
+// grid (batch, heads); HD threads.  Adds the partial results of the blocks along the context,
+// each of which covered pages_per_block pages.
 template <int HD>
 __global__ void attn_decode_merge_kernel(bf16_t* __restrict__ out, const float* __restrict__ partial,
-                                         const int* __restrict__ tok_pos, int n_heads, int n_z) {
+                                         const int* __restrict__ tok_pos, int n_heads, int n_z, int pages_per_block) {
     const int b = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
     const int n_pages = tok_pos[b] / kPageTokens + 1;
-    const int used = min(n_z, (n_pages + kAttnWaves - 1) / kAttnWaves);
+    const int used = min(n_z, (n_pages + pages_per_block - 1) / pages_per_block);
     const float* src = partial + ((size_t)b * n_heads + h) * n_z * (HD + 2);
     float m = -INFINITY;
     for (int z = 0; z < used; ++z) m = fmaxf(m, src[(size_t)z * (HD + 2)]);
@@ -571,10 +588,25 @@ static bool mfma_shape_ok(int n_heads, int n_kv_heads, int head_dim) {
     return (head_dim == 64 || head_dim == 128) && n_heads / n_kv_heads <= 16;
 }
 
+// Waves (= pages) per block of the decode kernel.  A block's pages all come through one CU's
+// vector memory path, so few large blocks are slower than many small ones: blocks grow only
+// while there are enough of them for every CU (then the merge kernel falls away for contexts
+// of up to 1,024 positions), within the LDS that the waves' outputs need.
+static int decode_waves(int group, int table_width, int sequences_x_kv_heads) {
+    int waves = group <= 4 ? 16 : (group <= 8 ? 8 : 4);
+    while (waves > 4 && (waves / 2 >= table_width ||
+                         (long long)sequences_x_kv_heads * ((table_width + waves - 1) / waves) < 256))
+        waves /= 2;
+    return waves;
+}
+
 // floats the decode workspace needs
-LLOGOS_EXPORT long long llogos_attn_decode_workspace(int batch, int n_heads, int head_dim, int table_width) {
-    const int n_z = (table_width + kAttnWaves - 1) / kAttnWaves;
-    return (long long)batch * n_heads * n_z * (head_dim + 2);
+LLOGOS_EXPORT long long llogos_attn_decode_workspace(int batch, int n_heads, int n_kv_heads, int head_dim,
+                                                     int table_width) {
+    if (n_kv_heads <= 0 || n_heads % n_kv_heads) return 0;
+    const int waves = decode_waves(n_heads / n_kv_heads, table_width, batch * n_kv_heads);
+    const int n_z = (table_width + waves - 1) / waves;
+    return n_z == 1 ? 0 : (long long)batch * n_heads * n_z * (head_dim + 2);
 }
 
 LLOGOS_EXPORT int llogos_attn_decode_bf16(void* out, const void* q, int q_stride, const void* k_pool,
@@ -584,16 +616,23 @@ LLOGOS_EXPORT int llogos_attn_decode_bf16(void* out, const void* q, int q_stride
                                           long long workspace_floats, hipStream_t stream) {
     if (batch <= 0 || table_width <= 0 || window < 0 || sinks < 0) return LLOGOS_BAD_ARGUMENT;
     if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || (q_stride % 8) || ((uintptr_t)q % 16)) return LLOGOS_UNSUPPORTED;
-    if (workspace_floats < llogos_attn_decode_workspace(batch, n_heads, head_dim, table_width)) return LLOGOS_BAD_ARGUMENT;
-    const int n_z = (table_width + kAttnWaves - 1) / kAttnWaves;
+    if (workspace_floats < llogos_attn_decode_workspace(batch, n_heads, n_kv_heads, head_dim, table_width))
+        return LLOGOS_BAD_ARGUMENT;
     const int group = n_heads / n_kv_heads;
+    const int waves = decode_waves(group, table_width, batch * n_kv_heads);
+    const int n_z = (table_width + waves - 1) / waves;
+    if (n_z > 1 && workspace == nullptr) return LLOGOS_BAD_ARGUMENT;
     dim3 grid(batch, n_kv_heads, n_z), mgrid(batch, n_heads);
-#define GO(HD) \
-    attn_decode_kernel<HD><<<grid, kAttnWaves * kWave, 0, stream>>>( \
-        workspace, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride, \
-        tok_pos, n_heads, n_kv_heads, group, scale, window, sinks); \
-    attn_decode_merge_kernel<HD><<<mgrid, HD, 0, stream>>>((bf16_t*)out, workspace, tok_pos, n_heads, n_z)
-    if (head_dim == 64) { GO(64); } else { GO(128); }
+    const size_t smem = decode_lds_bytes(waves, group, head_dim);
+#define GO(HD, W) do { \
+    attn_decode_kernel<HD, W><<<grid, W * kWave, smem, stream>>>( \
+        (bf16_t*)out, workspace, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, \
+        table_stride, tok_pos, n_heads, n_kv_heads, group, scale, window, sinks); \
+    if (n_z > 1) attn_decode_merge_kernel<HD><<<mgrid, HD, 0, stream>>>((bf16_t*)out, workspace, tok_pos, n_heads, \
+                                                                        n_z, W); } while (0)
+#define BY_WAVES(HD) do { if (waves == 16) GO(HD, 16); else if (waves == 8) GO(HD, 8); else GO(HD, 4); } while (0)
+    if (head_dim == 64) BY_WAVES(64); else BY_WAVES(128);
+#undef BY_WAVES
 #undef GO
     return LLOGOS_LAUNCH_CHECK();
 }

@@ -499,7 +499,7 @@ def attention_mfma_bf16(ctx, q: torch.Tensor, q_stride: int, k_pool: torch.Tenso
     lib = _lib()
     if ctx.is_decode:
         width = table.shape[1]
-        floats = lib.llogos_attn_decode_workspace(T, n_heads, head_dim, width)
+        floats = lib.llogos_attn_decode_workspace(T, n_heads, n_kv_heads, head_dim, width)
         ws = _attn_workspace(q.device, floats)
         code = lib.llogos_attn_decode_bf16(
             _p(out), _p(q), q_stride, _p(k_pool), _p(v_pool), _p(table), table.stride(0), width, _p(ctx.tok_pos),

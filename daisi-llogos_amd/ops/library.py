@@ -181,6 +181,7 @@ def load() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except OSError as e:
         raise KernelLibraryError(f"cannot load {path}: {e}") from e
+    lib.llogos_attn_decode_workspace.restype = ctypes.c_longlong       # every other entry returns an int code
     with _lock:
         _lib = lib
     return lib

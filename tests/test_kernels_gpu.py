@@ -243,6 +243,32 @@ def test_attention_whole_prompts_and_single_tokens(dtype, nh, nkv, hd):
         _close(out, _plain_attention(c, nh, nkv, hd), dtype)
 
 
+@pytest.mark.parametrize("nh,nkv,hd,batch,longest", [(8, 4, 128, 64, 700),      # 16 pages a block, no merge
+                                                     (8, 4, 64, 70, 1500),       # 16 pages a block, merged
+                                                     (16, 2, 64, 128, 700),      # 8 pages a block, merged
+                                                     (8, 4, 128, 3, 1500)])      # 4 pages a block
+def test_single_token_attention_with_blocks_of_every_size(nh, nkv, hd, batch, longest):
+    """The decode kernel gives a block more pages when there are many blocks; every form must
+    agree with the plain attention, whatever the lengths of the other sequences."""
+    rng = np.random.default_rng(batch)
+    lens = [int(x) for x in rng.integers(1, longest // 3, batch)]
+    lens[1], lens[batch // 2], lens[-1] = longest, 64, 65
+    new = [1] * batch
+    c = _attention_case("bfloat16", nh, nkv, hd, lens, new, seed=batch)
+    for b, l in enumerate(lens):                                        # unwritten page tails must not matter
+        if l % 64:
+            page = int(c["table"][b, l // 64])
+            c["kp"][page, :, l % 64:, :] = float("nan")
+            c["vp"][page, :, :, l % 64:] = float("nan")
+    ctx = type("Ctx", (), dict(tok_seq=_t(c["tok_seq"], torch.int32), tok_pos=_t(c["tok_pos"], torch.int32),
+                               is_decode=True, max_context=max(lens), batch=batch, n_tokens=batch,
+                               cu_seqlens=list(range(batch + 1)), cu_dev=None, starts=[l - 1 for l in lens],
+                               shared={}))()
+    out = K.attention_mfma_bf16(ctx, c["q"], c["stride"], c["kp"], c["vp"], c["table"], nh, nkv, hd, 1 / math.sqrt(hd))
+    assert out is not None
+    _close(out, _plain_attention(c, nh, nkv, hd), "bfloat16")
+
+
 @pytest.mark.parametrize("tile_rows", [64, 128])
 @pytest.mark.parametrize("nh,nkv,hd", [(6, 2, 64), (8, 2, 128), (3, 3, 128)])
 @pytest.mark.parametrize("window,sinks", [(0, 0), (100, 0), (70, 5)])
