@@ -367,7 +367,8 @@ __global__ __launch_bounds__(kAttnWaves * kWave) void attn_prefill_kernel(
 }
 
 // ---------------------------------------------------------------- prefill, pages shared through LDS
-// grid (tiles of 128 tokens over all sequences, heads); the 4 waves of a block take 32 rows
+// grid: one block per (tile of 128 tokens over all sequences, head), in the order given in the
+// kernel; the 4 waves of a block take 32 rows
 // each (two blocks of 16 columns) and walk the same pages: a page's keys and transposed
 // values are copied to LDS once per block (two buffers, the copy of the next page is in
 // flight while the current one is used), and every key fragment a wave reads serves both of
@@ -384,11 +385,11 @@ struct PageLds {
     bf16_t v[HD][kPageTokens + kVPad];
 };
 
-// the tile's queries, kept in LDS so that their fragments need no registers between pages
+// two page buffers: 2 * 35.8 KB for head size 128, so that two blocks share a compute unit and
+// one block's LDS and MFMA latencies are covered by the other
 template <int HD>
 struct TileLds {
     PageLds<HD> page[2];
-    bf16_t q[kTileRows][HD + kKPad];
 };
 
 template <int HD, int N>
@@ -413,17 +414,26 @@ __device__ __forceinline__ void stash_page(PageLds<HD>& pg, const uint4 (&kreg)[
 }
 
 template <int HD>
-__global__ __launch_bounds__(kAttnWaves * kWave) __attribute__((amdgpu_waves_per_eu(1, 1)))
+__global__ __launch_bounds__(kAttnWaves * kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attn_prefill_lds_kernel(
         bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int q_stride,
         const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
         const int* __restrict__ table, int table_stride, const int* __restrict__ cu,
-        const int* __restrict__ tok_pos, int batch, int n_heads, int n_kv_heads, int group,
+        const int* __restrict__ tok_pos, int batch, int n_tiles, int n_heads, int n_kv_heads, int group,
         float scale, int window, int sinks) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     TileLds<HD>& tl = *reinterpret_cast<TileLds<HD>*>(smem_raw);
     PageLds<HD>* lds = tl.page;                                       // two buffers
-    int tile = blockIdx.x, b = 0, first = 0;
+    // Blocks start in the order of their index, round-robin over the 8 XCDs.  Block L is the
+    // m-th block of XCD x (L = 8 m + x); an XCD takes the `group` query heads of one (tile, kv
+    // head) pair one after the other, so that the pair's pages stay in its L2, and the pairs go
+    // from the last tile to the first: late tiles of a causal prompt see the most keys, and
+    // starting with them keeps the compute units evenly busy to the end.
+    const int m_xcd = blockIdx.x / 8, xcd = blockIdx.x % 8;
+    const int pair = (m_xcd / group) * 8 + xcd;
+    if (pair >= n_tiles * n_kv_heads) return;
+    const int kvh = pair % n_kv_heads, h = kvh * group + m_xcd % group;
+    int tile = n_tiles - 1 - pair / n_kv_heads, b = 0, first = 0;
     for (; b < batch; ++b) {
         const int len = cu[b + 1] - cu[b];
         const int tiles = (len + kTileRows - 1) / kTileRows;
@@ -431,7 +441,6 @@ void attn_prefill_lds_kernel(
         tile -= tiles;
     }
     if (b >= batch) return;
-    const int h = blockIdx.y, kvh = h / group;
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int c = lane & 15, g = lane >> 4;
     const int seq_end = cu[b + 1];
@@ -444,12 +453,16 @@ void attn_prefill_lds_kernel(
     const int wave_rows = max(0, min(32, seq_end - row0));
     const bool ok0 = c < wave_rows, ok1 = 16 + c < wave_rows;
     const int q_pos0 = ok0 ? tok_pos[row0 + c] : -1, q_pos1 = ok1 ? tok_pos[row0 + 16 + c] : -1;
-    // the wave's 32 query rows go to LDS (rows past the sequence as zeros)
-    for (int piece = lane; piece < 32 * (HD / 8); piece += kWave) {
-        const int rr = piece / (HD / 8), col = (piece % (HD / 8)) * 8;
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (rr < wave_rows) v = *reinterpret_cast<const uint4*>(q + (size_t)(row0 + rr) * q_stride + (size_t)h * HD + col);
-        *reinterpret_cast<uint4*>(&tl.q[32 * wave + rr][col]) = v;
+    // the wave's 32 query rows as second operands (rows past the sequence as zeros)
+    bf16x8 qf0[HD / 32], qf1[HD / 32];
+    {
+        const bf16_t* qrow0 = q + (size_t)(row0 + (ok0 ? c : 0)) * q_stride + (size_t)h * HD + 8 * g;
+        const bf16_t* qrow1 = q + (size_t)(row0 + (ok1 ? 16 + c : 0)) * q_stride + (size_t)h * HD + 8 * g;
+#pragma unroll
+        for (int sk = 0; sk < HD / 32; ++sk) {
+            qf0[sk] = ok0 ? ld_frag(qrow0 + 32 * sk) : zero_frag();
+            qf1[sk] = ok1 ? ld_frag(qrow1 + 32 * sk) : zero_frag();
+        }
     }
     WaveState<HD> st0, st1;
     st0.init();
@@ -509,13 +522,11 @@ void attn_prefill_lds_kernel(
         }
 #pragma unroll
         for (int sk = 0; sk < HD / 32; ++sk) {
-            const bf16x8 qf0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&tl.q[32 * wave + c][32 * sk + 8 * g]));
-            const bf16x8 qf1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&tl.q[32 * wave + 16 + c][32 * sk + 8 * g]));
 #pragma unroll
             for (int rb = 0; rb < 4; ++rb) {
                 const bf16x8 kf = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&pg.k[16 * rb + c][32 * sk + 8 * g]));
-                s0[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf0, s0[rb], 0, 0, 0);
-                s1[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf1, s1[rb], 0, 0, 0);
+                s0[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf0[sk], s0[rb], 0, 0, 0);
+                s1[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf1[sk], s1[rb], 0, 0, 0);
             }
         }
         // lane (c, g) of block cb: column c, keys key0 + 16 rb + 4 g + r; step t of the value
@@ -650,14 +661,16 @@ LLOGOS_EXPORT int llogos_attn_prefill_bf16(void* out, const void* q, int q_strid
     const int group = n_heads / n_kv_heads;
     dim3 grid(n_tiles, n_heads);
     if (tile_rows == kTileRows) {
+        const long long pairs = (long long)n_tiles * n_kv_heads;
+        const dim3 lgrid((unsigned)((pairs + 7) / 8 * 8 * group));
 #define GOL(HD) do { \
         const size_t smem = sizeof(TileLds<HD>); \
         hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<HD>, \
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
         if (e != hipSuccess) return (int)e; \
-        attn_prefill_lds_kernel<HD><<<grid, kAttnWaves * kWave, smem, stream>>>( \
+        attn_prefill_lds_kernel<HD><<<lgrid, kAttnWaves * kWave, smem, stream>>>( \
             (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride, \
-            cu, tok_pos, batch, n_heads, n_kv_heads, group, scale, window, sinks); } while (0)
+            cu, tok_pos, batch, n_tiles, n_heads, n_kv_heads, group, scale, window, sinks); } while (0)
         if (head_dim == 64) GOL(64); else GOL(128);
 #undef GOL
         return LLOGOS_LAUNCH_CHECK();

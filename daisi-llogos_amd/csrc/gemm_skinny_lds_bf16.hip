@@ -20,7 +20,8 @@
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kChunkK = 256;                 // values of k per LDS chunk
+constexpr int kLdsWaves = 4;                 // waves per block (8 measured no faster)
+constexpr int kChunkK = 256;                 // values of k per LDS chunk (128 and 512 measured no faster)
 constexpr int kChunkSteps = kChunkK / 32;    // MFMA steps per chunk
 constexpr int kRowPad = 8;                   // bf16 of padding per LDS row (16 bytes)
 
@@ -75,7 +76,7 @@ __device__ __forceinline__ uint4 produce8(const ActSource& src, int m, int k, in
     }
 }
 
-template <int RB, int MB, int MODE, int kLdsWaves, typename TO>
+template <int RB, int MB, int MODE, typename TO>
 __global__ __launch_bounds__(kLdsWaves * kWave) void gemm_skinny_lds_kernel(
         TO* __restrict__ out, ActSource src, const bf16_t* __restrict__ w, const float* __restrict__ bias,
         int M, int N, int K, int ldo, size_t part_stride, int k_per_block) {
@@ -196,43 +197,31 @@ LLOGOS_EXPORT int llogos_gemm_skinny_lds_parts(int K, int splits) {
     return (K + kpb - 1) / kpb;
 }
 
-template <int RB, int MB, int MODE, int kLdsWaves>
-static int launch_lds_w(void* out, int out_dtype, const ActSource& src, const bf16_t* w, const float* bias,
-                        int M, int N, int K, int ldo, size_t part_stride, int kpb, int parts, hipStream_t stream) {
-    dim3 grid((N + 16 * RB * kLdsWaves - 1) / (16 * RB * kLdsWaves), parts);
-    if (out_dtype == DT_BF16)
-        gemm_skinny_lds_kernel<RB, MB, MODE, kLdsWaves, bf16_t><<<grid, kLdsWaves * kWave, 0, stream>>>(
-            (bf16_t*)out, src, w, bias, M, N, K, ldo, part_stride, kpb);
-    else
-        gemm_skinny_lds_kernel<RB, MB, MODE, kLdsWaves, float><<<grid, kLdsWaves * kWave, 0, stream>>>(
-            (float*)out, src, w, bias, M, N, K, ldo, part_stride, kpb);
-    return LLOGOS_LAUNCH_CHECK();
-}
-
-// waves per block: 4, or 8 when many rows of activations are staged (their copy is then
-// shared by twice as many rows of w)
 template <int RB, int MB, int MODE>
 static int launch_lds(void* out, int out_dtype, const ActSource& src, const bf16_t* w, const float* bias,
-                      int M, int N, int K, int ldo, size_t part_stride, int kpb, int parts, int waves,
-                      hipStream_t stream) {
-    if (waves == 8)
-        return launch_lds_w<RB, MB, MODE, 8>(out, out_dtype, src, w, bias, M, N, K, ldo, part_stride, kpb, parts, stream);
-    return launch_lds_w<RB, MB, MODE, 4>(out, out_dtype, src, w, bias, M, N, K, ldo, part_stride, kpb, parts, stream);
+                      int M, int N, int K, int ldo, size_t part_stride, int kpb, int parts, hipStream_t stream) {
+    dim3 grid((N + 16 * RB * kLdsWaves - 1) / (16 * RB * kLdsWaves), parts);
+    if (out_dtype == DT_BF16)
+        gemm_skinny_lds_kernel<RB, MB, MODE, bf16_t><<<grid, kLdsWaves * kWave, 0, stream>>>(
+            (bf16_t*)out, src, w, bias, M, N, K, ldo, part_stride, kpb);
+    else
+        gemm_skinny_lds_kernel<RB, MB, MODE, float><<<grid, kLdsWaves * kWave, 0, stream>>>(
+            (float*)out, src, w, bias, M, N, K, ldo, part_stride, kpb);
+    return LLOGOS_LAUNCH_CHECK();
 }
 
 // act: plain bf16 activations [M][lda] (mode 0), or the fused gate/up product [act_parts][M][2 K]
 // in float32 (mode 1) or bfloat16 (mode 2, act_parts = 1) from which silu(gate) * up is made on
 // the way.  out: [parts][M][ldo], parts = llogos_gemm_skinny_lds_parts(K, splits); float32 and
-// without bias when parts > 1.  row_blocks: 16-row blocks of w per wave (1 or 2); waves: 4 or 8
-// per block.
+// without bias when parts > 1.  row_blocks: 16-row blocks of w per wave (1 or 2).
 LLOGOS_EXPORT int llogos_gemm_skinny_lds_bf16(void* out, int out_dtype, const void* act, int mode, int lda,
                                               int act_parts, long long act_part_stride, const void* w,
                                               const float* bias, int M, int N, int K, int ldo,
-                                              long long part_stride, int splits, int row_blocks, int waves,
+                                              long long part_stride, int splits, int row_blocks,
                                               hipStream_t stream) {
     if (M <= 0 || N <= 0 || K <= 0 || ldo < N || splits < 1 || act_parts < 1) return LLOGOS_BAD_ARGUMENT;
     if (out_dtype != DT_BF16 && out_dtype != DT_F32) return LLOGOS_BAD_ARGUMENT;
-    if (mode < PRODUCE_PLAIN || mode > PRODUCE_SWIGLU_BF16 || (waves != 4 && waves != 8)) return LLOGOS_BAD_ARGUMENT;
+    if (mode < PRODUCE_PLAIN || mode > PRODUCE_SWIGLU_BF16) return LLOGOS_BAD_ARGUMENT;
     if (M > 64 || (K % 8) || (lda % 8) || ((uintptr_t)act % 16) || ((uintptr_t)w % 16) || (act_part_stride % 4))
         return LLOGOS_UNSUPPORTED;
     if (mode == PRODUCE_PLAIN ? lda < K : lda < 2 * K) return LLOGOS_BAD_ARGUMENT;
@@ -244,7 +233,7 @@ LLOGOS_EXPORT int llogos_gemm_skinny_lds_bf16(void* out, int out_dtype, const vo
     const bf16_t* W = (const bf16_t*)w;
     const int mb = (M + 15) / 16;
 #define GO(RB, MB, MODE) return launch_lds<RB, MB, MODE>(out, out_dtype, src, W, bias, M, N, K, ldo, \
-                                                         (size_t)part_stride, kpb, parts, waves, stream)
+                                                         (size_t)part_stride, kpb, parts, stream)
 #define BY_MODE(RB, MB) do { if (mode == PRODUCE_PLAIN) GO(RB, MB, PRODUCE_PLAIN); \
                              if (mode == PRODUCE_SWIGLU_F32) GO(RB, MB, PRODUCE_SWIGLU_F32); \
                              GO(RB, MB, PRODUCE_SWIGLU_BF16); } while (0)

@@ -341,8 +341,7 @@ def gemm_skinny_stationary_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional
 
 
 def gemm_skinny_lds_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype,
-                         splits: int = 1, row_blocks: int = 1, swiglu: bool = False,
-                         waves: int = 0) -> Optional[torch.Tensor]:
+                         splits: int = 1, row_blocks: int = 1, swiglu: bool = False) -> Optional[torch.Tensor]:
     """The few-row bfloat16 product with the activations shared through LDS: [parts, M, N].
     With `swiglu`, `a` is the fused gate/up product ([M, 2 K] bfloat16 or float32 partial sums
     [parts, M, 2 K]) and silu(gate) * up is made on the way.  None for shapes it does not take."""
@@ -380,8 +379,7 @@ def gemm_skinny_lds_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.
     out = torch.empty((parts, M, N), dtype=out_dtype, device=a.device)
     code = lib.llogos_gemm_skinny_lds_bf16(
         _p(out), _DT[out_dtype], _p(a), mode, lda, a_parts, ctypes.c_longlong(a_stride), _p(w), _p(bias),
-        M, N, K, N, ctypes.c_longlong(M * N), int(splits), int(row_blocks),
-        int(waves) or 4, _stream())
+        M, N, K, N, ctypes.c_longlong(M * N), int(splits), int(row_blocks), _stream())
     if code == -2:
         return None
     _check(code, "gemm_skinny_lds_bf16")
