@@ -45,6 +45,25 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 
 constexpr float kLog2e = 1.4426950408889634f;
 
+// Maximum and sum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (one column of an MFMA result),
+// left in all four.  v_permlane16_swap exchanges the odd rows of 16 lanes of its first operand
+// with the even rows of its second, v_permlane32_swap the upper half of the first with the
+// lower half of the second: fed the same value twice, the two results hold a lane's own value
+// and its partner's.  (A shuffle would go through the LDS pipeline and cost its latency.)
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float quad_max(float x) {
+    u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float quad_sum(float x) {
+    u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // Keeps the first n (0..8) of a fragment's eight values and zeroes the rest.
 __device__ __forceinline__ bf16x8 keep_first(bf16x8 f, int n) {
     uint4 u = __builtin_bit_cast(uint4, f);
@@ -93,8 +112,7 @@ __device__ __forceinline__ void softmax_page(f32x4 (&s)[4], WaveState<HD>& st, f
             }
             tile_max = fmaxf(tile_max, s[rb][r]);
         }
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, kWave));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, kWave));
+    tile_max = quad_max(tile_max);
     const float m_new = fmaxf(st.m, tile_max * scale_log2);              // scale > 0: the maximum commutes
     // a column that has seen no key yet keeps m = -inf; exp2(-inf - (-inf)) must not be taken
     const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
@@ -108,8 +126,7 @@ __device__ __forceinline__ void softmax_page(f32x4 (&s)[4], WaveState<HD>& st, f
             p[4 * rb + r] = e;
             sum += e;
         }
-    sum += __shfl_xor(sum, 16, kWave);
-    sum += __shfl_xor(sum, 32, kWave);
+    sum = quad_sum(sum);
     st.l = st.l * corr + sum;
     st.m = m_new;
 #pragma unroll
@@ -403,13 +420,20 @@ __device__ __forceinline__ void fetch_page(uint4 (&kreg)[N], uint4 (&vreg)[N], c
     }
 }
 
+// valid_keys: how many of the page's tokens have been written; the values of the others go to
+// LDS as zeros (their probabilities are zero, and 0 * NaN would be NaN).
 template <int HD, int N>
-__device__ __forceinline__ void stash_page(PageLds<HD>& pg, const uint4 (&kreg)[N], const uint4 (&vreg)[N]) {
+__device__ __forceinline__ void stash_page(PageLds<HD>& pg, const uint4 (&kreg)[N], const uint4 (&vreg)[N],
+                                           int valid_keys) {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
         const int piece = i * (kAttnWaves * kWave) + threadIdx.x;
         *reinterpret_cast<uint4*>(&pg.k[piece / (HD / 8)][(piece % (HD / 8)) * 8]) = kreg[i];
-        *reinterpret_cast<uint4*>(&pg.v[piece / (kPageTokens / 8)][(piece % (kPageTokens / 8)) * 8]) = vreg[i];
+        const int tok0 = (piece % (kPageTokens / 8)) * 8;
+        uint4 v = vreg[i];
+        if (valid_keys < kPageTokens)
+            v = __builtin_bit_cast(uint4, keep_first(__builtin_bit_cast(bf16x8, v), valid_keys - tok0));
+        *reinterpret_cast<uint4*>(&pg.v[piece / (kPageTokens / 8)][tok0]) = v;
     }
 }
 
@@ -495,7 +519,7 @@ void attn_prefill_lds_kernel(
     {
         const size_t base = page_base(cur_id);
         fetch_page<HD, kPerThread>(kreg, vreg, k_pool + base, v_pool + base);
-        stash_page<HD, kPerThread>(lds[0], kreg, vreg);
+        stash_page<HD, kPerThread>(lds[0], kreg, vreg, min(kPageTokens, written - cur * kPageTokens));
     }
     __syncthreads();
     int buf = 0;
@@ -511,7 +535,6 @@ void attn_prefill_lds_kernel(
         const int key0 = pi * kPageTokens;
         if (wave_rows <= 0 || key0 > wave_last_pos) break;                // nothing of this page for this wave
         if (!page_may_be_visible_to_range(wave_first_pos, wave_last_pos, key0, window, sinks)) break;
-        const int valid_keys = min(kPageTokens, written - key0);
         const PageLds<HD>& pg = lds[buf];
         // S^T for both column blocks; operand row c of block rb is key 16 rb + c
         f32x4 s0[4], s1[4];
@@ -529,9 +552,19 @@ void attn_prefill_lds_kernel(
                 s1[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf1[sk], s1[rb], 0, 0, 0);
             }
         }
+        // the value fragments are read now, so that their way from LDS is covered by the softmax.
         // lane (c, g) of block cb: column c, keys key0 + 16 rb + 4 g + r; step t of the value
         // product covers blocks 2 t and 2 t + 1: slots 0..3 keys 32 t + 4 g + e, slots 4..7 keys
         // 32 t + 16 + 4 g + e
+        auto read_v = [&](int db, int t) {
+            const bf16_t* vrow = &pg.v[16 * db + c][32 * t + 4 * g];
+            const uint2 lo = *reinterpret_cast<const uint2*>(vrow), hi = *reinterpret_cast<const uint2*>(vrow + 16);
+            return __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
+        };
+        constexpr int kEarly = 2;                                         // the others two steps ahead of their use
+        bf16x8 vf[HD / 16][2];
+#pragma unroll
+        for (int db = 0; db < kEarly; ++db) { vf[db][0] = read_v(db, 0); vf[db][1] = read_v(db, 1); }
         bf16x8 pf0[2], pf1[2];
         float corr0, corr1;
         const bool all_visible = wave_rows == 32 &&
@@ -544,8 +577,13 @@ void attn_prefill_lds_kernel(
             softmax_page<true, 4, 16, HD>(s1, st1, scale_log2, q_pos1, key0, window, sinks, pf1, corr1);
         }
         const bool rescale = __ballot(corr0 != 1.0f || corr1 != 1.0f) != 0;
+        __builtin_amdgcn_sched_barrier(0);                                // the late reads stay behind the softmax
 #pragma unroll
         for (int db = 0; db < HD / 16; ++db) {
+            if (db + kEarly < HD / 16) {
+                vf[db + kEarly][0] = read_v(db + kEarly, 0);
+                vf[db + kEarly][1] = read_v(db + kEarly, 1);
+            }
             f32x4 a0 = st0.acc[db], a1 = st1.acc[db];
             if (rescale) {
 #pragma unroll
@@ -553,24 +591,14 @@ void attn_prefill_lds_kernel(
             }
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
-                const bf16_t* vrow = &pg.v[16 * db + c][32 * t + 4 * g];
-                uint2 lo = *reinterpret_cast<const uint2*>(vrow), hi = *reinterpret_cast<const uint2*>(vrow + 16);
-                if (valid_keys < kPageTokens) {                           // zero the tokens that were never written
-                    const int n_lo = valid_keys - (32 * t + 4 * g), n_hi = n_lo - 16;
-                    lo.x &= (1 < n_lo) ? 0xffffffffu : ((0 < n_lo) ? 0x0000ffffu : 0u);
-                    lo.y &= (3 < n_lo) ? 0xffffffffu : ((2 < n_lo) ? 0x0000ffffu : 0u);
-                    hi.x &= (1 < n_hi) ? 0xffffffffu : ((0 < n_hi) ? 0x0000ffffu : 0u);
-                    hi.y &= (3 < n_hi) ? 0xffffffffu : ((2 < n_hi) ? 0x0000ffffu : 0u);
-                }
-                const bf16x8 vf = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
-                a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf0[t], a0, 0, 0, 0);
-                a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf1[t], a1, 0, 0, 0);
+                a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[db][t], pf0[t], a0, 0, 0, 0);
+                a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[db][t], pf1[t], a1, 0, 0, 0);
             }
             st0.acc[db] = a0;
             st1.acc[db] = a1;
         }
         } while (0);
-        stash_page<HD, kPerThread>(lds[buf ^ 1], kreg, vreg);
+        stash_page<HD, kPerThread>(lds[buf ^ 1], kreg, vreg, min(kPageTokens, written - min(nxt, n_pages - 1) * kPageTokens));
         __syncthreads();
         cur = nxt;
         nxt = nxt2;
