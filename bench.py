@@ -71,6 +71,7 @@ def main(argv=None) -> int:
     import torch
     llogos = importlib.import_module("daisi-llogos_amd")
     K = importlib.import_module("daisi-llogos_amd.ops.kernels")
+    fetch_tokens = importlib.import_module("daisi-llogos_amd.engine.generate").fetch_tokens
 
     cfg = dict(LLAMA31_8B)
     full_layers = cfg["num_hidden_layers"]
@@ -90,13 +91,20 @@ def main(argv=None) -> int:
         slots = [eng.alloc_slot() for _ in range(batch)]
         prompts = [rng.integers(0, cfg["vocab_size"], size=PROMPT).tolist() for _ in range(batch)]
         logits = eng.step(list(zip(slots, prompts)), want="last")
-        ids = K.argmax(logits).tolist()
+        ids = K.argmax(logits)
+        rows = list(range(batch))
+        placeholders = [(s, [0]) for s in slots]
 
         def run(n):
+            """Greedy single-token steps as the generation loop runs them: a step takes its
+            tokens from the device memory the last argmax wrote, and the host reads the last
+            step's tokens while this one runs."""
             nonlocal ids
             for _ in range(n):
-                logits = eng.step([(s, [t]) for s, t in zip(slots, ids)], want="last")
-                ids = K.argmax(logits).tolist()       # the tokens come to the host every step, as in generation
+                tokens = fetch_tokens(ids)
+                logits = eng.step(placeholders, want="last", device_ids=(ids, rows))
+                ids = K.argmax(logits)
+                tokens()
         run(warmup)
         torch.cuda.synchronize()
         t = time.perf_counter()

@@ -28,6 +28,23 @@ LLOGOS_EXPORT int llogos_embed(float* out, const void* table, int table_dtype, c
     return LLOGOS_LAUNCH_CHECK();
 }
 
+// dst[i] = src[rows[i]] for int32 values: a step's token ids picked from the ids another
+// step's sampler left on the device.  rows outside 0..n_src-1 give 0.
+__global__ void gather_i32_kernel(int* __restrict__ dst, const int* __restrict__ src,
+                                  const int* __restrict__ rows, int n, int n_src) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int r = rows[i];
+    dst[i] = (r >= 0 && r < n_src) ? src[r] : 0;
+}
+
+LLOGOS_EXPORT int llogos_gather_i32(int* dst, const int* src, const int* rows, int n, int n_src,
+                                    hipStream_t stream) {
+    if (n <= 0 || n_src <= 0) return LLOGOS_BAD_ARGUMENT;
+    gather_i32_kernel<<<(n + 255) / 256, 256, 0, stream>>>(dst, src, rows, n, n_src);
+    return LLOGOS_LAUNCH_CHECK();
+}
+
 // ---------------------------------------------------------------- RMSNorm (+ residual add)
 // For output row r (source row s = rows ? rows[r] : r):
 //   v = x[s] + delta[s]   (delta optional; written back to x when write_back)

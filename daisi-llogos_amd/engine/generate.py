@@ -63,10 +63,12 @@ class Generator:
     """Drives an engine (anything with alloc_slot, free_slot, step and cache.n_pages) and a
     sampler (anything with sample(logits, requests, indices, histories) -> ids)."""
 
-    def __init__(self, engine, max_batch: int = 64, synchronize: Optional[Callable[[], None]] = None):
+    def __init__(self, engine, max_batch: int = 64, synchronize: Optional[Callable[[], None]] = None,
+                 look_ahead: bool = True):
         self.engine = engine
         self.max_batch = max_batch
         self._sync = synchronize or (lambda: None)
+        self.look_ahead = look_ahead              # start a step before the host has seen the last one's tokens
 
     def stop_tokens(self, params: GenerationParams) -> Tuple[int, ...]:
         if params.stop_tokens is not None:
@@ -91,43 +93,102 @@ class Generator:
     def _run_batch(self, batch, prompts, params, sampler, stops, result, on_token) -> None:
         eng = self.engine
         slots = {r: eng.alloc_slot() for r in batch}
-        live = list(batch)
-        need_history = params.has_penalties
         try:
             if params.max_tokens == 0:
                 return
-            self._sync()
-            t0 = time.perf_counter()
-            logits = eng.step([(slots[r], prompts[r]) for r in live], want="last")
-            ids = self._sample(sampler, logits, live, prompts, result, need_history)
-            t1 = time.perf_counter()
-            result.prefill_seconds += t1 - t0
-            result.prompt_tokens += sum(len(prompts[r]) for r in live)
-            while True:
-                nxt = []
-                for r, tok in zip(live, ids):
-                    if tok in stops:
-                        result.finish_reasons[r] = "stop"
-                        eng.free_slot(slots.pop(r))          # an ended sequence gives its pages back at once
-                        continue
-                    result.tokens[r].append(tok)
-                    result.generated_tokens += 1
-                    if on_token is not None:
-                        on_token(r, tok)
-                    if len(result.tokens[r]) >= params.max_tokens:
-                        eng.free_slot(slots.pop(r))
-                        continue
-                    nxt.append((r, tok))
-                if not nxt:
-                    break
-                live = [r for r, _ in nxt]
-                logits = eng.step([(slots[r], [tok]) for r, tok in nxt], want="last")
-                ids = self._sample(sampler, logits, live, prompts, result, need_history)
-            self._sync()
-            result.decode_seconds += time.perf_counter() - t1
+            if self.look_ahead and getattr(eng, "takes_device_ids", False) and not params.has_penalties:
+                self._decode_ahead(batch, slots, prompts, params, sampler, stops, result, on_token)
+            else:
+                self._decode_in_step(batch, slots, prompts, params, sampler, stops, result, on_token)
         finally:
             for r in list(slots):
                 eng.free_slot(slots.pop(r))
+
+    def _decode_in_step(self, batch, slots, prompts, params, sampler, stops, result, on_token) -> None:
+        """Every step waits for its tokens on the host before the next one starts (needed when
+        the sampler wants each row's token history for penalties)."""
+        eng = self.engine
+        live = list(batch)
+        need_history = params.has_penalties
+        self._sync()
+        t0 = time.perf_counter()
+        logits = eng.step([(slots[r], prompts[r]) for r in live], want="last")
+        ids = self._sample(sampler, logits, live, prompts, result, need_history)
+        t1 = time.perf_counter()
+        result.prefill_seconds += t1 - t0
+        result.prompt_tokens += sum(len(prompts[r]) for r in live)
+        while True:
+            nxt = []
+            for r, tok in zip(live, ids):
+                if self._take_token(r, tok, slots, params, stops, result, on_token):
+                    nxt.append((r, tok))
+            if not nxt:
+                break
+            live = [r for r, _ in nxt]
+            logits = eng.step([(slots[r], [tok]) for r, tok in nxt], want="last")
+            ids = self._sample(sampler, logits, live, prompts, result, need_history)
+        self._sync()
+        result.decode_seconds += time.perf_counter() - t1
+
+    def _take_token(self, r, tok, slots, params, stops, result, on_token) -> bool:
+        """Books request r's next drawn token; False when the request is finished with it (a
+        stop token, which is not emitted, or the last token it may have).  A finished request
+        gives its slot and pages back at once."""
+        if tok in stops:
+            result.finish_reasons[r] = "stop"
+            self.engine.free_slot(slots.pop(r))
+            return False
+        result.tokens[r].append(tok)
+        result.generated_tokens += 1
+        if on_token is not None:
+            on_token(r, tok)
+        if len(result.tokens[r]) >= params.max_tokens:
+            self.engine.free_slot(slots.pop(r))
+            return False
+        return True
+
+    def _decode_ahead(self, batch, slots, prompts, params, sampler, stops, result, on_token) -> None:
+        """The same loop with the host one step behind the device: step t + 1 takes its tokens
+        from the device memory that step t's sampler wrote and is started before the host has
+        seen them, so the host's work per step (bookkeeping, page tables, the launch) runs while
+        the device computes.  The host reads step t's tokens while step t + 1 runs.  A request
+        whose token turns out to be a stop token has then run one step too many: its result is
+        dropped, and its slot is given back as usual (later work on the device comes after that
+        step in stream order).  Requests never take more steps than their share of the cache
+        allows: one that has its last permitted token coming is not stepped ahead."""
+        eng = self.engine
+        live = list(batch)
+        self._sync()
+        t0 = time.perf_counter()
+        logits = eng.step([(slots[r], prompts[r]) for r in live], want="last")
+        ids = sampler.sample(logits, live, [0] * len(live), None)
+        # rows: (request, its row in ids); fetch: the tokens on their way to the host
+        rows, fetch = [(r, i) for i, r in enumerate(live)], fetch_tokens(ids)
+        fetch_first = fetch
+        result.prompt_tokens += sum(len(prompts[r]) for r in live)
+        t1 = None
+        while rows:
+            # requests that go on if their pending token is no stop token: step them now
+            ahead = [(r, i) for r, i in rows if len(result.tokens[r]) + 1 < params.max_tokens]
+            nxt_ids = nxt_fetch = None
+            if ahead:
+                logits = eng.step([(slots[r], [0]) for r, _ in ahead], want="last",
+                                  device_ids=(ids, [i for _, i in ahead]))
+                nxt_ids = sampler.sample(logits, [r for r, _ in ahead],
+                                         [len(result.tokens[r]) + 1 for r, _ in ahead], None)
+                nxt_fetch = fetch_tokens(nxt_ids)
+            toks = fetch()
+            if t1 is None and fetch is fetch_first:                       # the prompt step has ended
+                t1 = time.perf_counter()
+                result.prefill_seconds += t1 - t0
+            went_on = set()
+            for r, i in rows:
+                if self._take_token(r, int(toks[i]), slots, params, stops, result, on_token):
+                    went_on.add(r)
+            rows = [(r, j) for j, (r, _) in enumerate(ahead) if r in went_on]
+            ids, fetch = nxt_ids, nxt_fetch
+        self._sync()
+        result.decode_seconds += time.perf_counter() - (t1 if t1 is not None else t0)
 
     @staticmethod
     def _sample(sampler, logits, live, prompts, result, need_history) -> List[int]:
@@ -135,3 +196,21 @@ class Generator:
         histories = [prompts[r] + result.tokens[r] for r in live] if need_history else None
         ids = sampler.sample(logits, live, indices, histories)
         return [int(t) for t in (ids.tolist() if hasattr(ids, "tolist") else ids)]
+
+
+def fetch_tokens(ids):
+    """Starts bringing sampled token ids to the host; the returned function waits for them and
+    gives a list.  Device tensors are copied into pinned memory behind the work already queued
+    on their stream; anything else (arrays of a stand-in engine) is taken as it is."""
+    if hasattr(ids, "is_cuda") and ids.is_cuda:
+        import torch
+        host = torch.empty(ids.shape, dtype=ids.dtype, pin_memory=True)
+        host.copy_(ids, non_blocking=True)
+        done = torch.cuda.Event()
+        done.record()
+
+        def wait():
+            done.synchronize()
+            return host.tolist()
+        return wait
+    return lambda: [int(t) for t in (ids.tolist() if hasattr(ids, "tolist") else ids)]

@@ -16,6 +16,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import numpy as np
 import torch
 
+from ..ops import kernels as K
 from ..parts.base import StepContext
 
 TABLE_BUCKET = 16          # page-table widths are rounded up to this many pages (1024 positions)
@@ -34,7 +35,8 @@ class DecodeGraph:
         self.batch, self.widths = batch, widths
         rt = engine.rt
         B = batch
-        self.sizes = [B, B, B, B, B] + [B * w for w in widths]          # ids, seq, pos, slots, rows, tables
+        # ids, seq, pos, slots, rows, tables, rows of another step's ids to take the ids from
+        self.sizes = [B, B, B, B, B] + [B * w for w in widths] + [B]
         total = sum(self.sizes)
         self.host = torch.empty(total, dtype=torch.int32, pin_memory=True)
         self.host_np = self.host.numpy()
@@ -47,7 +49,7 @@ class DecodeGraph:
         self.logits: Optional[torch.Tensor] = None
         self.copied = torch.cuda.Event()
 
-    def _fill(self, ids, tok_pos, slot_ids, tables: List[np.ndarray]) -> None:
+    def _fill(self, ids, tok_pos, slot_ids, tables: List[np.ndarray], id_rows=None) -> None:
         B = self.batch
         h = self.host_np
         self.copied.synchronize()                  # the last step's copy has left the staging buffer
@@ -62,6 +64,7 @@ class DecodeGraph:
             block[:, :t.shape[1]] = t
             block[:, t.shape[1]:] = -1
             o += B * w
+        h[o:o + B] = id_rows if id_rows is not None else 0
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
 
@@ -70,11 +73,17 @@ class DecodeGraph:
         ctx = StepContext(runtime=eng.rt, n_tokens=B, batch=B, ids=v[0], tok_seq=v[1], tok_pos=v[2], slots=v[3],
                           cu_seqlens=list(range(B + 1)), starts=[], slot_ids=[], is_decode=True,
                           max_context=max_context, in_graph=True)
-        tables = [t.view(B, w) for t, w in zip(v[5:], self.widths)]
+        tables = [t.view(B, w) for t, w in zip(v[5:5 + len(self.widths)], self.widths)]
         return eng.model.forward(ctx, eng.cache.layer_caches(tables), v[4])
 
-    def run(self, ids, tok_pos, slot_ids, tables: List[np.ndarray]) -> torch.Tensor:
-        self._fill(ids, tok_pos, slot_ids, tables)
+    def run(self, ids, tok_pos, slot_ids, tables: List[np.ndarray], device_ids=None) -> torch.Tensor:
+        """device_ids: (int32 device vector, rows): the step's ids are that vector's values at
+        `rows`, picked on the device before the replay, instead of `ids`."""
+        if device_ids is None:
+            self._fill(ids, tok_pos, slot_ids, tables)
+        else:
+            self._fill(ids, tok_pos, slot_ids, tables, np.asarray(device_ids[1], dtype=np.int32))
+            K.gather_i32(self.views[0], device_ids[0], self.views[-1])
         if self.graph is None:
             # the longest context this graph may ever see: what its page tables can hold
             cap = max(self.widths) * 64 if self.widths else 64
@@ -107,7 +116,7 @@ class GraphCache:
     def clear(self) -> None:
         self.graphs.clear()
 
-    def step(self, ids, tok_pos, slot_ids, tables: List[np.ndarray]) -> torch.Tensor:
+    def step(self, ids, tok_pos, slot_ids, tables: List[np.ndarray], device_ids=None) -> torch.Tensor:
         key = (len(slot_ids), tuple(bucket_width(t.shape[1]) for t in tables))
         g = self.graphs.get(key)
         if g is None:
@@ -117,4 +126,4 @@ class GraphCache:
             self.graphs[key] = g
         else:
             self.graphs.move_to_end(key)
-        return g.run(ids, tok_pos, slot_ids, tables)
+        return g.run(ids, tok_pos, slot_ids, tables, device_ids)

@@ -17,6 +17,7 @@ from ..cache.kv_cache import Cache
 from ..config.model_config import read_config_json
 from ..config.registry import architecture_of
 from ..models.model import Model
+from ..ops import kernels as K
 from ..ops import library
 from ..parts.base import Runtime, StepContext
 from ..weights.loader import Checkpoint
@@ -73,7 +74,8 @@ class Engine:
     # ---- construction ---------------------------------------------------------------
     @classmethod
     def from_folder(cls, folder: str, dtype: Union[str, torch.dtype] = "bfloat16", max_tokens: int = 4096,
-                    n_slots: int = 64, device: Union[str, torch.device] = "cuda:0", **spec_options) -> "Engine":
+                    n_slots: int = 64, device: Union[str, torch.device] = "cuda:0",
+                    use_graphs: Optional[bool] = None, **spec_options) -> "Engine":
         """config.json chooses the model class through the registry; model.safetensors is
         checked against what the model needs before any tensor is read."""
         dev = require_gpu(device)
@@ -91,12 +93,12 @@ class Engine:
                 torch.cuda.synchronize()
         finally:
             ckpt.close()
-        return cls(model, rt, max_tokens, n_slots, config)
+        return cls(model, rt, max_tokens, n_slots, config, use_graphs)
 
     @classmethod
     def from_config(cls, config: dict, seed: int = 0, dtype: Union[str, torch.dtype] = "bfloat16",
                     max_tokens: int = 4096, n_slots: int = 64, device: Union[str, torch.device] = "cuda:0",
-                    std: float = 0.02, **spec_options) -> "Engine":
+                    std: float = 0.02, use_graphs: Optional[bool] = None, **spec_options) -> "Engine":
         """A model of the parsed config.json `config` with random weights made on the device
         (matrices N(0, std), norm weights 1 + U(-0.1, 0.1)), without a model folder."""
         import hashlib
@@ -122,7 +124,7 @@ class Engine:
         with torch.cuda.device(dev):
             model.bind(get, rt)
             torch.cuda.synchronize()
-        return cls(model, rt, max_tokens, n_slots, typed)
+        return cls(model, rt, max_tokens, n_slots, typed, use_graphs)
 
     # ---- slots ---------------------------------------------------------------------
     def _graph_slots(self) -> int:
@@ -141,12 +143,21 @@ class Engine:
         self.cache.free_slot(slot)
 
     # ---- the step --------------------------------------------------------------------
+    # single-token steps can take their token ids from device memory (`device_ids`)
+    takes_device_ids = True
+
     def step(self, entries: Sequence[Tuple[int, Sequence[int]]],
-             want: Union[str, Sequence[Sequence[int]], None] = "last") -> Optional[torch.Tensor]:
+             want: Union[str, Sequence[Sequence[int]], None] = "last",
+             device_ids: Optional[Tuple[torch.Tensor, Sequence[int]]] = None) -> Optional[torch.Tensor]:
         """entries: (slot, next tokens) for each sequence of the batch.  want: 'last', 'all',
         None, or for each entry the places among its tokens whose logits are asked for.
         Returns float32 logits [wanted places, vocab] in the order of the entries and of
-        `want`, or None when nothing is wanted."""
+        `want`, or None when nothing is wanted.
+
+        device_ids = (ids, rows): every entry brings one token, and entry i's token is
+        ids[rows[i]] of an int32 vector on the device (what a sampler wrote after an earlier
+        step); the tokens in `entries` are then placeholders.  The host need not know the
+        tokens, so the step can be queued while the earlier one still runs."""
         if not entries:
             raise StepError("a step needs at least one sequence")
         slot_ids = [int(s) for s, _ in entries]
@@ -158,6 +169,15 @@ class Engine:
         ids = np.concatenate([np.asarray(t, dtype=np.int64).reshape(-1) for _, t in entries])
         if ids.min() < 0 or ids.max() >= self.vocab_size:
             raise StepError(f"token id outside 0..{self.vocab_size - 1}")
+        if device_ids is not None:
+            src, id_rows = device_ids
+            if max(counts) != 1 or len(id_rows) != len(entries):
+                raise StepError("device_ids needs one token and one row for each sequence")
+            if not (isinstance(src, torch.Tensor) and src.dtype == torch.int32 and src.dim() == 1
+                    and src.device == self.rt.device):
+                raise StepError("device_ids must be an int32 vector on the engine's device")
+            if min(id_rows) < 0 or max(id_rows) >= src.numel():
+                raise StepError(f"device_ids rows outside 0..{src.numel() - 1}")
         starts = [self.cache.length(s) for s in slot_ids]
         new_lens = [s + c for s, c in zip(starts, counts)]
         cu = np.zeros(len(entries) + 1, dtype=np.int64)
@@ -171,7 +191,8 @@ class Engine:
                 and self.cache.slots.n_slots == self._graph_slots():
             with torch.cuda.device(self.rt.device):
                 logits = self.graphs.step(ids.astype(np.int32), np.asarray(starts, dtype=np.int32),
-                                          np.asarray(slot_ids, dtype=np.int32), self.cache.step_tables(slot_ids))
+                                          np.asarray(slot_ids, dtype=np.int32), self.cache.step_tables(slot_ids),
+                                          device_ids)
                 logits = logits.clone()          # the graph's own buffer is overwritten by its next replay
             self.cache.commit(slot_ids, new_lens)
             self.steps_run += 1
@@ -181,12 +202,16 @@ class Engine:
         tables = self.cache.step_tables(slot_ids)
         parts = [ids.astype(np.int32), tok_seq, tok_pos, np.asarray(slot_ids, dtype=np.int32),
                  np.asarray(rows, dtype=np.int32), cu.astype(np.int32)] + [t.reshape(-1) for t in tables]
+        if device_ids is not None:
+            parts.append(np.asarray(device_ids[1], dtype=np.int32))
         dev = self._upload(parts)
         with torch.cuda.device(self.rt.device):
+            if device_ids is not None:
+                K.gather_i32(dev[0], device_ids[0], dev[-1])
             ctx = StepContext(runtime=self.rt, n_tokens=T, batch=B, ids=dev[0], tok_seq=dev[1], tok_pos=dev[2],
                               slots=dev[3], cu_seqlens=[int(c) for c in cu], starts=starts, slot_ids=slot_ids,
                               is_decode=max(counts) == 1, max_context=max(new_lens), cu_dev=dev[5])
-            dev_tables = [d.view(t.shape) for d, t in zip(dev[6:], tables)]
+            dev_tables = [d.view(t.shape) for d, t in zip(dev[6:6 + len(tables)], tables)]
             caches = self.cache.layer_caches(dev_tables)
             logits = self.model.forward(ctx, caches, dev[4] if len(rows) else None)
         self.cache.commit(slot_ids, new_lens)

@@ -96,6 +96,15 @@ def embed(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def gather_i32(dst: torch.Tensor, src: torch.Tensor, rows: torch.Tensor) -> None:
+    """dst[i] = src[rows[i]] for int32 vectors on the device."""
+    _dev(dst, src, rows)
+    _i32(dst, "dst"); _i32(src, "src"); _i32(rows, "rows")
+    _need(dst.dim() == 1 and src.dim() == 1 and rows.dim() == 1 and dst.numel() == rows.numel()
+          and dst.is_contiguous() and src.is_contiguous() and rows.is_contiguous(), "gather_i32: contiguous vectors, dst like rows")
+    _check(_lib().llogos_gather_i32(_p(dst), _p(src), _p(rows), dst.numel(), src.numel(), _stream()), "gather_i32")
+
+
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
             delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
             write_back: bool = True) -> torch.Tensor:

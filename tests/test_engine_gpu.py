@@ -2,6 +2,8 @@
 alone and whole; the last 32 tokens one by one; batches of unequal lengths whose shorter
 requests end earlier, one batch after another so that slots and pages are used again;
 long decoding; the first tokens of a sequence; greedy generation through the entry point."""
+import importlib
+
 import numpy as np
 import pytest
 import torch
@@ -205,6 +207,70 @@ def test_step_errors():
     assert eng.cache.length(s) == 0 and eng.cache.free_pages() == [2]          # refused steps change nothing
     eng.step([(s, [1, 2, 3])])
     assert eng.cache.length(s) == 3
+
+
+@pytest.mark.parametrize("graphs", [True, False])
+@pytest.mark.parametrize("dtype", H.DTYPES)
+def test_a_step_can_take_its_tokens_from_the_device(dtype, graphs):
+    """Single-token steps fed from an int32 vector on the device (in any order of rows) give
+    bit for bit what the same tokens from the host give, replayed as a graph or not."""
+    import torch
+    name = "tiny_b"
+    seqs = [list(H.tokens(name, n, 70 + n)) for n in (9, 70, 6)]
+    outs = []
+    for fed in (False, True):
+        eng = H.engine(name, dtype, max_tokens=1024, n_slots=4, use_graphs=graphs)
+        slots = [eng.alloc_slot() for _ in seqs]
+        eng.step([(s, q[:-4]) for s, q in zip(slots, seqs)], want=None)
+        got = []
+        for k in range(4, 0, -1):
+            toks = [q[-k] for q in seqs]
+            if fed:
+                # the tokens lie in another order in a longer vector, as after sequences have ended
+                src = torch.tensor([7, toks[2], toks[0], 1, toks[1]], dtype=torch.int32, device="cuda:0")
+                got.append(eng.step([(s, [0]) for s in slots], want="last", device_ids=(src, [2, 4, 1])))
+            else:
+                got.append(eng.step([(s, [t]) for s, t in zip(slots, toks)], want="last"))
+        outs.append(_np(torch.stack(got)))
+        if fed:
+            with pytest.raises(H.llogos.StepError, match="rows"):
+                eng.step([(s, [0]) for s in slots], device_ids=(src, [0, 1, 5]))
+            with pytest.raises(H.llogos.StepError, match="one token"):
+                eng.step([(slots[0], [0, 0])], device_ids=(src, [0]))
+            with pytest.raises(H.llogos.StepError, match="int32"):
+                eng.step([(slots[0], [0])], device_ids=(src.float(), [0]))
+    assert np.array_equal(outs[0], outs[1])
+    plain_rows = np.stack([np.stack([H.plain_logits(name, tuple(q))[len(q) - k] for q in seqs]) for k in range(4, 0, -1)])
+    H.close(outs[1], plain_rows, dtype, "device-fed steps")
+
+
+@pytest.mark.parametrize("temperature", [0.0, 0.7])
+@pytest.mark.parametrize("dtype", H.DTYPES)
+def test_generation_that_looks_ahead_gives_the_same_tokens(dtype, temperature):
+    """The loop that starts a step before the host has read the last one's tokens against
+    the loop that waits: same tokens, stop tokens honoured, every slot and page given back."""
+    import torch
+    name = "tiny_a"
+    gen_mod = importlib.import_module("daisi-llogos_amd.engine.generate")
+    prompts = [list(H.tokens(name, n, 90 + n)) for n in (5, 17, 1, 32, 8, 3)]
+    eng = H.engine(name, dtype, max_tokens=64 * 8, n_slots=4)
+    params = H.llogos.GenerationParams(max_tokens=20, temperature=temperature, top_k=0 if temperature == 0 else 20,
+                                       top_p=1.0, repetition_penalty=1.0, seed=5, stop_tokens=())
+    free = eng.cache.free_pages()
+    base = gen_mod.Generator(eng, max_batch=4, synchronize=torch.cuda.synchronize, look_ahead=False).generate(prompts, params)
+    # tokens that the requests draw at different times become stop tokens
+    stops = tuple({base.tokens[0][3], base.tokens[1][9], base.tokens[4][0], base.tokens[5][19]})
+    params = H.llogos.GenerationParams(max_tokens=20, temperature=temperature, top_k=0 if temperature == 0 else 20,
+                                       top_p=1.0, repetition_penalty=1.0, seed=5, stop_tokens=stops)
+    res = []
+    for ahead in (False, True):
+        g = gen_mod.Generator(eng, max_batch=4, synchronize=torch.cuda.synchronize, look_ahead=ahead)
+        res.append(g.generate(prompts, params))
+        assert eng.cache.live_slots == [] and eng.cache.free_pages() == free
+    assert res[0].tokens == res[1].tokens and res[0].finish_reasons == res[1].finish_reasons
+    assert "stop" in res[1].finish_reasons
+    for toks, full, why in zip(res[1].tokens, base.tokens, res[1].finish_reasons):
+        assert toks == full[:len(toks)] and (len(toks) == 20) == (why == "length")
 
 
 @pytest.mark.parametrize("dtype", H.DTYPES)

@@ -46,6 +46,19 @@ class FakeEngine:
         return out
 
 
+class AheadEngine(FakeEngine):
+    """The same, able to take a step's tokens from the ids a sampler left behind."""
+    takes_device_ids = True
+
+    def step(self, entries, want="last", device_ids=None):
+        if device_ids is not None:
+            ids, rows = device_ids
+            assert all(len(t) == 1 for _, t in entries) and len(rows) == len(entries)
+            self.fed = getattr(self, "fed", 0) + len(entries)
+            entries = [(s, [int(ids[i])]) for (s, _), i in zip(entries, rows)]
+        return super().step(entries, want)
+
+
 class ArgmaxSampler:
     def sample(self, logits, requests, indices, histories):
         self.last = (list(requests), list(indices))
@@ -155,3 +168,35 @@ def test_uniform_stream_is_per_request():
     assert a != [rng.uniform(8, 2, i) for i in range(50)] and a != [rng.uniform(7, 3, i) for i in range(50)]
     us = [rng.uniform(1, r, i) for r in range(40) for i in range(50)]
     assert abs(sum(us) / len(us) - 0.5) < 0.02
+
+
+@pytest.mark.parametrize("max_tokens", [1, 2, 3, 12])
+def test_looking_ahead_changes_no_result(max_tokens):
+    """With the host one step behind, a request that drew a stop token has run one step too
+    many; tokens, finish reasons and the slots given back are the same as without."""
+    prompts = [[1, 2, 3], [7], [4, 4, 4, 4, 4, 4], [9, 9], [3], [5, 6]]
+    stops = (13, 30, 14)
+    p = GenerationParams.greedy(max_tokens=max_tokens, stop_tokens=stops)
+    results = []
+    for engine in (FakeEngine(n_slots=4), AheadEngine(n_slots=4)):
+        g = gen.Generator(engine, max_batch=4)
+        seen = []
+        res = g.generate(prompts, p, sampler=ArgmaxSampler(), on_token=lambda r, t: seen.append((r, t)))
+        for i, pr in enumerate(prompts):
+            want, why = expected(pr, max_tokens, stops)
+            assert res.tokens[i] == want and res.finish_reasons[i] == why
+        assert sorted(seen) == sorted((i, t) for i, toks in enumerate(res.tokens) for t in toks)
+        assert not engine.cache.live_slots and not engine.sums          # every slot came back
+        assert engine.cache.free_pages() == [engine.cache.n_pages]
+        results.append(res)
+    assert results[0].generated_tokens == results[1].generated_tokens
+    # the engine that looks ahead also stepped every stop token it drew, unless that token would
+    # have been the request's last anyway; it never stepped a request past its last token
+    ahead = AheadEngine(n_slots=4)
+    res = gen.Generator(ahead, max_batch=4).generate(prompts, p, sampler=ArgmaxSampler())
+    single = getattr(ahead, "fed", 0)
+    want_single = 0
+    for toks, why in zip(res.tokens, res.finish_reasons):
+        n = len(toks)
+        want_single += n - 1 if why == "length" else n + (1 if n + 1 < max_tokens else 0)
+    assert single == want_single
