@@ -59,6 +59,7 @@ def main(argv=None) -> int:
     ap.add_argument("--steps", type=int, default=248)   # + 8 warm-up = 256 new tokens
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=PROMPT, help="tokens of each sequence's prompt before decoding")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration has (0 = all)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--only-prefill", action="store_true", help="time the 2,048-token prompt alone (for profiling)")
@@ -78,7 +79,7 @@ def main(argv=None) -> int:
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
     max_batch = max(args.batch, 1 if (args.no_points or args.only_prefill) else 64)
-    per_seq = PROMPT + args.steps + args.warmup + 64
+    per_seq = args.prompt_len + args.steps + args.warmup + 64
     t0 = time.time()
     eng = llogos.Engine.from_config(cfg, seed=0, dtype="bfloat16",
                                     max_tokens=max(max_batch * (per_seq + 64), PREFILL_TOKENS + 128), n_slots=max_batch)
@@ -89,7 +90,7 @@ def main(argv=None) -> int:
     def decode_run(batch, steps, warmup):
         """Prompts in one step, then greedy single-token steps: `warmup` untimed, `steps` timed."""
         slots = [eng.alloc_slot() for _ in range(batch)]
-        prompts = [rng.integers(0, cfg["vocab_size"], size=PROMPT).tolist() for _ in range(batch)]
+        prompts = [rng.integers(0, cfg["vocab_size"], size=args.prompt_len).tolist() for _ in range(batch)]
         logits = eng.step(list(zip(slots, prompts)), want="last")
         ids = K.argmax(logits)
         rows = list(range(batch))
@@ -111,7 +112,7 @@ def main(argv=None) -> int:
         run(steps)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
-        ctx_mid = PROMPT + warmup + steps / 2.0
+        ctx_mid = args.prompt_len + warmup + steps / 2.0
         for s in slots:
             eng.free_slot(s)
         return dt, ctx_mid
@@ -139,7 +140,7 @@ def main(argv=None) -> int:
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"model": "Llama-3.1-8B sizes, random weights", "global_batch": args.batch, "seq_len": CONTEXT,
-                   "parallelism": "single GPU", "prompt_len": PROMPT, "layers": cfg["num_hidden_layers"],
+                   "parallelism": "single GPU", "prompt_len": args.prompt_len, "layers": cfg["num_hidden_layers"],
                    "layers_full": full_layers, "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
                    "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
                    "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],

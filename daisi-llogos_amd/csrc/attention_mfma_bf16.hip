@@ -300,7 +300,9 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_decode_kernel(
 }
 
 // grid (batch, heads); HD threads.  Adds the partial results of the blocks along the context,
-// each of which covered pages_per_block pages.
+// each of which covered pages_per_block pages.  (Letting the last block to finish add them,
+// behind a device-wide fence and a ticket counter, was measured: the fence writes back whatever
+// earlier kernels left dirty in the L2 and cost 20 us a layer at batch 8; this kernel costs 4.6.)
 template <int HD>
 __global__ void attn_decode_merge_kernel(bf16_t* __restrict__ out, const float* __restrict__ partial,
                                          const int* __restrict__ tok_pos, int n_heads, int n_z, int pages_per_block) {

@@ -477,14 +477,16 @@ PREFILL_TILE_ROWS = 0        # 0: chosen by the step; 64 or 128 force a prefill 
 
 
 def _attn_workspace(device: torch.device, floats: int) -> torch.Tensor:
+    """Scratch memory of the decode attention, at least `floats` long.  A workspace that has
+    become too small stays alive beside its successor: captured steps keep its address."""
     key = (device.type, device.index)
-    ws = _attn_workspaces.get(key)
-    if ws is None or ws.numel() < floats:
+    held = _attn_workspaces.setdefault(key, [])
+    if not held or held[-1].numel() < floats:
         if torch.cuda.is_current_stream_capturing():
             raise KernelError("attention workspace must be made before a step is captured")
-        ws = torch.empty(max(floats, 1 << 20), dtype=torch.float32, device=device)
-        _attn_workspaces[key] = ws
-    return ws
+        size = max(floats, 1 << 20, 2 * held[-1].numel() if held else 0)
+        held.append(torch.empty(size, dtype=torch.float32, device=device))
+    return held[-1]
 
 
 def attention_mfma_bf16(ctx, q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
