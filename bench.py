@@ -1,7 +1,7 @@
 """Decode and prefill throughput of the Llama-3.1-8B layer sizes with random bfloat16
 weights on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--prompt-len P] [--model NAME]
 
 A step is one decode step of the whole batch.  The line printed at the end is the record:
 value = decoded tokens a second at the default batch of 8 (512-token random prompts, the
@@ -25,6 +25,15 @@ LLAMA31_8B = {
                      "original_max_position_embeddings": 8192},
     "attention_bias": False, "tie_word_embeddings": False, "torch_dtype": "bfloat16", "eos_token_id": 128001,
 }
+QWEN3_14B = {
+    "architectures": ["Qwen3ForCausalLM"], "vocab_size": 151936, "hidden_size": 5120, "intermediate_size": 17408,
+    "num_hidden_layers": 40, "num_attention_heads": 40, "num_key_value_heads": 8, "head_dim": 128,
+    "rms_norm_eps": 1e-6, "rope_theta": 1000000.0, "max_position_embeddings": 40960,
+    "attention_bias": False, "tie_word_embeddings": False, "torch_dtype": "bfloat16", "eos_token_id": 151645,
+}
+LLAMA31_70B = dict(LLAMA31_8B, hidden_size=8192, intermediate_size=28672, num_hidden_layers=80, num_attention_heads=64)
+MODELS = {"llama-3.1-8b": ("Llama-3.1-8B", LLAMA31_8B), "qwen3-14b": ("Qwen3-14B", QWEN3_14B),
+          "llama-3.1-70b": ("Llama-3.1-70B", LLAMA31_70B)}
 CONTEXT, PROMPT, PREFILL_TOKENS = 4096, 512, 2048
 
 
@@ -59,6 +68,7 @@ def main(argv=None) -> int:
     ap.add_argument("--steps", type=int, default=248)   # + 8 warm-up = 256 new tokens
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--model", choices=sorted(MODELS), default="llama-3.1-8b", help="whose layer sizes to run")
     ap.add_argument("--prompt-len", type=int, default=PROMPT, help="tokens of each sequence's prompt before decoding")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration has (0 = all)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
@@ -74,7 +84,8 @@ def main(argv=None) -> int:
     K = importlib.import_module("daisi-llogos_amd.ops.kernels")
     fetch_tokens = importlib.import_module("daisi-llogos_amd.engine.generate").fetch_tokens
 
-    cfg = dict(LLAMA31_8B)
+    model_name, cfg = MODELS[args.model]
+    cfg = dict(cfg)
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
@@ -136,15 +147,15 @@ def main(argv=None) -> int:
     step_bytes = weight_bytes(cfg) + args.batch * ctx_mid * kv_bytes_per_token(cfg)
     achieved = step_bytes / (dt / args.steps)
     record = {
-        "metric": "decode tok/s, Llama-3.1-8B bf16", "value": round(value, 1), "unit": "tok/s", "n_gpus": 1,
+        "metric": f"decode tok/s, {model_name} bf16", "value": round(value, 1), "unit": "tok/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"model": "Llama-3.1-8B sizes, random weights", "global_batch": args.batch, "seq_len": CONTEXT,
+        "config": {"model": f"{model_name} sizes, random weights", "global_batch": args.batch, "seq_len": CONTEXT,
                    "parallelism": "single GPU", "prompt_len": args.prompt_len, "layers": cfg["num_hidden_layers"],
                    "layers_full": full_layers, "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
                    "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
                    "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
-                   "rope_theta": cfg["rope_theta"], "rope_scaling": "llama3 x8", "rms_eps": cfg["rms_norm_eps"],
+                   "rope_theta": cfg["rope_theta"], "rope_scaling": "llama3 x8" if cfg.get("rope_scaling") else "none", "rms_eps": cfg["rms_norm_eps"],
                    "sampling": "greedy", "hip_graphs": eng.graphs is not None},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4)},

@@ -168,25 +168,27 @@ def test_window_and_sinks_as_run_time_strategy(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", H.DTYPES)
-def test_llama_8b_layer_sizes(dtype):
-    """Two layers of the 8B layer sizes (hidden 4096, 32/8 heads of 128, feed-forward 14336):
-    whole, the last tokens one by one, and an unequal batch, against the plain implementation."""
-    name = "layer_8b"
+@pytest.mark.parametrize("name", ["layer_8b", "layer_14b"])
+def test_layer_sizes_of_large_models(name, dtype):
+    """Two layers of the Llama-3.1-8B layer sizes (hidden 4096, 32/8 heads of 128, feed-forward
+    14336) and one of the Qwen3-14B sizes (hidden 5120, 40/8 heads with their norm, feed-forward
+    17408): whole, the last tokens one by one, and an unequal batch, against the plain
+    implementation."""
     eng = H.engine(name, dtype, max_tokens=64 * 12, n_slots=3)
     a, b, c = H.tokens(name, 150, 1), H.tokens(name, 70, 2), H.tokens(name, 3, 3)
     pa, pb, pc = (H.plain_logits(name, t) for t in (a, b, c))
     s = eng.alloc_slot()
     rows = [_np(eng.step([(s, a[:140])], want="all"))] + [_np(eng.step([(s, [t])])) for t in a[140:]]
-    H.close(np.concatenate(rows), pa, dtype, "8B sizes: prompt then tokens")
+    H.close(np.concatenate(rows), pa, dtype, f"{name}: prompt then tokens")
     eng.free_slot(s)
     slots = [eng.alloc_slot() for _ in range(3)]
     out = _np(eng.step([(slots[0], a[:100]), (slots[1], b[:66]), (slots[2], c[:2])], want="all"))
-    H.close(out, np.concatenate([pa[:100], pb[:66], pc[:2]]), dtype, "8B sizes: unequal batch")
+    H.close(out, np.concatenate([pa[:100], pb[:66], pc[:2]]), dtype, f"{name}: unequal batch")
     out = _np(eng.step([(slots[0], [a[100]]), (slots[1], [b[66]]), (slots[2], [c[2]])], want="last"))
-    H.close(out, np.stack([pa[100], pb[66], pc[2]]), dtype, "8B sizes: one token each")
+    H.close(out, np.stack([pa[100], pb[66], pc[2]]), dtype, f"{name}: one token each")
     eng.free_slot(slots[2])
     out = _np(eng.step([(slots[0], a[101:150]), (slots[1], [b[67]])], want=[[48], [0]]))
-    H.close(out, np.stack([pa[149], pb[67]]), dtype, "8B sizes: a continued prompt beside a single token")
+    H.close(out, np.stack([pa[149], pb[67]]), dtype, f"{name}: a continued prompt beside a single token")
 
 
 def test_step_errors():

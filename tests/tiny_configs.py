@@ -49,4 +49,11 @@ LAYER_8B = {   # two layers of the Llama-3.1-8B layer sizes with a small vocabul
     "tie_word_embeddings": False, "torch_dtype": "bfloat16", "eos_token_id": 2,
 }
 
-ALL = {"tiny_a": TINY_A, "tiny_b": TINY_B, "tiny_c": TINY_C, "tiny_w": TINY_W, "tiny_d": TINY_D, "layer_8b": LAYER_8B}
+LAYER_14B = {  # one layer of the Qwen3-14B layer sizes: widths that are no power of two, five query heads per kv head
+    "architectures": ["Qwen3ForCausalLM"], "vocab_size": 1033, "hidden_size": 5120, "intermediate_size": 17408,
+    "num_hidden_layers": 1, "num_attention_heads": 40, "num_key_value_heads": 8, "head_dim": 128,
+    "rms_norm_eps": 1e-6, "rope_theta": 1000000.0, "max_position_embeddings": 40960,
+    "tie_word_embeddings": False, "torch_dtype": "bfloat16", "eos_token_id": 2,
+}
+
+ALL = {"tiny_a": TINY_A, "tiny_b": TINY_B, "tiny_c": TINY_C, "tiny_w": TINY_W, "tiny_d": TINY_D, "layer_8b": LAYER_8B, "layer_14b": LAYER_14B}
