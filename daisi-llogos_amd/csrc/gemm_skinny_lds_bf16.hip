@@ -19,6 +19,8 @@
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kLdsWaves = 4;                 // waves per block (8 measured no faster)
 constexpr int kChunkK = 256;                 // values of k per LDS chunk (128 and 512 measured no faster)
@@ -65,12 +67,16 @@ __device__ __forceinline__ uint4 produce8(const ActSource& src, int m, int k, in
                 u[2 * j] = __uint_as_float(uw[j] << 16); u[2 * j + 1] = __uint_as_float(uw[j] & 0xffff0000u);
             }
         }
+        // silu(g) * u with the hardware's exp2 and reciprocal (about 1 ulp each, far below the
+        // rounding to bfloat16 that follows); every block of a column of blocks repeats this work,
+        // so it has to be cheap
         uint32_t o[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const float a = g[2 * j] / (1.0f + expf(-g[2 * j])) * u[2 * j];
-            const float b = g[2 * j + 1] / (1.0f + expf(-g[2 * j + 1])) * u[2 * j + 1];
-            o[j] = (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+            const float a = g[2 * j] * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g[2 * j])) * u[2 * j];
+            const float b = g[2 * j + 1] * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g[2 * j + 1])) * u[2 * j + 1];
+            const f32x2 ab = {a, b};
+            o[j] = __builtin_bit_cast(uint32_t, __builtin_convertvector(ab, bf16x2));
         }
         return make_uint4(o[0], o[1], o[2], o[3]);
     }
