@@ -231,16 +231,36 @@ __host__ __device__ constexpr size_t decode_lds_bytes(int waves, int group, int 
     return (size_t)waves * (group * (hd + 1) + 32) * sizeof(float);
 }
 
-template <int HD, int WAVES>
+// The fused form (FUSED, head size 128 rotated whole with split-half pairing) starts from the
+// projection itself: a block first makes its queries (sum of the projection's partial products,
+// bias, per-head norm, rotation) into LDS, and the block whose pages hold the step's position
+// also makes the step's key and value and writes them to their page, which the rotation kernel
+// does otherwise.  One token a sequence: token b is sequence b.
+struct QkvSource {
+    const float* qkv;          // [parts][batch][row_stride]: partial sums of the fused rows [q | k | v]
+    int parts;
+    size_t part_stride;
+    int row_stride;
+    const float* bias;         // [(heads + 2 kv heads) * 128] or null
+    const float* q_norm_w;     // [128] or null
+    const float* k_norm_w;
+    float eps;
+    const float2* cs;          // [batch][64] (cos, sin) of each sequence's position
+    bf16_t* k_pool;            // the pools, writable
+    bf16_t* v_pool;
+};
+
+template <int HD, int WAVES, bool FUSED>
 __global__ __launch_bounds__(WAVES * kWave) void attn_decode_kernel(
         bf16_t* __restrict__ out, float* __restrict__ partial, const bf16_t* __restrict__ q, int q_stride,
-        const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
+        QkvSource src, const bf16_t* k_pool, const bf16_t* v_pool,
         const int* __restrict__ table, int table_stride, const int* __restrict__ tok_pos,
         int n_heads, int n_kv_heads, int group, float scale, int window, int sinks) {
     extern __shared__ float lds[];
     float* lds_m = lds;                                   // [WAVES][16]
     float* lds_l = lds + WAVES * 16;                      // [WAVES][16]
     float* lds_o = lds + WAVES * 32;                      // [WAVES][group][HD + 1]
+    __shared__ __attribute__((aligned(16))) bf16_t q_lds[FUSED ? 16 : 1][HD];
     const int b = blockIdx.x, kvh = blockIdx.y, z = blockIdx.z;
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int c = lane & 15, g = lane >> 4;
@@ -249,12 +269,59 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_decode_kernel(
     if (z * WAVES >= n_pages) return;                            // nothing of this sequence here
     const int page_idx = z * WAVES + wave;
 
+    if (FUSED) {
+        // items 0 .. group - 1: the kv head's query heads; then, in the block that holds the
+        // step's position, its key and its value.  A wave takes an item; lane l holds
+        // dimensions 2 l and 2 l + 1, the rotation partner (64 dimensions away) is lane l ^ 32.
+        const bool writer = (n_pages - 1) / WAVES == z;
+        const int items = group + (writer ? 2 : 0);
+        const int d = 2 * lane;
+        const size_t page_base = writer
+            ? ((size_t)table[(size_t)b * table_stride + n_pages - 1] * n_kv_heads + kvh) * kPageTokens * HD : 0;
+        for (int item = wave; item < items; item += WAVES) {
+            const bool is_q = item < group, is_k = item == group;
+            const int head = is_q ? kvh * group + item : (is_k ? n_heads + kvh : n_heads + n_kv_heads + kvh);
+            const size_t col = (size_t)head * HD + d;
+            const float* p = src.qkv + (size_t)b * src.row_stride + col;
+            float2 x = *reinterpret_cast<const float2*>(p);
+            for (int part = 1; part < src.parts; ++part) {           // ascending order, as everywhere
+                const float2 y = *reinterpret_cast<const float2*>(p + part * src.part_stride);
+                x.x += y.x;
+                x.y += y.y;
+            }
+            if (src.bias) { x.x += src.bias[col]; x.y += src.bias[col + 1]; }
+            if (!is_q && !is_k) {
+                bf16_t* vdst = src.v_pool + page_base + (pos % kPageTokens);
+                vdst[(size_t)d * kPageTokens] = f32_to_bf16(x.x);
+                vdst[(size_t)(d + 1) * kPageTokens] = f32_to_bf16(x.y);
+                continue;
+            }
+            const float* norm_w = is_q ? src.q_norm_w : src.k_norm_w;
+            if (norm_w) {
+                const float ss = wave_sum(x.x * x.x + x.y * x.y);
+                const float inv = 1.0f / sqrtf(ss / (float)HD + src.eps);
+                x.x = x.x * inv * norm_w[d];
+                x.y = x.y * inv * norm_w[d + 1];
+            }
+            const float p0 = __shfl_xor(x.x, 32, kWave), p1 = __shfl_xor(x.y, 32, kWave);
+            const float2 c0 = src.cs[(size_t)b * 64 + (d & 63)], c1 = src.cs[(size_t)b * 64 + (d & 63) + 1];
+            float y0, y1;
+            if (lane < 32) { y0 = x.x * c0.x - p0 * c0.y; y1 = x.y * c1.x - p1 * c1.y; }
+            else           { y0 = p0 * c0.y + x.x * c0.x; y1 = p1 * c1.y + x.y * c1.x; }
+            const uint32_t packed = (uint32_t)f32_to_bf16(y0) | ((uint32_t)f32_to_bf16(y1) << 16);
+            if (is_q) *reinterpret_cast<uint32_t*>(&q_lds[item][d]) = packed;
+            else *reinterpret_cast<uint32_t*>(src.k_pool + page_base + (size_t)(pos % kPageTokens) * HD + d) = packed;
+        }
+        __syncthreads();          // the queries in LDS, and the key and value in memory, for every wave of the block
+    }
+
     WaveState<HD> st;
     st.init();
     if (page_idx < n_pages && page_may_be_visible(pos, page_idx * kPageTokens, window, sinks)) {
         bf16x8 qf[HD / 32];
         const bool col_ok = c < group;
-        const bf16_t* qrow = q + (size_t)b * q_stride + (size_t)(kvh * group + (col_ok ? c : 0)) * HD + 8 * g;
+        const bf16_t* qrow = FUSED ? &q_lds[col_ok ? c : 0][8 * g]
+                                   : q + (size_t)b * q_stride + (size_t)(kvh * group + (col_ok ? c : 0)) * HD + 8 * g;
 #pragma unroll
         for (int sk = 0; sk < HD / 32; ++sk) qf[sk] = col_ok ? ld_frag(qrow + 32 * sk) : zero_frag();
         const int page = table[(size_t)b * table_stride + page_idx];
@@ -650,13 +717,13 @@ LLOGOS_EXPORT long long llogos_attn_decode_workspace(int batch, int n_heads, int
     return n_z == 1 ? 0 : (long long)batch * n_heads * n_z * (head_dim + 2);
 }
 
-LLOGOS_EXPORT int llogos_attn_decode_bf16(void* out, const void* q, int q_stride, const void* k_pool,
-                                          const void* v_pool, const int* table, int table_stride, int table_width,
-                                          const int* tok_pos, int batch, int n_heads, int n_kv_heads, int head_dim,
-                                          float scale, int window, int sinks, float* workspace,
-                                          long long workspace_floats, hipStream_t stream) {
+static int launch_decode(void* out, const void* q, int q_stride, const QkvSource* src, const void* k_pool,
+                         const void* v_pool, const int* table, int table_stride, int table_width,
+                         const int* tok_pos, int batch, int n_heads, int n_kv_heads, int head_dim,
+                         float scale, int window, int sinks, float* workspace, long long workspace_floats,
+                         hipStream_t stream) {
     if (batch <= 0 || table_width <= 0 || window < 0 || sinks < 0) return LLOGOS_BAD_ARGUMENT;
-    if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || (q_stride % 8) || ((uintptr_t)q % 16)) return LLOGOS_UNSUPPORTED;
+    if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim)) return LLOGOS_UNSUPPORTED;
     if (workspace_floats < llogos_attn_decode_workspace(batch, n_heads, n_kv_heads, head_dim, table_width))
         return LLOGOS_BAD_ARGUMENT;
     const int group = n_heads / n_kv_heads;
@@ -665,17 +732,50 @@ LLOGOS_EXPORT int llogos_attn_decode_bf16(void* out, const void* q, int q_stride
     if (n_z > 1 && workspace == nullptr) return LLOGOS_BAD_ARGUMENT;
     dim3 grid(batch, n_kv_heads, n_z), mgrid(batch, n_heads);
     const size_t smem = decode_lds_bytes(waves, group, head_dim);
-#define GO(HD, W) do { \
-    attn_decode_kernel<HD, W><<<grid, W * kWave, smem, stream>>>( \
-        (bf16_t*)out, workspace, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, \
-        table_stride, tok_pos, n_heads, n_kv_heads, group, scale, window, sinks); \
+    const QkvSource none{};
+#define GO(HD, W, FUSED) do { \
+    attn_decode_kernel<HD, W, FUSED><<<grid, W * kWave, smem, stream>>>( \
+        (bf16_t*)out, workspace, (const bf16_t*)q, q_stride, FUSED ? *src : none, (const bf16_t*)k_pool, \
+        (const bf16_t*)v_pool, table, table_stride, tok_pos, n_heads, n_kv_heads, group, scale, window, sinks); \
     if (n_z > 1) attn_decode_merge_kernel<HD><<<mgrid, HD, 0, stream>>>((bf16_t*)out, workspace, tok_pos, n_heads, \
                                                                         n_z, W); } while (0)
-#define BY_WAVES(HD) do { if (waves == 16) GO(HD, 16); else if (waves == 8) GO(HD, 8); else GO(HD, 4); } while (0)
-    if (head_dim == 64) BY_WAVES(64); else BY_WAVES(128);
+#define BY_WAVES(HD, FUSED) do { if (waves == 16) GO(HD, 16, FUSED); else if (waves == 8) GO(HD, 8, FUSED); \
+                                 else GO(HD, 4, FUSED); } while (0)
+    if (src != nullptr) BY_WAVES(128, true);
+    else if (head_dim == 64) BY_WAVES(64, false);
+    else BY_WAVES(128, false);
 #undef BY_WAVES
 #undef GO
     return LLOGOS_LAUNCH_CHECK();
+}
+
+LLOGOS_EXPORT int llogos_attn_decode_bf16(void* out, const void* q, int q_stride, const void* k_pool,
+                                          const void* v_pool, const int* table, int table_stride, int table_width,
+                                          const int* tok_pos, int batch, int n_heads, int n_kv_heads, int head_dim,
+                                          float scale, int window, int sinks, float* workspace,
+                                          long long workspace_floats, hipStream_t stream) {
+    if ((q_stride % 8) || ((uintptr_t)q % 16)) return LLOGOS_UNSUPPORTED;
+    return launch_decode(out, q, q_stride, nullptr, k_pool, v_pool, table, table_stride, table_width, tok_pos, batch,
+                         n_heads, n_kv_heads, head_dim, scale, window, sinks, workspace, workspace_floats, stream);
+}
+
+// The same from the fused projection (see QkvSource): head size 128 only; also writes the
+// step's keys and values to their pages.  cs: [batch][64][2] floats.
+LLOGOS_EXPORT int llogos_attn_decode_fused_bf16(void* out, const float* qkv, int parts, long long part_stride,
+                                                int row_stride, const float* bias, const float* q_norm_w,
+                                                const float* k_norm_w, float eps, const void* cs, void* k_pool,
+                                                void* v_pool, const int* table, int table_stride, int table_width,
+                                                const int* tok_pos, int batch, int n_heads, int n_kv_heads,
+                                                int head_dim, float scale, int window, int sinks, float* workspace,
+                                                long long workspace_floats, hipStream_t stream) {
+    if (head_dim != 128) return LLOGOS_UNSUPPORTED;
+    if (parts < 1 || (row_stride % 2) || (part_stride % 2) || ((uintptr_t)qkv % 8) ||
+        row_stride < (n_heads + 2 * n_kv_heads) * head_dim)
+        return LLOGOS_BAD_ARGUMENT;
+    const QkvSource src{qkv, parts, (size_t)part_stride, row_stride, bias, q_norm_w, k_norm_w, eps,
+                        (const float2*)cs, (bf16_t*)k_pool, (bf16_t*)v_pool};
+    return launch_decode(out, nullptr, 0, &src, k_pool, v_pool, table, table_stride, table_width, tok_pos, batch,
+                         n_heads, n_kv_heads, head_dim, scale, window, sinks, workspace, workspace_floats, stream);
 }
 
 // tile_rows: 64 for the kernel whose waves read pages from global memory, 128 for the kernel

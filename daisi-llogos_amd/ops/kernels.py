@@ -408,9 +408,10 @@ def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swigl
     uses a library for its prompt products, Daisi.Llogos.Cuda/CudaBackend.cs:158-316)."""
     M = a.shape[-2]
     if w.dtype == torch.bfloat16 and M <= SKINNY_MAX_ROWS and out_dtype == torch.bfloat16:
+        few_dtype = torch.float32 if f32_ok else out_dtype              # what a product in one part is written as
         kernel, splits, row_blocks = skinny_plan(M, w.shape[0], w.shape[1])
         if kernel == "stationary" and not swiglu_input and a.dim() == 2:
-            out = gemm_skinny_stationary_bf16(a, w, None, out_dtype, row_blocks)
+            out = gemm_skinny_stationary_bf16(a, w, None, few_dtype, row_blocks)
             if out is not None:
                 return out
             kernel, splits, row_blocks = "lds", 1, 1
@@ -421,12 +422,12 @@ def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swigl
         if swiglu_input and not (M <= 16 and a.dtype == torch.bfloat16 and (a.dim() == 2 or a.shape[0] == 1)):
             a, swiglu_input = swiglu(a, out_dtype), False
         if swiglu_input or kernel == "lds":
-            out = gemm_skinny_lds_bf16(a, w, None, out_dtype, splits if kernel == "lds" else 1, row_blocks,
+            out = gemm_skinny_lds_bf16(a, w, None, few_dtype, splits if kernel == "lds" else 1, row_blocks,
                                        swiglu_input)
             if out is not None:
                 return out
         if not swiglu_input and a.dtype == torch.bfloat16:
-            out = gemm_skinny_bf16(a, w, None, out_dtype, splits if kernel == "regs" else 1, row_blocks)
+            out = gemm_skinny_bf16(a, w, None, few_dtype, splits if kernel == "regs" else 1, row_blocks)
             if out is not None:
                 return out
     if swiglu_input:
@@ -529,6 +530,50 @@ def attention_mfma_bf16(ctx, q: torch.Tensor, q_stride: int, k_pool: torch.Tenso
     if code == -2:
         return None
     _check(code, "attention_mfma_bf16")
+    return out
+
+
+def attention_decode_fused(ctx, qkv: torch.Tensor, bias: Optional[torch.Tensor], n_heads: int, n_kv_heads: int,
+                           head_dim: int, rot: int, pairing: int, q_norm_w: Optional[torch.Tensor],
+                           k_norm_w: Optional[torch.Tensor], eps: float, cs: torch.Tensor, k_pool: torch.Tensor,
+                           v_pool: torch.Tensor, table: torch.Tensor, scale: float, window: int = 0,
+                           sinks: int = 0) -> Optional[torch.Tensor]:
+    """A single-token step's attention straight from the fused projection rows [q | k | v]
+    (float32 [T, W] or partial sums [parts, T, W]): bias, per-head norm, rotation and the cache
+    write happen inside the attention kernel.  For bfloat16 caches, head size 128 rotated whole
+    with split-half pairing; None for anything else (the caller then runs the steps apart)."""
+    if not (ctx.is_decode and qkv.dtype == torch.float32 and k_pool.dtype == torch.bfloat16 and head_dim == 128
+            and rot == 128 and pairing == 0 and n_heads % n_kv_heads == 0 and n_heads // n_kv_heads <= 16):
+        return None
+    parts, part_stride = _parts(qkv)
+    T = qkv.shape[-2]
+    width = (n_heads + 2 * n_kv_heads) * head_dim
+    if qkv.stride(-1) != 1 or qkv.stride(-2) % 2 or part_stride % 2 or qkv.data_ptr() % 8:
+        return None
+    _dev(qkv, bias, q_norm_w, k_norm_w, cs, k_pool, v_pool, table, ctx.tok_pos)
+    _i32(table, "table"); _i32(ctx.tok_pos, "tok_pos")
+    _need(T == ctx.n_tokens == ctx.batch and qkv.shape[-1] == width, f"attention: qkv must be [{ctx.batch}, {width}]")
+    _need(cs.dtype == torch.float32 and cs.shape == (T, rot // 2, 2) and cs.is_contiguous(), "attention: rotary table shape")
+    _need(table.dim() == 2 and table.shape[0] == T and ctx.tok_pos.numel() == T, "attention: one table row and position a sequence")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.shape == (width,), f"attention: bias must be float32 [{width}]")
+    for wgt in (q_norm_w, k_norm_w):
+        if wgt is not None:
+            _need(wgt.dtype == torch.float32 and wgt.shape == (head_dim,), "attention: norm weight float32 [head_dim]")
+    _check_pools(k_pool, v_pool, n_kv_heads, head_dim, "attention")
+    _need(v_pool.dtype == torch.bfloat16, "attention: cache types differ")
+    out = torch.empty((T, n_heads * head_dim), dtype=torch.bfloat16, device=qkv.device)
+    lib = _lib()
+    width_pages = table.shape[1]
+    ws = _attn_workspace(qkv.device, lib.llogos_attn_decode_workspace(T, n_heads, n_kv_heads, head_dim, width_pages))
+    code = lib.llogos_attn_decode_fused_bf16(
+        _p(out), _p(qkv), parts, ctypes.c_longlong(part_stride), qkv.stride(-2), _p(bias), _p(q_norm_w), _p(k_norm_w),
+        ctypes.c_float(eps), _p(cs), _p(k_pool), _p(v_pool), _p(table), table.stride(0), width_pages, _p(ctx.tok_pos),
+        T, n_heads, n_kv_heads, head_dim, ctypes.c_float(scale), window, sinks, _p(ws),
+        ctypes.c_longlong(ws.numel()), _stream())
+    if code == -2:
+        return None
+    _check(code, "attention_decode_fused")
     return out
 
 

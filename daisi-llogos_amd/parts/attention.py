@@ -44,6 +44,7 @@ class Attention(Mixer):
         self.o = Linear([prefix + "o_proj"], q_w, [hidden])
         self.q_norm_w: Optional[torch.Tensor] = None
         self.k_norm_w: Optional[torch.Tensor] = None
+        self.fuse_decode = True     # single-token steps: one kernel from the projection to the attention output
 
     def kv_spec(self) -> KVSpec:
         return KVSpec(self.n_kv_heads, self.head_dim, self.window, self.sinks)
@@ -70,6 +71,14 @@ class Attention(Mixer):
         cs = self.position.prepare(ctx)
         if cache.writes:
             qkv = self.qkv.product(h, f32_ok=True)                      # [(parts,) T, (nh + 2 nkv) hd]
+            if ctx.is_decode and self.fuse_decode:
+                # one token a sequence: norm, rotation and cache write inside the attention kernel
+                a = K.attention_decode_fused(ctx, qkv, self.qkv.bias_rows(), nh, nkv, hd, self.position.rot,
+                                             self.position.pairing, self.q_norm_w, self.k_norm_w, self.eps, cs,
+                                             cache.k_pool, cache.v_pool, cache.table, self.scale, self.window,
+                                             self.sinks)
+                if a is not None:
+                    return self.o.product(a, f32_ok=True)
             q = K.qk_rope_cache(qkv, self.qkv.bias_rows(), self.rt.dtype, nh, nkv, hd, self.position.rot,
                                 self.position.pairing, self.q_norm_w, self.k_norm_w, self.eps, cs,
                                 cache.k_pool, cache.v_pool, cache.table, ctx.tok_seq, ctx.tok_pos)

@@ -144,6 +144,64 @@ def test_attention_part_alone(dtype, nh, nkv, hd, bias, qk_norm, window):
     assert np.abs(got - want).max() <= TOL[dtype] * max(1.0, np.abs(want).max())
 
 
+@pytest.mark.parametrize("nh,nkv,bias,qk_norm,window", [(8, 2, True, True, 0), (16, 1, False, False, 0),
+                                                        (5, 5, False, True, 70), (12, 4, True, False, 0)])
+def test_single_token_steps_from_the_projection_in_one_kernel(nh, nkv, bias, qk_norm, window, monkeypatch):
+    """Head size 128 in bfloat16: the attention kernel that makes its queries and the step's key
+    and value from the projection itself gives, bit for bit, the outputs and the cache pages of
+    the rotation kernel followed by the attention kernel, across a page's end, and both agree
+    with the plain parts."""
+    dtype, hd, hidden = "bfloat16", 128, 72
+    rng = np.random.default_rng(nh)
+    rt = P.Runtime(DEV, DT[dtype])
+    att = P.Attention("a.", hidden, nh, nkv, hd, P.Rotary(hd, hd, 1e4), bias=bias, qk_norm=qk_norm, eps=1e-5,
+                      window=window)
+    tensors, plain = {}, {}
+    for spec in att.tensor_specs():
+        t, a = _rand(rng, spec.shape, dtype, 0.2 if spec.kind == "matrix" else 1.0)
+        if spec.kind == "norm":
+            t = (1 + 0.1 * t.float()).to(DT[dtype]); a = t.double().numpy()
+        tensors[spec.name], plain[spec.name] = t, a
+    att.bind(tensors.get, rt)
+    taken = []
+    fused_kernel = K.attention_decode_fused
+    monkeypatch.setattr(K, "attention_decode_fused", lambda *a, **k: (taken.append(fused_kernel(*a, **k)), taken[-1])[1])
+    lens, steps = [62, 130, 5], 4
+    xs = [_rand(rng, (l + steps, hidden), dtype) for l in lens]
+    table = torch.tensor([[5, 1, 7, 9], [0, 8, 2, 6], [4, 3, 10, 11]], dtype=torch.int32, device=DEV)
+    results = []
+    for fused in (False, True):
+        att.fuse_decode = fused
+        pool = lambda *shape: torch.full((12, nkv) + shape, float("nan"), dtype=DT[dtype], device=DEV)
+        cache = P.LayerCache(k_pool=pool(64, hd), v_pool=pool(hd, 64), table=table)
+        x0 = torch.cat([x[:l] for (x, _), l in zip(xs, lens)]).to(DEV)
+        outs = [K.sum_parts(att.forward(_ctx(rt, lens, lens), x0, cache), None, DT[dtype])]
+        for t in range(steps):
+            xt = torch.stack([x[l + t] for (x, _), l in zip(xs, lens)]).to(DEV)
+            outs.append(K.sum_parts(att.forward(_ctx(rt, [l + t + 1 for l in lens], [1] * 3), xt, cache), None, DT[dtype]))
+        results.append((torch.cat(outs), cache.k_pool.clone(), cache.v_pool.clone()))
+    assert len(taken) == steps and all(t is not None for t in taken)       # the fused kernel took every single-token step
+    for a, b in zip(*results):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))       # bit for bit, NaN of unwritten pages included
+    # against the plain parts, sequence by sequence
+    got = _np(results[1][0])
+    o = sum(lens)
+    for i, ((_, x_), l) in enumerate(zip(xs, lens)):
+        q = pm.linear(x_, plain["a.q_proj.weight"], plain.get("a.q_proj.bias"))
+        k = pm.linear(x_, plain["a.k_proj.weight"], plain.get("a.k_proj.bias"))
+        v = pm.linear(x_, plain["a.v_proj.weight"], plain.get("a.v_proj.bias"))
+        if qk_norm:
+            q = pm.per_head_rms_norm(q, plain["a.q_norm.weight"], nh, hd, 1e-5)
+            k = pm.per_head_rms_norm(k, plain["a.k_norm.weight"], nkv, hd, 1e-5)
+        f = pm.rope_frequencies(hd, 1e4)
+        n = l + steps
+        q, k = pm.rope_split_half(q, range(n), nh, hd, f), pm.rope_split_half(k, range(n), nkv, hd, f)
+        want = pm.linear(pm.attention(q, k, v, nh, nkv, hd, window=window), plain["a.o_proj.weight"])
+        for t in range(steps):
+            row = got[o + 3 * t + i]
+            assert np.abs(row - want[l + t]).max() <= TOL[dtype] * max(1.0, np.abs(want).max())
+
+
 @pytest.mark.parametrize("dtype", H.DTYPES)
 def test_swiglu_part_alone(dtype):
     rng = np.random.default_rng(3)
