@@ -118,34 +118,35 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny_kernel(
     }
 }
 
-// Third form, for up to 16 activation rows, K <= 4096 and very many rows of w (gate/up, the
-// output head): the activations stay in registers.  The 4 waves of a block split k; each
-// wave loads its quarter of the activation fragments once (up to 32 steps = 128 registers)
+// Third form, for up to 16 activation rows and very many rows of w (gate/up, the output head):
+// the activations stay in registers.  The WAVES waves of a block split k; each wave loads its
+// share of the activation fragments once (STEPS steps of 32 values of k = 4 STEPS registers)
 // and then streams `strips` strips of 16 rows of w past them, so that the activations cost
 // 1 / strips of what they cost when every strip fetches its own.  The waves' sums of a strip
-// are added through LDS in wave order, as in the first form.
-constexpr int kStatSteps = 32;          // MFMA steps of 32 values of k per wave at most
+// are added through LDS in wave order, as in the first form.  K <= 32 * STEPS * WAVES:
+// 4 waves x 32 steps for K <= 4096, 8 x 20 for K <= 5120, 8 x 32 for K <= 8192.
 constexpr int kStatU = 4;               // steps per prefetched chunk
 
-template <typename TO>
-__global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny_stationary_kernel(
+template <typename TO, int WAVES, int STEPS>
+__global__ __launch_bounds__(WAVES * kWave) void gemm_skinny_stationary_kernel(
         TO* __restrict__ out, const bf16_t* __restrict__ a, const bf16_t* __restrict__ w,
         const float* __restrict__ bias, int M, int N, int K, int lda, int ldo, int strips_per_block) {
-    __shared__ float red[kSkinnyWaves][kWave][4];
+    static_assert(STEPS % kStatU == 0, "whole chunks");
+    __shared__ float red[WAVES][kWave][4];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int r = lane & 15, g = lane >> 4;
-    const int k_per_wave = (((K + 31) / 32 + kSkinnyWaves - 1) / kSkinnyWaves) * 32;     // <= 32 * kStatSteps
+    const int k_per_wave = (((K + 31) / 32 + WAVES - 1) / WAVES) * 32;               // <= 32 * STEPS
     const int k_begin = wave * k_per_wave;
     const int k_end = min(K, k_begin + k_per_wave);
-    constexpr int kChunks = kStatSteps / kStatU;
+    constexpr int kChunks = STEPS / kStatU;
 
     // this wave's activation fragments, once
-    bf16x8 af[kStatSteps];
+    bf16x8 af[STEPS];
     {
         const bool row_ok = r < M;
         const bf16_t* arow = a + (size_t)min(r, M - 1) * lda + g * 8;
 #pragma unroll
-        for (int s = 0; s < kStatSteps; ++s) {
+        for (int s = 0; s < STEPS; ++s) {
             const int kk = k_begin + s * kStepK;
             af[s] = load_frag(arow + kk, row_ok && kk + g * 8 < k_end);
         }
@@ -181,12 +182,14 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny_stationary_k
         for (int i = 0; i < 4; ++i) red[wave][lane][i] = acc[i];
         acc = f32x4{0.f, 0.f, 0.f, 0.f};
         __syncthreads();
-        const int t_lane = threadIdx.x & (kWave - 1), t_i = threadIdx.x / kWave;
-        float sum = 0.f;
+        if (threadIdx.x < 4 * kWave) {                                   // one thread per value of the strip
+            const int t_lane = threadIdx.x & (kWave - 1), t_i = threadIdx.x / kWave;
+            float sum = 0.f;
 #pragma unroll
-        for (int wv = 0; wv < kSkinnyWaves; ++wv) sum += red[wv][t_lane][t_i];
-        const int n = strip * 16 + 4 * (t_lane >> 4) + t_i, m = t_lane & 15;
-        if (m < M && n < N) store_f32(out + (size_t)m * ldo + n, sum + (bias ? bias[n] : 0.f));
+            for (int wv = 0; wv < WAVES; ++wv) sum += red[wv][t_lane][t_i];
+            const int n = strip * 16 + 4 * (t_lane >> 4) + t_i, m = t_lane & 15;
+            if (m < M && n < N) store_f32(out + (size_t)m * ldo + n, sum + (bias ? bias[n] : 0.f));
+        }
         __syncthreads();
     };
 
@@ -204,24 +207,31 @@ __global__ __launch_bounds__(kSkinnyWaves * kWave) void gemm_skinny_stationary_k
     }
 }
 
-// The few-row product with stationary activations: M <= 16, K <= 4096.  One part, bias allowed.
+template <int WAVES, int STEPS>
+static int launch_stationary(void* out, int out_dtype, const void* a, const void* w, const float* bias, int M, int N,
+                             int K, int lda, int ldo, int strips_per_block, hipStream_t stream) {
+    const int n_strips = (N + 15) / 16;
+    const int blocks = (n_strips + strips_per_block - 1) / strips_per_block;
+    if (out_dtype == DT_BF16)
+        gemm_skinny_stationary_kernel<bf16_t, WAVES, STEPS><<<blocks, WAVES * kWave, 0, stream>>>(
+            (bf16_t*)out, (const bf16_t*)a, (const bf16_t*)w, bias, M, N, K, lda, ldo, strips_per_block);
+    else
+        gemm_skinny_stationary_kernel<float, WAVES, STEPS><<<blocks, WAVES * kWave, 0, stream>>>(
+            (float*)out, (const bf16_t*)a, (const bf16_t*)w, bias, M, N, K, lda, ldo, strips_per_block);
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+// The few-row product with stationary activations: M <= 16, K <= 8192.  One part, bias allowed.
 LLOGOS_EXPORT int llogos_gemm_skinny_stationary_bf16(void* out, int out_dtype, const void* a, const void* w,
                                                      const float* bias, int M, int N, int K, int lda, int ldo,
                                                      int strips_per_block, hipStream_t stream) {
     if (M <= 0 || N <= 0 || K <= 0 || lda < K || ldo < N || strips_per_block < 1) return LLOGOS_BAD_ARGUMENT;
     if (out_dtype != DT_BF16 && out_dtype != DT_F32) return LLOGOS_BAD_ARGUMENT;
-    if (M > 16 || K > 32 * kStatSteps * kSkinnyWaves || (K % 8) || (lda % 8) || ((uintptr_t)a % 16) ||
-        ((uintptr_t)w % 16))
+    if (M > 16 || K > 8192 || (K % 8) || (lda % 8) || ((uintptr_t)a % 16) || ((uintptr_t)w % 16))
         return LLOGOS_UNSUPPORTED;
-    const int n_strips = (N + 15) / 16;
-    const int blocks = (n_strips + strips_per_block - 1) / strips_per_block;
-    if (out_dtype == DT_BF16)
-        gemm_skinny_stationary_kernel<bf16_t><<<blocks, kSkinnyWaves * kWave, 0, stream>>>(
-            (bf16_t*)out, (const bf16_t*)a, (const bf16_t*)w, bias, M, N, K, lda, ldo, strips_per_block);
-    else
-        gemm_skinny_stationary_kernel<float><<<blocks, kSkinnyWaves * kWave, 0, stream>>>(
-            (float*)out, (const bf16_t*)a, (const bf16_t*)w, bias, M, N, K, lda, ldo, strips_per_block);
-    return LLOGOS_LAUNCH_CHECK();
+    if (K <= 4096) return launch_stationary<4, 32>(out, out_dtype, a, w, bias, M, N, K, lda, ldo, strips_per_block, stream);
+    if (K <= 5120) return launch_stationary<8, 20>(out, out_dtype, a, w, bias, M, N, K, lda, ldo, strips_per_block, stream);
+    return launch_stationary<8, 32>(out, out_dtype, a, w, bias, M, N, K, lda, ldo, strips_per_block, stream);
 }
 
 template <int RB, int MB, int U>

@@ -285,6 +285,8 @@ def skinny_plan(M: int, N: int, K: int) -> Tuple[str, int, int]:
     does not depend on how many other rows the batch has."""
     if N >= 16384 and K <= 4096 and (M <= 8 or (M <= 16 and N >= 65536)):
         return "stationary", 1, (8 if N >= 65536 else 4)      # third value: strips per block
+    if N >= 16384 and 5120 < K <= 8192 and M <= 16:           # 8 waves of 32 steps (8 x 20 at k = 5120 measured slower)
+        return "stationary", 1, 8
     if M <= 4 and N >= 16384:
         strips = -(-N // 16)
         return "regs", max(1, min(-(-1024 // strips), K // 1024, 8)), 1
@@ -327,12 +329,12 @@ def gemm_skinny_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tens
 def gemm_skinny_stationary_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
                                 out_dtype: torch.dtype, strips: int = 4) -> Optional[torch.Tensor]:
     """The few-row bfloat16 product with the activations held in registers while `strips` strips
-    of 16 rows of w stream past: up to 16 rows, K <= 4096.  [1, M, N]; None for other shapes."""
+    of 16 rows of w stream past: up to 16 rows, K <= 8192.  [1, M, N]; None for other shapes."""
     if a.dim() != 2:
         return None
     M, K = a.shape
     N = w.shape[0]
-    if not (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and 0 < M <= 16 and K <= 4096 and K % 8 == 0
+    if not (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and 0 < M <= 16 and K <= 8192 and K % 8 == 0
             and a.stride(1) == 1 and a.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
             and w.is_contiguous()):
         return None

@@ -85,7 +85,8 @@ def test_gemm(dtype, M, N, K_):
 
 
 @pytest.mark.parametrize("M,N,K_", [(1, 4096, 4096), (8, 331, 1000), (16, 100, 72), (17, 4096, 14336), (64, 257, 2048),
-                                    (33, 6144, 4096), (5, 20000, 4096), (16, 70001, 1000)])
+                                    (33, 6144, 4096), (5, 20000, 4096), (16, 70001, 1000), (7, 1000, 5120),
+                                    (9, 333, 8192), (3, 200, 6000)])
 def test_gemm_few_rows_on_the_matrix_cores(M, N, K_):
     rng = np.random.default_rng(7)
     a = _t(rng.standard_normal((M, K_)), torch.bfloat16)
@@ -99,7 +100,7 @@ def test_gemm_few_rows_on_the_matrix_cores(M, N, K_):
                 out = kernel(a, w, None, torch.float32, splits, rb)
                 assert out is not None and out.dtype == torch.float32 and out.shape[1:] == (M, N)
                 assert np.abs(_np(out).sum(0) - want).max() <= 2e-6 * scale * math.sqrt(K_)
-    if M <= 16 and K_ <= 4096:                                          # activations held in registers
+    if M <= 16 and K_ <= 8192:                                          # activations held in registers
         for strips in (1, 3, 8):
             out = K.gemm_skinny_stationary_bf16(a, w, b, torch.float32, strips)
             assert out is not None and np.abs(_np(out)[0] - (want + _np(b))).max() <= 2e-6 * scale * math.sqrt(K_)
