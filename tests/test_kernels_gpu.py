@@ -353,6 +353,20 @@ def test_swiglu(dtype):
     _close(K.sum_parts(parts, None, DT[dtype]), _np(gu), dtype)
 
 
+def test_gather_of_token_ids():
+    src = _t([5, 9, 2, 7, 11], torch.int32)
+    rows = _t([4, 0, 0, 3], torch.int32)
+    dst = torch.full((4,), -1, dtype=torch.int32, device=DEV)
+    K.gather_i32(dst, src, rows)
+    assert dst.cpu().tolist() == [11, 5, 5, 7]
+    K.gather_i32(dst, src, _t([1, 7, -1, 2], torch.int32))               # rows outside the vector give 0, never a fault
+    assert dst.cpu().tolist() == [9, 0, 0, 2]
+    with pytest.raises(K.KernelError):
+        K.gather_i32(dst, src, rows[:3])
+    with pytest.raises(K.KernelError):
+        K.gather_i32(dst, src.float(), rows)
+
+
 def test_argmax_first_maximum_wins():
     rng = np.random.default_rng(6)
     x = rng.standard_normal((5, 128257)).astype(np.float32)
