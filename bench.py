@@ -70,10 +70,12 @@ def main(argv=None) -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--model", choices=sorted(MODELS), default="llama-3.1-8b", help="whose layer sizes to run")
     ap.add_argument("--prompt-len", type=int, default=PROMPT, help="tokens of each sequence's prompt before decoding")
+    ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS, help="tokens of the timed prompt")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration has (0 = all)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--only-prefill", action="store_true", help="time the 2,048-token prompt alone (for profiling)")
     args = ap.parse_args(argv)
+    prefill_tokens = args.prefill_tokens
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU library")
         return 2
@@ -93,7 +95,7 @@ def main(argv=None) -> int:
     per_seq = args.prompt_len + args.steps + args.warmup + 64
     t0 = time.time()
     eng = llogos.Engine.from_config(cfg, seed=0, dtype="bfloat16",
-                                    max_tokens=max(max_batch * (per_seq + 64), PREFILL_TOKENS + 128), n_slots=max_batch)
+                                    max_tokens=max(max_batch * (per_seq + 64), prefill_tokens + 128), n_slots=max_batch)
     print(f"[bench] model ready in {time.time() - t0:.1f} s; weights {weight_bytes(cfg) / 1e9:.2f} GB, "
           f"cache {eng.cache.bytes() / 1e9:.2f} GB", file=sys.stderr, flush=True)
     rng = np.random.default_rng(0)
@@ -129,14 +131,14 @@ def main(argv=None) -> int:
         return dt, ctx_mid
 
     if args.only_prefill:
-        prompt = rng.integers(0, cfg["vocab_size"], size=PREFILL_TOKENS).tolist()
+        prompt = rng.integers(0, cfg["vocab_size"], size=prefill_tokens).tolist()
         for it in range(4):
             s = eng.alloc_slot()
             torch.cuda.synchronize()
             t = time.perf_counter()
             eng.step([(s, prompt)], want="last")
             torch.cuda.synchronize()
-            print(f"[bench] prefill {PREFILL_TOKENS} tokens, {cfg['num_hidden_layers']} layers: "
+            print(f"[bench] prefill {prefill_tokens} tokens, {cfg['num_hidden_layers']} layers: "
                   f"{(time.perf_counter() - t) * 1e3:.2f} ms", file=sys.stderr, flush=True)
             eng.free_slot(s)
         return 0
@@ -172,7 +174,7 @@ def main(argv=None) -> int:
             print(f"[bench] decode b{b}: {points[f'decode_b{b}']:.1f} tok/s, {d / steps * 1e3:.3f} ms/step",
                   file=sys.stderr, flush=True)
         record["points"] = points
-        prompt = rng.integers(0, cfg["vocab_size"], size=PREFILL_TOKENS).tolist()
+        prompt = rng.integers(0, cfg["vocab_size"], size=prefill_tokens).tolist()
         times = []
         for it in range(3):
             s = eng.alloc_slot()
@@ -183,10 +185,10 @@ def main(argv=None) -> int:
             times.append(time.perf_counter() - t)
             eng.free_slot(s)
         pt = min(times[1:])
-        flops = prefill_flops(cfg, PREFILL_TOKENS)
-        record["prefill"] = {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS, "ms": round(pt * 1e3, 3),
+        flops = prefill_flops(cfg, prefill_tokens)
+        record["prefill"] = {"value": round(prefill_tokens / pt, 1), "tokens": prefill_tokens, "ms": round(pt * 1e3, 3),
                              "frac": round(flops / pt / MFMA_PEAK["bf16"], 4)}
-        print(f"[bench] prefill {PREFILL_TOKENS}: {PREFILL_TOKENS / pt:.0f} tok/s, {pt * 1e3:.2f} ms", file=sys.stderr,
+        print(f"[bench] prefill {prefill_tokens}: {prefill_tokens / pt:.0f} tok/s, {pt * 1e3:.2f} ms", file=sys.stderr,
               flush=True)
     print(json.dumps(record), flush=True)
     return 0
