@@ -211,6 +211,38 @@ def test_step_errors():
     assert eng.cache.length(s) == 3
 
 
+@pytest.mark.parametrize("name", ["tiny_b", "tiny_w", "layer_14b"])
+@pytest.mark.parametrize("dtype", H.DTYPES)
+def test_replayed_steps_equal_steps_launched_kernel_by_kernel(name, dtype):
+    """Single-token steps replayed as a captured graph against the same steps launched kernel
+    by kernel, bit for bit, replay after replay, with other work of the engine between the
+    replays: prompts of other sequences, sequences that end, and a batch that shrinks and
+    grows (another graph each)."""
+    engines = [H.engine(name, dtype, max_tokens=64 * 24, n_slots=4, use_graphs=g) for g in (True, False)]
+    assert engines[0].graphs is not None and engines[1].graphs is None
+    rng = np.random.default_rng(3)
+    vocab = tc.ALL[name]["vocab_size"]
+    new = lambda n: [int(t) for t in rng.integers(0, vocab, n)]
+    plan = [("prompt", 0, new(70)), ("prompt", 1, new(5))] + [("tokens", (0, 1), None)] * 6 + \
+           [("prompt", 2, new(130))] + [("tokens", (0, 1, 2), None)] * 5 + [("end", 1, None)] + \
+           [("tokens", (0, 2), None)] * 4 + [("prompt", 3, new(64))] + [("tokens", (3, 0, 2), None)] * 5
+    slots = [{}, {}]
+    for what, arg, toks in plan:
+        outs = []
+        step_tokens = new(len(arg)) if what == "tokens" else None
+        for e, (eng, sl) in enumerate(zip(engines, slots)):
+            if what == "prompt":
+                sl[arg] = eng.alloc_slot()
+                outs.append(eng.step([(sl[arg], toks)], want="last"))
+            elif what == "end":
+                eng.free_slot(sl.pop(arg))
+            else:
+                outs.append(eng.step([(sl[r], [t]) for r, t in zip(arg, step_tokens)], want="last"))
+        if outs:
+            assert torch.equal(outs[0], outs[1]), (what, arg)
+    assert len(engines[0].graphs.graphs) >= 2
+
+
 @pytest.mark.parametrize("graphs", [True, False])
 @pytest.mark.parametrize("dtype", H.DTYPES)
 def test_a_step_can_take_its_tokens_from_the_device(dtype, graphs):
