@@ -284,10 +284,15 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_decode_kernel(
             const size_t col = (size_t)head * HD + d;
             const float* p = src.qkv + (size_t)b * src.row_stride + col;
             float2 x = *reinterpret_cast<const float2*>(p);
-            for (int part = 1; part < src.parts; ++part) {           // ascending order, as everywhere
-                const float2 y = *reinterpret_cast<const float2*>(p + part * src.part_stride);
-                x.x += y.x;
-                x.y += y.y;
+            for (int part0 = 1; part0 < src.parts; part0 += 8) {     // eight loads in flight, added in ascending order
+                float2 y[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    y[j] = part0 + j < src.parts ? *reinterpret_cast<const float2*>(p + (part0 + j) * src.part_stride)
+                                                 : float2{0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (part0 + j < src.parts) { x.x += y[j].x; x.y += y[j].y; }
             }
             if (src.bias) { x.x += src.bias[col]; x.y += src.bias[col + 1]; }
             if (!is_q && !is_k) {

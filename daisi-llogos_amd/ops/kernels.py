@@ -275,14 +275,43 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
 SKINNY_MAX_ROWS = 64
 
 
+def lds_splits(M: int, N: int, K: int, n_cus: int = 256) -> int:
+    """Blocks along k for the LDS few-row product.  Measured on the MI355X, three things decide:
+    how evenly the blocks fill the compute units (544 blocks on 256 units run as long as 768),
+    whether there are enough of them to keep the memory system busy (about 1.5 a unit), and the
+    float32 partial sums every further block along k writes and the consumer reads (they cost
+    about 6 M / K of the weights' time each).  64 rows of activations leave LDS for two blocks a
+    unit, so blocks come in rounds of twice the units there.  More blocks along k are taken only
+    for a clear gain (8 %), since they also cost the consumer a fused form or a launch."""
+    n_blocks = -(-N // 64)
+    chunks = -(-K // 256)
+    rows = 16 if M <= 16 else (32 if M <= 32 else 64)
+    per_round = n_cus * (2 if rows == 64 else 1)
+    best, best_score, seen = 1, -1.0, set()
+    for s in range(1, 9):
+        per = -(-chunks // s)
+        parts = -(-chunks // per)
+        if parts in seen or (parts > 1 and per < 2):
+            continue
+        seen.add(parts)
+        blocks = n_blocks * parts
+        evenness = blocks / (-(-blocks // per_round) * per_round)
+        enough = min(1.0, blocks / (1.5 * n_cus))
+        partial_sums = 1.0 + (parts - 1) * 6.0 * rows / K
+        score = evenness * enough / partial_sums * (1.0 - 0.01 * (parts - 1))
+        if score > best_score * 1.08:
+            best, best_score = parts, score
+    return best
+
+
 def skinny_plan(M: int, N: int, K: int) -> Tuple[str, int, int]:
     """(kernel, blocks along k, 16-row blocks of w per wave) for the few-row product.
     'stationary': activations held in registers while strips of w stream past; best for few
     rows and very many rows of w (gate/up, the head).  'regs': every wave fetches its own
     activation fragments; for up to 4 rows where k is too long for 'stationary'.  'lds': the
     block shares the activations through LDS; its speed hardly depends on the number of rows.
-    Within a kernel the split of k depends on N and K alone, so the order of a row's additions
-    does not depend on how many other rows the batch has."""
+    The plan depends on the shape and on the number of rows rounded up to 16, 32 or 64, so a
+    row's additions come in the same order for every batch of that class."""
     if N >= 16384 and K <= 4096 and (M <= 8 or (M <= 16 and N >= 65536)):
         return "stationary", 1, (8 if N >= 65536 else 4)      # third value: strips per block
     if N >= 16384 and 5120 < K <= 8192 and M <= 16:           # 8 waves of 32 steps (8 x 20 at k = 5120 measured slower)
@@ -290,10 +319,7 @@ def skinny_plan(M: int, N: int, K: int) -> Tuple[str, int, int]:
     if M <= 4 and N >= 16384:
         strips = -(-N // 16)
         return "regs", max(1, min(-(-1024 // strips), K // 1024, 8)), 1
-    blocks = -(-N // 64)
-    if blocks >= 256:
-        return "lds", 1, 1
-    return "lds", max(1, min(-(-512 // blocks), K // 512, 8)), 1
+    return "lds", lds_splits(M, N, K), 1
 
 
 def gemm_skinny_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype,
