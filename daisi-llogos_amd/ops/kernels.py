@@ -332,7 +332,7 @@ def skinny_plan(M: int, N: int, K: int) -> Tuple[str, int, int]:
     row's additions come in the same order for every batch of that class."""
     if N >= 16384 and K <= 4096 and (M <= 8 or (M <= 16 and N >= 65536)):
         return "stationary", 1, stationary_strips(N, K)       # third value: strips per block
-    if N >= 16384 and 5120 < K <= 8192 and M <= 16:           # 8 waves of 32 steps (8 x 20 at k = 5120 measured slower)
+    if N >= 16384 and 4096 < K <= 8192 and M <= 16:           # 8 waves a block
         return "stationary", 1, stationary_strips(N, K)
     if M <= 4 and N >= 16384:
         strips = -(-N // 16)
