@@ -215,10 +215,17 @@ class PlainConfig:
     def frequencies(self) -> np.ndarray:
         f = rope_frequencies(self.rot_dim, self.theta)
         rs = self.rope_scaling
-        if rs and rs.get("rope_type", rs.get("type")) == "llama3":
+        kind = rs.get("rope_type", rs.get("type")) if rs else None
+        if kind == "llama3":
             f = f / llama3_frequency_factors(f, float(rs["factor"]), float(rs["low_freq_factor"]),
                                              float(rs["high_freq_factor"]),
                                              int(rs["original_max_position_embeddings"]))
+        elif kind == "linear":
+            # one factor for every pair in the reference's per-pair table, f_i / factor_i (Cpu/Rope.cs:42-63):
+            # positions are stretched by `factor`
+            f = f / float(rs["factor"])
+        elif kind not in (None, "default"):
+            raise ValueError(f"unknown rotary scaling '{kind}'")
         return f
 
 

@@ -122,6 +122,22 @@ def test_llama3_factors():
     assert np.allclose(pm.llama3_frequency_factors(f, 1.0, 1.0, 4.0, 8192), 1.0)
 
 
+def test_linear_scaling_stretches_positions():
+    """rope_scaling 'linear' with factor s: position s * p of the scaled model is position p of
+    the unscaled one; unknown kinds are refused."""
+    base = dict(vocab_size=50, hidden_size=32, intermediate_size=48, num_hidden_layers=1, num_attention_heads=2,
+                head_dim=16, rope_theta=1e4)
+    plain_f = pm.PlainConfig(dict(base, architectures=["LlamaForCausalLM"])).frequencies()
+    scaled = pm.PlainConfig(dict(base, architectures=["LlamaForCausalLM"], rope_scaling={"rope_type": "linear", "factor": 4.0}))
+    assert np.allclose(scaled.frequencies(), plain_f / 4.0, rtol=1e-15)
+    x = np.random.default_rng(0).standard_normal((3, 32))
+    a = pm.rope_split_half(x, [0, 8, 20], 2, 16, scaled.frequencies())
+    b = pm.rope_split_half(x, [0, 2, 5], 2, 16, plain_f)
+    assert np.allclose(a, b, atol=1e-12)
+    with pytest.raises(ValueError, match="yarn"):
+        pm.PlainConfig(dict(base, architectures=["LlamaForCausalLM"], rope_scaling={"rope_type": "yarn", "factor": 2.0})).frequencies()
+
+
 def _sdpa(q, k, v, n_heads, n_kv, hd, causal=True):
     t = q.shape[0]
     qt = torch.tensor(q).reshape(t, n_heads, hd).transpose(0, 1)
