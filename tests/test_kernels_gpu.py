@@ -131,6 +131,27 @@ def test_gemm_few_rows_on_the_matrix_cores(M, N, K_):
     assert K.gemm_skinny_bf16(a[:, :K_ - 4], w[:, :K_ - 4].contiguous(), None, torch.float32) is None   # k % 8
 
 
+def test_products_of_random_shapes_through_the_dispatch():
+    """Whatever kernel and split of k the plan picks for a shape, the product is right: row
+    counts up to 64 and beyond, widths and depths that are multiples of 8 and of nothing else."""
+    rng = np.random.default_rng(21)
+    for case in range(40):
+        M = int(rng.choice([1, 2, 5, 8, 13, 16, 17, 31, 33, 64, 70]))
+        K_ = 8 * int(rng.integers(1, 1100))                                # up to 8,792
+        N = int(rng.integers(1, 40000)) if case % 4 else int(rng.integers(16384, 72000))
+        a = _t(rng.standard_normal((M, K_)), torch.bfloat16)
+        w = torch.randn((N, K_), device=DEV, dtype=torch.bfloat16, generator=torch.Generator(device=DEV).manual_seed(case)) * 0.05
+        b = _t(rng.standard_normal(N))
+        want = _np(a.float() @ w.float().t())                              # float32 on the device stands in for float64 here
+        scale = max(1.0, np.abs(want).max())
+        prod = K.gemm_product(a, w, torch.bfloat16, f32_ok=bool(case % 2))
+        got = _np(K.sum_parts(prod, b, torch.float32))
+        tol = (1e-2 if prod.dtype == torch.bfloat16 else 2e-5) * scale
+        assert np.abs(got - (want + _np(b))).max() <= tol, (case, M, N, K_, K.skinny_plan(M, N, K_))
+        got = _np(K.gemm(a, w, b, torch.float32))
+        assert np.abs(got - (want + _np(b))).max() <= 2e-5 * scale, (case, M, N, K_)
+
+
 def test_rope_table_is_double_precision():
     pos = _t([0, 1, 4095, 100000], torch.int32)
     f = pm.rope_frequencies(64, 5e5)
@@ -273,6 +294,38 @@ def test_single_token_attention_with_blocks_of_every_size(nh, nkv, hd, batch, lo
     out = K.attention_mfma_bf16(ctx, c["q"], c["stride"], c["kp"], c["vp"], c["table"], nh, nkv, hd, 1 / math.sqrt(hd))
     assert out is not None
     _close(out, _plain_attention(c, nh, nkv, hd), "bfloat16")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_attention_of_random_shapes(dtype):
+    """Heads, groups, head sizes, lengths, windows and sinks drawn at random: prompts whole and
+    continued, and single tokens, whichever kernel the dispatch takes."""
+    rng = np.random.default_rng(31)
+    for case in range(24):
+        hd = int(rng.choice([16, 32, 48, 64, 64, 96, 128, 128, 256]))
+        nkv = int(rng.choice([1, 2, 3, 8]))
+        nh = nkv * int(rng.choice([1, 2, 4, 5, 16]))
+        B = int(rng.integers(1, 5))
+        lens = [int(rng.integers(1, 400)) for _ in range(B)]
+        kind = case % 3
+        new = [1] * B if kind == 0 else (lens if kind == 1 else [int(rng.integers(1, l + 1)) for l in lens])
+        window = int(rng.choice([0, 0, 1, 64, 100]))
+        sinks = int(rng.choice([0, 4])) if window else 0
+        c = _attention_case(dtype, nh, nkv, hd, lens, new, seed=100 + case)
+        for b, l in enumerate(lens):                                        # unwritten page tails must not matter
+            if l % 64:
+                page = int(c["table"][b, l // 64])
+                c["kp"][page, :, l % 64:, :] = float("nan")
+                c["vp"][page, :, :, l % 64:] = float("nan")
+        ctx = type("Ctx", (), dict(tok_seq=_t(c["tok_seq"], torch.int32), tok_pos=_t(c["tok_pos"], torch.int32),
+                                   is_decode=max(new) == 1, max_context=max(lens), batch=B, n_tokens=sum(new),
+                                   cu_seqlens=np.concatenate([[0], np.cumsum(new)]).tolist(),
+                                   cu_dev=_t(np.concatenate([[0], np.cumsum(new)]), torch.int32),
+                                   starts=[l - n for l, n in zip(lens, new)], shared={}))()
+        out = K.attention(ctx, c["q"], c["stride"], c["kp"], c["vp"], c["table"], nh, nkv, hd, 1 / math.sqrt(hd), window, sinks)
+        want = _plain_attention(c, nh, nkv, hd, window, sinks)
+        err = np.abs(_np(out) - want).max()
+        assert err <= RT[dtype] * max(1.0, np.abs(want).max()), (case, nh, nkv, hd, lens, new, window, sinks, err)
 
 
 @pytest.mark.parametrize("tile_rows", [64, 128])
