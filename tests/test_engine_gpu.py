@@ -140,6 +140,25 @@ def test_long_decoding(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", H.DTYPES)
+@pytest.mark.parametrize("name", ["tiny_d", "tiny_w"])
+def test_a_context_of_thousands_of_positions(name, dtype):
+    """2,300 positions: a prompt of 36 pages in one step, a second one continued across a page's
+    end beside it, then single tokens for both (page tables wider than one bucket of the
+    captured steps, many blocks along the context and their merge)."""
+    eng = H.engine(name, dtype, max_tokens=64 * 80, n_slots=2)
+    a, b = H.tokens(name, 2300, 21), H.tokens(name, 2200, 22)
+    pa, pb = H.plain_logits(name, a), H.plain_logits(name, b)
+    sa, sb = eng.alloc_slot(), eng.alloc_slot()
+    got = _np(eng.step([(sa, a[:2290]), (sb, b[:2000])], want=[[0, 63, 64, 2289], [1999]]))
+    H.close(got, np.stack([pa[0], pa[63], pa[64], pa[2289], pb[1999]]), dtype, f"{name}: long prompts")
+    got = _np(eng.step([(sa, [a[2290]]), (sb, b[2000:2190])], want=[[0], [0, 47, 189]]))
+    H.close(got, np.stack([pa[2290], pb[2000], pb[2047], pb[2189]]), dtype, f"{name}: a token beside a continued prompt")
+    for t in range(2291, 2296):
+        got = _np(eng.step([(sa, [a[t]]), (sb, [b[t - 101]])], want="last"))
+        H.close(got, np.stack([pa[t], pb[t - 101]]), dtype, f"{name}: token {t}")
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
 @pytest.mark.parametrize("name", CONFIGS)
 def test_first_tokens(name, dtype):
     eng = H.engine(name, dtype)
