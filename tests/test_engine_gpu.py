@@ -262,6 +262,24 @@ def test_replayed_steps_equal_steps_launched_kernel_by_kernel(name, dtype):
     assert len(engines[0].graphs.graphs) >= 2
 
 
+def test_captured_steps_are_dropped_and_made_again(monkeypatch):
+    """More batch shapes than captured steps are kept: the least recently used one goes, and
+    a shape that comes back is captured again; results stay those of uncaptured steps."""
+    graph_mod = importlib.import_module("daisi-llogos_amd.engine.graph")
+    monkeypatch.setattr(graph_mod, "MAX_GRAPHS", 2)
+    name, dtype = "tiny_b", "bfloat16"
+    engines = [H.engine(name, dtype, max_tokens=64 * 12, n_slots=6, use_graphs=g) for g in (True, False)]
+    rng = np.random.default_rng(8)
+    slots = [[eng.alloc_slot() for _ in range(5)] for eng in engines]
+    for eng, sl in zip(engines, slots):
+        eng.step([(s, list(H.tokens(name, 3 + i, 40 + i))) for i, s in enumerate(sl)], want=None)
+    for batch in (1, 2, 3, 4, 5, 1, 3, 5, 2, 2, 4):
+        toks = [int(t) for t in rng.integers(0, tc.ALL[name]["vocab_size"], batch)]
+        outs = [eng.step([(s, [t]) for s, t in zip(sl[:batch], toks)], want="last") for eng, sl in zip(engines, slots)]
+        assert torch.equal(outs[0], outs[1]), batch
+        assert len(engines[0].graphs.graphs) <= 2
+
+
 @pytest.mark.parametrize("graphs", [True, False])
 @pytest.mark.parametrize("dtype", H.DTYPES)
 def test_a_step_can_take_its_tokens_from_the_device(dtype, graphs):
