@@ -61,8 +61,8 @@ class Engine:
     def __init__(self, model: Model, rt: Runtime, max_tokens: int, n_slots: int = 64, config=None,
                  use_graphs: Optional[bool] = None):
         self.model, self.rt, self.config = model, rt, config
-        # single-token steps are replayed as HIP graphs when every mixer allows it
-        graph_ok = all(layer.mixer.graph_safe for layer in model.layers)
+        # single-token steps are replayed as HIP graphs when every mixer and feed-forward allows it
+        graph_ok = all(layer.mixer.graph_safe and getattr(layer.ffn, "graph_safe", False) for layer in model.layers)
         if use_graphs is None:
             use_graphs = os.environ.get("LLOGOS_GRAPHS", "1") != "0"
         self.graphs = GraphCache(self) if (use_graphs and graph_ok) else None

@@ -127,6 +127,10 @@ class Mixer(Part):
 class FeedForward(Part):
     """forward(ctx, h [T, H]) -> [T, H], or float32 partial sums [parts, T, H]."""
 
+    # True when forward launches the same kernels with the same shapes whatever the tokens are
+    # (no routing decided on the host), so that a captured single-token step can be replayed.
+    graph_safe = False
+
     def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 

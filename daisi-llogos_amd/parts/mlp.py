@@ -13,6 +13,8 @@ from .linear import Linear
 
 @register_feed_forward("swiglu")
 class SwiGLU(FeedForward):
+    graph_safe = True
+
     def __init__(self, prefix: str, hidden: int, intermediate: int):
         self.prefix = prefix
         self.hidden, self.intermediate = hidden, intermediate

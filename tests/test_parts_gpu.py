@@ -1,6 +1,7 @@
 """Each part alone against its plain counterpart, the order of layers as data (a layer run
-twice, a layer reading another's cache), and a toy mixer with state of its own that is
-registered, built and stepped without a change to the library's files."""
+twice, a layer reading another's cache), and toy parts defined here that are registered, built
+and stepped without a change to the library's files: a mixer with state of its own, a
+feed-forward with a router and experts, and another position encoding."""
 import dataclasses
 import importlib
 import math
@@ -405,3 +406,144 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
         H.close(np.concatenate(rows[i]), want[i], "float32", f"toy batch seq {i}")
     with pytest.raises(L.CacheError, match="state"):
         s = eng.alloc_slot(); eng.step([(s, [1, 2, 3])]); eng.cache.truncate(s, 1)
+
+
+# ---------------------------------------------------------------------------
+# a toy feed-forward with routing and a toy position encoding, defined here
+# ---------------------------------------------------------------------------
+@P.register_feed_forward("toy_routed")
+class ToyRoutedFeedForward(P.FeedForward):
+    """A router picks one of `n_experts` SwiGLU experts for each token; the expert's output is
+    scaled by the router's probability of it.  The routing is decided on the host (tokens are
+    gathered per expert), so steps with it are not captured."""
+
+    def __init__(self, prefix: str, hidden: int, intermediate: int, n_experts: int):
+        self.router = P.Linear([prefix + "router"], hidden, [n_experts])
+        self.experts = [P.SwiGLU(f"{prefix}experts.{e}.", hidden, intermediate) for e in range(n_experts)]
+
+    def tensor_specs(self):
+        return self.router.tensor_specs() + [s for e in self.experts for s in e.tensor_specs()]
+
+    def bind(self, get, rt):
+        super().bind(get, rt)
+        self.router.bind(get, rt)
+        for e in self.experts:
+            e.bind(get, rt)
+
+    def forward(self, ctx, h):
+        logits = self.router.forward(h, out_dtype=torch.float32)            # router logits in 32-bit
+        prob = torch.softmax(logits, dim=-1)
+        choice = torch.argmax(logits, dim=-1)
+        out = torch.zeros((h.shape[0], h.shape[1]), dtype=torch.float32, device=h.device)
+        for e, expert in enumerate(self.experts):
+            rows = torch.nonzero(choice == e).flatten()
+            if rows.numel():
+                y = K.sum_parts(expert.forward(ctx, h[rows].contiguous()), None, torch.float32)
+                out[rows] = y * prob[rows, e:e + 1]
+        return out
+
+
+@P.register_position("toy_restarting")
+class RestartingRotary(P.Rotary):
+    """Rotary angles of position modulo `period`: another encoding behind the same interface."""
+
+    def __init__(self, head_dim: int, theta: float, period: int):
+        super().__init__(head_dim, head_dim, theta)
+        self.period = period
+
+    def prepare(self, ctx):
+        key = ("toy_restarting", id(self))
+        if key not in ctx.shared:
+            ctx.shared[key] = K.rope_table(torch.remainder(ctx.tok_pos, self.period).to(torch.int32), self.inv_freq)
+        return ctx.shared[key]
+
+
+@dataclasses.dataclass(frozen=True)
+class RoutedConfig:
+    vocab_size: int
+    hidden_size: int
+    n_layers: int
+    num_hidden_layers: int = 0
+    num_attention_heads: int = 4
+    num_key_value_heads: int = 2
+
+
+def _routed_spec(cfg, **kw):
+    models = importlib.import_module("daisi-llogos_amd.models")
+    layers = []
+    for i in range(cfg.n_layers):
+        p = f"layers.{i}."
+        pos = RestartingRotary(16, 1e4, 8) if i % 2 == 0 else P.Rotary(16, 16, 1e4)
+        ffn = ("toy_routed", dict(prefix=p + "moe.", hidden=cfg.hidden_size, intermediate=24, n_experts=3)) if i != 1 else \
+            ("swiglu", dict(prefix=p + "ffn.", hidden=cfg.hidden_size, intermediate=56))
+        layers.append(models.LayerSpec(
+            mixer=("attention", dict(prefix=p + "attn.", hidden=cfg.hidden_size, n_heads=4, n_kv_heads=2, head_dim=16,
+                                     position=pos)),
+            ffn=ffn,
+            mixer_norm=("rmsnorm", dict(name=p + "n1", width=cfg.hidden_size, eps=1e-6)),
+            ffn_norm=("rmsnorm", dict(name=p + "n2", width=cfg.hidden_size, eps=1e-6))))
+    return models.ModelSpec(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size, embed_name="embed.weight",
+                            layers=layers, final_norm=("rmsnorm", dict(name="norm", width=cfg.hidden_size, eps=1e-6)),
+                            head_name="head", tie_head=True)
+
+
+L.register_architecture("ToyRoutedForCausalLM",
+                        lambda d: RoutedConfig(d["vocab_size"], d["hidden_size"], d["n_layers"]), _routed_spec)
+
+
+def _plain_routed(w, tokens, n_layers):
+    T = len(tokens)
+    x = pm.embedding(w["embed.weight"], tokens)
+    f = pm.rope_frequencies(16, 1e4)
+    for i in range(n_layers):
+        p = f"layers.{i}."
+        n = pm.rms_norm(x, w[p + "n1.weight"], 1e-6)
+        positions = [t % 8 for t in range(T)] if i % 2 == 0 else list(range(T))
+        q = pm.rope_split_half(pm.linear(n, w[p + "attn.q_proj.weight"]), positions, 4, 16, f)
+        k = pm.rope_split_half(pm.linear(n, w[p + "attn.k_proj.weight"]), positions, 2, 16, f)
+        x = x + pm.linear(pm.attention(q, k, pm.linear(n, w[p + "attn.v_proj.weight"]), 4, 2, 16), w[p + "attn.o_proj.weight"])
+        n = pm.rms_norm(x, w[p + "n2.weight"], 1e-6)
+        if i == 1:
+            x = x + pm.swiglu_mlp(n, w[p + "ffn.gate_proj.weight"], w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
+            continue
+        logits = pm.linear(n, w[p + "moe.router.weight"])
+        prob = pm.softmax(logits)
+        d = np.zeros_like(x)
+        for t in range(T):
+            e = int(np.argmax(logits[t]))
+            q_ = f"{p}moe.experts.{e}."
+            d[t] = prob[t, e] * pm.swiglu_mlp(n[t:t + 1], w[q_ + "gate_proj.weight"], w[q_ + "up_proj.weight"], w[q_ + "down_proj.weight"])[0]
+        x = x + d
+    return pm.linear(pm.rms_norm(x, w["norm.weight"], 1e-6), w["embed.weight"])
+
+
+def test_a_toy_feed_forward_with_routing_and_another_position_encoding(tmp_path):
+    """Registered here, built from a model description and stepped by the engine, whole and in
+    an unequal batch followed by single tokens, without a change to the library's files; a model
+    with a part that cannot be captured runs its single-token steps kernel by kernel."""
+    from safetensors.torch import load_file
+    cfg = {"architectures": ["ToyRoutedForCausalLM"], "vocab_size": 70, "hidden_size": 48, "n_layers": 3,
+           "torch_dtype": "float32"}
+    folder = L.write_random_model(str(tmp_path / "routed"), cfg, seed=4)
+    w = {k: v.double().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    # spread the router's logits so that the experts in use differ from token to token
+    assert sorted(k for k in w if "router" in k) == ["layers.0.moe.router.weight", "layers.2.moe.router.weight"]
+    eng = L.Engine.from_folder(folder, dtype="float32", max_tokens=512, n_slots=3)
+    assert eng.graphs is None                                           # the routed part decides on the host
+    rng = np.random.default_rng(1)
+    seqs = [rng.integers(0, 70, size=n).tolist() for n in (40, 9, 21)]
+    want = [_plain_routed(w, s, 3) for s in seqs]
+    used = {int(np.argmax(pm.linear(pm.rms_norm(pm.embedding(w["embed.weight"], s), w["layers.0.n2.weight"], 1e-6),
+                                    w["layers.0.moe.router.weight"])[t])) for s in seqs for t in range(len(s))}
+    assert len(used) >= 2                                               # more than one expert is in play
+    slot = eng.alloc_slot()
+    H.close(_np(eng.step([(slot, seqs[0])], want="all")), want[0], "float32", "routed whole")
+    eng.free_slot(slot)
+    slots = [eng.alloc_slot() for _ in seqs]
+    cut = [30, 4, 20]
+    out = _np(eng.step([(sl, s[:c]) for sl, s, c in zip(slots, seqs, cut)], want="all"))
+    H.close(out, np.concatenate([wnt[:c] for wnt, c in zip(want, cut)]), "float32", "routed unequal batch")
+    for t in range(5):
+        live = [i for i in range(3) if cut[i] + t < len(seqs[i])]
+        out = _np(eng.step([(slots[i], [seqs[i][cut[i] + t]]) for i in live], want="last"))
+        H.close(out, np.stack([want[i][cut[i] + t] for i in live]), "float32", f"routed token {t}")
