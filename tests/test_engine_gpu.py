@@ -350,9 +350,9 @@ def test_greedy_generation_through_the_entry_point(name, dtype):
     cfg, w = H.plain(name)
     prompts = [list(H.tokens(name, n, 50 + n)) for n in (5, 17, 1, 32, 8)]
     llm = H.llogos.Llogos(H.folder(name), dtype=dtype, max_context=64, max_batch=3)
-    res = llm.generate(prompts, max_tokens=12, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0,
+    res = llm.generate(prompts, max_tokens=16, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0,
                        stop_tokens=())
-    assert res.batches == [[0, 1, 2], [3, 4]] and all(len(t) == 12 for t in res.tokens)
+    assert res.batches == [[0, 1, 2], [3, 4]] and all(len(t) == 16 for t in res.tokens)
     for p, toks in zip(prompts, res.tokens):
         logits = pm.forward(cfg, w, p + toks)
         for i, t in enumerate(toks):
@@ -361,7 +361,7 @@ def test_greedy_generation_through_the_entry_point(name, dtype):
             assert row.max() - row[t] <= (0 if dtype == "float32" else 2 * H.TOL[dtype]), (name, dtype, i)
     # stop tokens end a sequence and are not emitted
     first = res.tokens[0]
-    res2 = llm.generate([prompts[0]], max_tokens=12, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0,
+    res2 = llm.generate([prompts[0]], max_tokens=16, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0,
                         stop_tokens=(first[4],))
     cut = first.index(first[4])
     assert res2.tokens[0] == first[:cut] and res2.finish_reasons == ["stop"]

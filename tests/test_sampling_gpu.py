@@ -115,3 +115,25 @@ def test_prevent_eos_and_sampled_generation():
     b = llm.generate([prompts[0]], max_tokens=8, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0,
                      stop_tokens=(banned,), prevent_eos=True).tokens[0]
     assert len(b) == 8 and banned not in b
+
+
+def test_sampled_generation_draws_what_the_plain_sampler_draws():
+    """Three prompts of 40 / 3 / 9 tokens, 24 new tokens each at temperature 0.8 with a fixed
+    seed, in float32: along the engine's own token history, every token is the one the plain
+    sampler draws from the plain logits with the same uniform number (the stream depends on
+    seed, request and token index alone)."""
+    rng_mod = importlib.import_module("daisi-llogos_amd.sampling.rng")
+    name = "tiny_b"
+    llm = H.llogos.Llogos(H.folder(name), dtype="float32", max_context=96, max_batch=3)
+    prompts = [list(H.tokens(name, n, 60 + n)) for n in (40, 3, 9)]
+    opts = dict(temperature=0.8, top_k=40, top_p=0.95, repetition_penalty=1.1)
+    got = llm.generate(prompts, max_tokens=24, seed=1234, stop_tokens=(), **opts).tokens
+    cfg, w = H.plain(name)
+    differ = 0
+    for r, (p, toks) in enumerate(zip(prompts, got)):
+        logits = pm.forward(cfg, w, p + toks)
+        for i, t in enumerate(toks):
+            u = rng_mod.uniform(1234, r, i)
+            want = pm.sample(logits[len(p) + i - 1], u, history=p + toks[:i], **opts)
+            differ += int(want != t)
+    assert differ == 0
