@@ -218,6 +218,42 @@ def test_swiglu_part_alone(dtype):
     assert np.abs(_np(got) - want).max() <= TOL[dtype] * max(1.0, np.abs(want).max())
 
 
+@pytest.mark.parametrize("dtype", H.DTYPES)
+def test_block_arrangement_alone(dtype):
+    """The pre-norm block built from its parts: the pending sum handed in is added by the first
+    norm, the mixer's output by the second, and the feed-forward's output is handed on; against
+    the plain layer of the first tiny configuration, a prompt and then a single token."""
+    name = "tiny_a"
+    cfg, w = H.plain(name)
+    rt = P.Runtime(DEV, DT[dtype])
+    models = importlib.import_module("daisi-llogos_amd.models")
+    arch = L.architecture_of(tc.ALL[name])
+    spec = arch.model_spec(arch.read_config(tc.ALL[name]))
+    block = models.model.build_layer(spec.layers[1])
+    from safetensors.torch import load_file
+    tensors = load_file(os.path.join(H.folder(name), "model.safetensors"))
+    block.bind(tensors.get, rt)
+    rng = np.random.default_rng(12)
+    T = 37
+    x0, pend = rng.standard_normal((T + 1, cfg.hidden)), rng.standard_normal((T + 1, cfg.hidden)) * 0.3
+    f = cfg.frequencies()
+    want = pm.decoder_layer(cfg, w, 1, x0 + pend, list(range(T + 1)), f)
+    kv = block.mixer.kv_spec()
+    pool = lambda *shape: torch.zeros((2, kv.n_kv_heads) + shape, dtype=DT[dtype], device=DEV)
+    cache = P.LayerCache(k_pool=pool(64, kv.head_dim), v_pool=pool(kv.head_dim, 64),
+                         table=torch.tensor([[1]], dtype=torch.int32, device=DEV))
+    got = []
+    for lo, hi in ((0, T), (T, T + 1)):
+        x = torch.tensor(x0[lo:hi], dtype=torch.float32, device=DEV)
+        p = torch.tensor(pend[lo:hi], dtype=torch.float32, device=DEV)
+        x_out, pending = block.forward(_ctx(rt, [hi], [hi - lo]), x, p, cache)
+        assert x_out is x                                                # the stream is updated in place
+        got.append(_np(x_out) + _np(K.sum_parts(pending, None, torch.float32)))
+    got = np.concatenate(got)
+    tol = 1e-4 if dtype == "float32" else TOL[dtype] * max(1.0, np.abs(want).max())
+    assert np.abs(got - want).max() <= tol
+
+
 # ---------------------------------------------------------------------------
 # the order of layers is data
 # ---------------------------------------------------------------------------
