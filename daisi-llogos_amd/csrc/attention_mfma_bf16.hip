@@ -231,7 +231,7 @@ __host__ __device__ constexpr size_t decode_lds_bytes(int waves, int group, int 
     return (size_t)waves * (group * (hd + 1) + 32) * sizeof(float);
 }
 
-// The fused form (FUSED, head size 128 rotated whole with split-half pairing) starts from the
+// The fused form (FUSED, head size 64 or 128 rotated whole with split-half pairing) starts from the
 // projection itself: a block first makes its queries (sum of the projection's partial products,
 // bias, per-head norm, rotation) into LDS, and the block whose pages hold the step's position
 // also makes the step's key and value and writes them to their page, which the rotation kernel
@@ -241,11 +241,11 @@ struct QkvSource {
     int parts;
     size_t part_stride;
     int row_stride;
-    const float* bias;         // [(heads + 2 kv heads) * 128] or null
-    const float* q_norm_w;     // [128] or null
+    const float* bias;         // [(heads + 2 kv heads) * head size] or null
+    const float* q_norm_w;     // [head size] or null
     const float* k_norm_w;
     float eps;
-    const float2* cs;          // [batch][64] (cos, sin) of each sequence's position
+    const float2* cs;          // [batch][head size / 2] (cos, sin) of each sequence's position
     bf16_t* k_pool;            // the pools, writable
     bf16_t* v_pool;
 };
@@ -272,10 +272,13 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_decode_kernel(
     if (FUSED) {
         // items 0 .. group - 1: the kv head's query heads; then, in the block that holds the
         // step's position, its key and its value.  A wave takes an item; lane l holds
-        // dimensions 2 l and 2 l + 1, the rotation partner (64 dimensions away) is lane l ^ 32.
+        // dimensions PER l .. PER l + PER - 1 (two for head size 128, one for 64), and the
+        // rotation partner, HD / 2 dimensions away, is lane l ^ 32.
+        constexpr int PER = HD / kWave;
+        static_assert(PER == 1 || PER == 2, "head sizes 64 and 128");
         const bool writer = (n_pages - 1) / WAVES == z;
         const int items = group + (writer ? 2 : 0);
-        const int d = 2 * lane;
+        const int d = PER * lane;
         const size_t page_base = writer
             ? ((size_t)table[(size_t)b * table_stride + n_pages - 1] * n_kv_heads + kvh) * kPageTokens * HD : 0;
         for (int item = wave; item < items; item += WAVES) {
@@ -283,39 +286,52 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_decode_kernel(
             const int head = is_q ? kvh * group + item : (is_k ? n_heads + kvh : n_heads + n_kv_heads + kvh);
             const size_t col = (size_t)head * HD + d;
             const float* p = src.qkv + (size_t)b * src.row_stride + col;
-            float2 x = *reinterpret_cast<const float2*>(p);
+            float x[PER];
+#pragma unroll
+            for (int e = 0; e < PER; ++e) x[e] = p[e];
             for (int part0 = 1; part0 < src.parts; part0 += 8) {     // eight loads in flight, added in ascending order
-                float2 y[8];
+                float y[8][PER];
 #pragma unroll
                 for (int j = 0; j < 8; ++j)
-                    y[j] = part0 + j < src.parts ? *reinterpret_cast<const float2*>(p + (part0 + j) * src.part_stride)
-                                                 : float2{0.f, 0.f};
+#pragma unroll
+                    for (int e = 0; e < PER; ++e)
+                        y[j][e] = part0 + j < src.parts ? p[(part0 + j) * src.part_stride + e] : 0.f;
 #pragma unroll
                 for (int j = 0; j < 8; ++j)
-                    if (part0 + j < src.parts) { x.x += y[j].x; x.y += y[j].y; }
+                    if (part0 + j < src.parts) {
+#pragma unroll
+                        for (int e = 0; e < PER; ++e) x[e] += y[j][e];
+                    }
             }
-            if (src.bias) { x.x += src.bias[col]; x.y += src.bias[col + 1]; }
+            if (src.bias) {
+#pragma unroll
+                for (int e = 0; e < PER; ++e) x[e] += src.bias[col + e];
+            }
             if (!is_q && !is_k) {
                 bf16_t* vdst = src.v_pool + page_base + (pos % kPageTokens);
-                vdst[(size_t)d * kPageTokens] = f32_to_bf16(x.x);
-                vdst[(size_t)(d + 1) * kPageTokens] = f32_to_bf16(x.y);
+#pragma unroll
+                for (int e = 0; e < PER; ++e) vdst[(size_t)(d + e) * kPageTokens] = f32_to_bf16(x[e]);
                 continue;
             }
             const float* norm_w = is_q ? src.q_norm_w : src.k_norm_w;
             if (norm_w) {
-                const float ss = wave_sum(x.x * x.x + x.y * x.y);
-                const float inv = 1.0f / sqrtf(ss / (float)HD + src.eps);
-                x.x = x.x * inv * norm_w[d];
-                x.y = x.y * inv * norm_w[d + 1];
+                float sq = 0.f;
+#pragma unroll
+                for (int e = 0; e < PER; ++e) sq += x[e] * x[e];
+                const float inv = 1.0f / sqrtf(wave_sum(sq) / (float)HD + src.eps);
+#pragma unroll
+                for (int e = 0; e < PER; ++e) x[e] = x[e] * inv * norm_w[d + e];
             }
-            const float p0 = __shfl_xor(x.x, 32, kWave), p1 = __shfl_xor(x.y, 32, kWave);
-            const float2 c0 = src.cs[(size_t)b * 64 + (d & 63)], c1 = src.cs[(size_t)b * 64 + (d & 63) + 1];
-            float y0, y1;
-            if (lane < 32) { y0 = x.x * c0.x - p0 * c0.y; y1 = x.y * c1.x - p1 * c1.y; }
-            else           { y0 = p0 * c0.y + x.x * c0.x; y1 = p1 * c1.y + x.y * c1.x; }
-            const uint32_t packed = (uint32_t)f32_to_bf16(y0) | ((uint32_t)f32_to_bf16(y1) << 16);
-            if (is_q) *reinterpret_cast<uint32_t*>(&q_lds[item][d]) = packed;
-            else *reinterpret_cast<uint32_t*>(src.k_pool + page_base + (size_t)(pos % kPageTokens) * HD + d) = packed;
+            bf16_t y[PER];
+#pragma unroll
+            for (int e = 0; e < PER; ++e) {
+                const float partner = __shfl_xor(x[e], 32, kWave);
+                const float2 c = src.cs[(size_t)b * (HD / 2) + ((d + e) & (HD / 2 - 1))];
+                y[e] = f32_to_bf16(lane < 32 ? x[e] * c.x - partner * c.y : partner * c.y + x[e] * c.x);
+            }
+            bf16_t* dst = is_q ? &q_lds[item][d] : src.k_pool + page_base + (size_t)(pos % kPageTokens) * HD + d;
+#pragma unroll
+            for (int e = 0; e < PER; ++e) dst[e] = y[e];
         }
         __syncthreads();          // the queries in LDS, and the key and value in memory, for every wave of the block
     }
@@ -746,7 +762,8 @@ static int launch_decode(void* out, const void* q, int q_stride, const QkvSource
                                                                         n_z, W); } while (0)
 #define BY_WAVES(HD, FUSED) do { if (waves == 16) GO(HD, 16, FUSED); else if (waves == 8) GO(HD, 8, FUSED); \
                                  else GO(HD, 4, FUSED); } while (0)
-    if (src != nullptr) BY_WAVES(128, true);
+    if (src != nullptr && head_dim == 64) BY_WAVES(64, true);
+    else if (src != nullptr) BY_WAVES(128, true);
     else if (head_dim == 64) BY_WAVES(64, false);
     else BY_WAVES(128, false);
 #undef BY_WAVES
@@ -764,8 +781,8 @@ LLOGOS_EXPORT int llogos_attn_decode_bf16(void* out, const void* q, int q_stride
                          n_heads, n_kv_heads, head_dim, scale, window, sinks, workspace, workspace_floats, stream);
 }
 
-// The same from the fused projection (see QkvSource): head size 128 only; also writes the
-// step's keys and values to their pages.  cs: [batch][64][2] floats.
+// The same from the fused projection (see QkvSource): head sizes 64 and 128; also writes the
+// step's keys and values to their pages.  cs: [batch][head size / 2][2] floats.
 LLOGOS_EXPORT int llogos_attn_decode_fused_bf16(void* out, const float* qkv, int parts, long long part_stride,
                                                 int row_stride, const float* bias, const float* q_norm_w,
                                                 const float* k_norm_w, float eps, const void* cs, void* k_pool,
@@ -773,7 +790,7 @@ LLOGOS_EXPORT int llogos_attn_decode_fused_bf16(void* out, const float* qkv, int
                                                 const int* tok_pos, int batch, int n_heads, int n_kv_heads,
                                                 int head_dim, float scale, int window, int sinks, float* workspace,
                                                 long long workspace_floats, hipStream_t stream) {
-    if (head_dim != 128) return LLOGOS_UNSUPPORTED;
+    if (head_dim != 128 && head_dim != 64) return LLOGOS_UNSUPPORTED;
     if (parts < 1 || (row_stride % 2) || (part_stride % 2) || ((uintptr_t)qkv % 8) ||
         row_stride < (n_heads + 2 * n_kv_heads) * head_dim)
         return LLOGOS_BAD_ARGUMENT;

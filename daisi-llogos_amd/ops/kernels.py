@@ -593,10 +593,10 @@ def attention_decode_fused(ctx, qkv: torch.Tensor, bias: Optional[torch.Tensor],
                            sinks: int = 0) -> Optional[torch.Tensor]:
     """A single-token step's attention straight from the fused projection rows [q | k | v]
     (float32 [T, W] or partial sums [parts, T, W]): bias, per-head norm, rotation and the cache
-    write happen inside the attention kernel.  For bfloat16 caches, head size 128 rotated whole
-    with split-half pairing; None for anything else (the caller then runs the steps apart)."""
-    if not (ctx.is_decode and qkv.dtype == torch.float32 and k_pool.dtype == torch.bfloat16 and head_dim == 128
-            and rot == 128 and pairing == 0 and n_heads % n_kv_heads == 0 and n_heads // n_kv_heads <= 16):
+    write happen inside the attention kernel.  For bfloat16 caches, head sizes 64 and 128 rotated
+    whole with split-half pairing; None for anything else (the caller then runs the steps apart)."""
+    if not (ctx.is_decode and qkv.dtype == torch.float32 and k_pool.dtype == torch.bfloat16 and head_dim in (64, 128)
+            and rot == head_dim and pairing == 0 and n_heads % n_kv_heads == 0 and n_heads // n_kv_heads <= 16):
         return None
     parts, part_stride = _parts(qkv)
     T = qkv.shape[-2]

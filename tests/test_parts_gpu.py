@@ -145,14 +145,15 @@ def test_attention_part_alone(dtype, nh, nkv, hd, bias, qk_norm, window):
     assert np.abs(got - want).max() <= TOL[dtype] * max(1.0, np.abs(want).max())
 
 
+@pytest.mark.parametrize("hd", [128, 64])
 @pytest.mark.parametrize("nh,nkv,bias,qk_norm,window", [(8, 2, True, True, 0), (16, 1, False, False, 0),
                                                         (5, 5, False, True, 70), (12, 4, True, False, 0)])
-def test_single_token_steps_from_the_projection_in_one_kernel(nh, nkv, bias, qk_norm, window, monkeypatch):
-    """Head size 128 in bfloat16: the attention kernel that makes its queries and the step's key
-    and value from the projection itself gives, bit for bit, the outputs and the cache pages of
-    the rotation kernel followed by the attention kernel, across a page's end, and both agree
-    with the plain parts."""
-    dtype, hd, hidden = "bfloat16", 128, 72
+def test_single_token_steps_from_the_projection_in_one_kernel(nh, nkv, bias, qk_norm, window, hd, monkeypatch):
+    """Head sizes 128 and 64 in bfloat16: the attention kernel that makes its queries and the
+    step's key and value from the projection itself gives, bit for bit, the outputs and the cache
+    pages of the rotation kernel followed by the attention kernel, across a page's end, and both
+    agree with the plain parts."""
+    dtype, hidden = "bfloat16", 72
     rng = np.random.default_rng(nh)
     rt = P.Runtime(DEV, DT[dtype])
     att = P.Attention("a.", hidden, nh, nkv, hd, P.Rotary(hd, hd, 1e4), bias=bias, qk_norm=qk_norm, eps=1e-5,
