@@ -50,6 +50,67 @@ def test_replay_of_two_batches(tmp_path, dtype):
     H.close(read(4), pc[[0, 39]], dtype, "step 4")
 
 
+@pytest.mark.parametrize("dtype", H.DTYPES)
+@pytest.mark.parametrize("name", ["tiny_c", "tiny_d"])
+def test_the_same_requests_whole_token_by_token_and_in_unequal_batches(tmp_path, name, dtype):
+    """Three requests replayed three ways through the program: each alone and whole; each alone
+    with its last 32 tokens one by one; and as batches of unequal lengths whose shorter requests
+    end earlier, a second batch taking the slots of the first.  Every way against the plain
+    implementation, and the ways against each other."""
+    import tiny_configs as tc
+    vocab = tc.ALL[name]["vocab_size"]
+    reqs = {"a": H.tokens(name, 100, 11), "b": H.tokens(name, 45, 12), "c": H.tokens(name, 70, 13)}
+    plain = {k: H.plain_logits(name, v) for k, v in reqs.items()}
+
+    def replay(steps, max_tokens, tag):
+        out = str(tmp_path / tag)
+        lines = _run(H.folder(name), dtype, steps, out, max_tokens)
+        assert [l for l in lines if l] == [f"done {s['step']}" for s in steps]
+        got = {k: np.full((len(v), vocab), np.nan) for k, v in reqs.items()}
+        fed = {k: 0 for k in reqs}
+        for s in steps:
+            rows = np.fromfile(os.path.join(out, f"{s['step']}.f32"), dtype="<f4").reshape(-1, vocab) if any(e["want"] for e in s["entries"]) else None
+            o = 0
+            for e in s["entries"]:
+                for w_ in e["want"]:
+                    got[e["id"]][fed[e["id"]] + w_] = rows[o]
+                    o += 1
+                fed[e["id"]] += len(e["tokens"])
+        return got
+
+    # 1. whole, one request after the other
+    steps = [{"step": i, "entries": [{"id": k, "tokens": list(v), "want": list(range(len(v)))}], "end": [k]}
+             for i, (k, v) in enumerate(reqs.items())]
+    whole = replay(steps, 128, "whole")
+    # 2. the last 32 tokens one by one
+    steps, n = [], 0
+    for k, v in reqs.items():
+        cut = len(v) - 32
+        steps.append({"step": n, "entries": [{"id": k, "tokens": list(v[:cut]), "want": list(range(cut))}], "end": []}); n += 1
+        for t in range(cut, len(v)):
+            steps.append({"step": n, "entries": [{"id": k, "tokens": [v[t]], "want": [0]}], "end": [k] if t == len(v) - 1 else []}); n += 1
+    single = replay(steps, 128, "single")
+    # 3. unequal batches: a and b start together with prompts of 60 and 40 tokens, then one token each; b ends
+    #    first; then c and a copy of b ("b2") as a second batch in the slots and pages that came back
+    steps, n = [], 0
+    steps.append({"step": n, "entries": [{"id": "a", "tokens": list(reqs["a"][:60]), "want": list(range(60))},
+                                         {"id": "b", "tokens": list(reqs["b"][:40]), "want": list(range(40))}], "end": []}); n += 1
+    for t in range(40):
+        entries = [{"id": "a", "tokens": [reqs["a"][60 + t]], "want": [0]}]
+        if t < 5:
+            entries.append({"id": "b", "tokens": [reqs["b"][40 + t]], "want": [0]})
+        steps.append({"step": n, "entries": entries, "end": (["b"] if t == 4 else []) + (["a"] if t == 39 else [])}); n += 1
+    steps.append({"step": n, "entries": [{"id": "c", "tokens": list(reqs["c"][:69]), "want": list(range(69))}], "end": []}); n += 1
+    steps.append({"step": n, "entries": [{"id": "c", "tokens": [reqs["c"][69]], "want": [0]}], "end": ["c"]}); n += 1
+    batched = replay(steps, 192, "batched")
+    tol = 2e-5 if dtype == "float32" else H.TOL[dtype]
+    for k in reqs:
+        for way, got in (("whole", whole), ("token by token", single), ("batched", batched)):
+            assert not np.isnan(got[k]).any(), (k, way)
+            H.close(got[k], plain[k], dtype, f"{name} {k} {way}")
+        assert np.abs(whole[k] - single[k]).max() <= tol and np.abs(whole[k] - batched[k]).max() <= tol
+
+
 def test_replay_refuses_more_than_the_cache_holds(tmp_path):
     steps = [{"step": 0, "entries": [{"id": "a", "tokens": list(range(65)), "want": []}], "end": []}]
     cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", H.folder("tiny_a"),
