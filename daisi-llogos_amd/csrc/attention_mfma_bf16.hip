@@ -543,7 +543,12 @@ void attn_prefill_lds_kernel(
     // head) pair one after the other, so that the pair's pages stay in its L2, and the pairs go
     // from the last tile to the first: late tiles of a causal prompt see the most keys, and
     // starting with them keeps the compute units evenly busy to the end.
-    const int m_xcd = blockIdx.x / 8, xcd = blockIdx.x % 8;
+    // A grid of at most two blocks per compute unit starts all at once, and the m-th and the
+    // (m + 32)-th block of an XCD share a compute unit: the second half runs in rising order
+    // then, so that the longest block shares with the shortest.
+    int m_xcd = blockIdx.x / 8;
+    const int xcd = blockIdx.x % 8, per_xcd = gridDim.x / 8;
+    if (per_xcd > 32 && per_xcd <= 64 && m_xcd >= 32) m_xcd = per_xcd - 1 - (m_xcd - 32);
     const int pair = (m_xcd / group) * 8 + xcd;
     if (pair >= n_tiles * n_kv_heads) return;
     const int kvh = pair % n_kv_heads, h = kvh * group + m_xcd % group;

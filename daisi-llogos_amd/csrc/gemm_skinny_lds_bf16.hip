@@ -1,4 +1,4 @@
-// out[M, N] = a[M, K] . w[N, K]^T for few rows (M <= 64), second form: the activations are
+// out[M, N] = a[M, K] . w[N, K]^T for few rows (M <= 128), second form: the activations are
 // staged in LDS and shared by all waves of a block.
 //
 // The address path of a compute unit handles a fixed number of lanes per clock, so in the
@@ -25,6 +25,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 constexpr int kLdsWaves = 4;                 // waves per block (8 measured no faster)
 constexpr int kChunkK = 256;                 // values of k per LDS chunk (128 and 512 measured no faster)
 constexpr int kChunkSteps = kChunkK / 32;    // MFMA steps per chunk
+constexpr int kLdsMaxRows = 128;            // rows of activations (64 with a fused producer)
 constexpr int kRowPad = 8;                   // bf16 of padding per LDS row (16 bytes)
 
 enum { PRODUCE_PLAIN = 0, PRODUCE_SWIGLU_F32 = 1, PRODUCE_SWIGLU_BF16 = 2 };
@@ -82,23 +83,26 @@ __device__ __forceinline__ uint4 produce8(const ActSource& src, int m, int k, in
     }
 }
 
-template <int RB, int MB, int MODE, typename TO>
+template <int RB, int MB, int MODE, typename TO, int CHUNK>
 __global__ __launch_bounds__(kLdsWaves * kWave) void gemm_skinny_lds_kernel(
         TO* __restrict__ out, ActSource src, const bf16_t* __restrict__ w, const float* __restrict__ bias,
-        int M, int N, int K, int ldo, size_t part_stride, int k_per_block) {
+        int M, int N, int K, int ldo, size_t part_stride, int k_per_block, int parts) {
     constexpr int kRows = MB * 16;
-    constexpr int kRowLen = kChunkK + kRowPad;
-    constexpr int kPieces = kRows * (kChunkK / 8);                    // 16-byte pieces of a chunk
+    constexpr int kRowLen = CHUNK + kRowPad;
+    constexpr int kPieces = kRows * (CHUNK / 8);                    // 16-byte pieces of a chunk
     constexpr int kPiecesPerThread = (kPieces + kLdsWaves * kWave - 1) / (kLdsWaves * kWave);
     __shared__ __attribute__((aligned(16))) bf16_t lds[2][kRows][kRowLen];
 
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int r = lane & 15, g = lane >> 4;
-    const int split = blockIdx.y;
-    const int n0 = (blockIdx.x * kLdsWaves + wave) * (16 * RB);
+    // Blocks go to the 8 XCDs in turn, each with an L2 of its own: a block's part of k is its
+    // index modulo the parts, so that an XCD sees few parts and its L2 keeps their activations
+    // (with 8 parts one each) while the weights stream through.
+    const int split = blockIdx.x % parts, n_block = blockIdx.x / parts;
+    const int n0 = (n_block * kLdsWaves + wave) * (16 * RB);
     const int k_begin = split * k_per_block;
     const int k_end = min(K, k_begin + k_per_block);
-    const int n_chunks = (k_end - k_begin + kChunkK - 1) / kChunkK;
+    const int n_chunks = (k_end - k_begin + CHUNK - 1) / CHUNK;
 
     const bf16_t* wrow[RB];
 #pragma unroll
@@ -116,7 +120,7 @@ __global__ __launch_bounds__(kLdsWaves * kWave) void gemm_skinny_lds_kernel(
 #pragma unroll
         for (int i = 0; i < kPiecesPerThread; ++i) {
             const int piece = i * (kLdsWaves * kWave) + threadIdx.x;
-            const int m = piece / (kChunkK / 8), kk = k0 + (piece % (kChunkK / 8)) * 8;
+            const int m = piece / (CHUNK / 8), kk = k0 + (piece % (CHUNK / 8)) * 8;
             stage[i] = make_uint4(0, 0, 0, 0);
             if (piece < kPieces && m < M && kk < k_end) stage[i] = produce8<MODE>(src, m, kk, K);
         }
@@ -126,13 +130,13 @@ __global__ __launch_bounds__(kLdsWaves * kWave) void gemm_skinny_lds_kernel(
         for (int i = 0; i < kPiecesPerThread; ++i) {
             const int piece = i * (kLdsWaves * kWave) + threadIdx.x;
             if (piece < kPieces)
-                *reinterpret_cast<uint4*>(&lds[buf][piece / (kChunkK / 8)][(piece % (kChunkK / 8)) * 8]) = stage[i];
+                *reinterpret_cast<uint4*>(&lds[buf][piece / (CHUNK / 8)][(piece % (CHUNK / 8)) * 8]) = stage[i];
         }
     };
-    bf16x8 wf0[kChunkSteps][RB], wf1[kChunkSteps][RB];
-    auto fetch_w = [&](bf16x8 (&wf)[kChunkSteps][RB], int k0) {
+    bf16x8 wf0[(CHUNK / 32)][RB], wf1[(CHUNK / 32)][RB];
+    auto fetch_w = [&](bf16x8 (&wf)[(CHUNK / 32)][RB], int k0) {
 #pragma unroll
-        for (int s = 0; s < kChunkSteps; ++s) {
+        for (int s = 0; s < (CHUNK / 32); ++s) {
             const int kk = k0 + s * 32 + g * 8;
             const bool ok = kk < k_end;                                   // K % 8 == 0
 #pragma unroll
@@ -143,9 +147,9 @@ __global__ __launch_bounds__(kLdsWaves * kWave) void gemm_skinny_lds_kernel(
             }
         }
     };
-    auto multiply = [&](const bf16x8 (&wf)[kChunkSteps][RB], int buf) {
+    auto multiply = [&](const bf16x8 (&wf)[(CHUNK / 32)][RB], int buf) {
 #pragma unroll
-        for (int s = 0; s < kChunkSteps; ++s) {
+        for (int s = 0; s < (CHUNK / 32); ++s) {
             bf16x8 af[MB];
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb)
@@ -165,13 +169,13 @@ __global__ __launch_bounds__(kLdsWaves * kWave) void gemm_skinny_lds_kernel(
         __syncthreads();
     }
     for (int c = 0; c < n_chunks; c += 2) {
-        const int k0 = k_begin + c * kChunkK;
+        const int k0 = k_begin + c * CHUNK;
         const bool has1 = c + 1 < n_chunks, has2 = c + 2 < n_chunks;
-        if (has1) { fetch_acts(k0 + kChunkK); fetch_w(wf1, k0 + kChunkK); }
+        if (has1) { fetch_acts(k0 + CHUNK); fetch_w(wf1, k0 + CHUNK); }
         multiply(wf0, 0);
         if (has1) store_acts(1);
         __syncthreads();
-        if (has2) { fetch_acts(k0 + 2 * kChunkK); fetch_w(wf0, k0 + 2 * kChunkK); }
+        if (has2) { fetch_acts(k0 + 2 * CHUNK); fetch_w(wf0, k0 + 2 * CHUNK); }
         if (has1) multiply(wf1, 1);
         if (has2) store_acts(0);
         __syncthreads();
@@ -203,16 +207,16 @@ LLOGOS_EXPORT int llogos_gemm_skinny_lds_parts(int K, int splits) {
     return (K + kpb - 1) / kpb;
 }
 
-template <int RB, int MB, int MODE>
+template <int RB, int MB, int MODE, int CHUNK = kChunkK>
 static int launch_lds(void* out, int out_dtype, const ActSource& src, const bf16_t* w, const float* bias,
                       int M, int N, int K, int ldo, size_t part_stride, int kpb, int parts, hipStream_t stream) {
-    dim3 grid((N + 16 * RB * kLdsWaves - 1) / (16 * RB * kLdsWaves), parts);
+    const int n_blocks = (N + 16 * RB * kLdsWaves - 1) / (16 * RB * kLdsWaves);
     if (out_dtype == DT_BF16)
-        gemm_skinny_lds_kernel<RB, MB, MODE, bf16_t><<<grid, kLdsWaves * kWave, 0, stream>>>(
-            (bf16_t*)out, src, w, bias, M, N, K, ldo, part_stride, kpb);
+        gemm_skinny_lds_kernel<RB, MB, MODE, bf16_t, CHUNK><<<n_blocks * parts, kLdsWaves * kWave, 0, stream>>>(
+            (bf16_t*)out, src, w, bias, M, N, K, ldo, part_stride, kpb, parts);
     else
-        gemm_skinny_lds_kernel<RB, MB, MODE, float><<<grid, kLdsWaves * kWave, 0, stream>>>(
-            (float*)out, src, w, bias, M, N, K, ldo, part_stride, kpb);
+        gemm_skinny_lds_kernel<RB, MB, MODE, float, CHUNK><<<n_blocks * parts, kLdsWaves * kWave, 0, stream>>>(
+            (float*)out, src, w, bias, M, N, K, ldo, part_stride, kpb, parts);
     return LLOGOS_LAUNCH_CHECK();
 }
 
@@ -228,8 +232,9 @@ LLOGOS_EXPORT int llogos_gemm_skinny_lds_bf16(void* out, int out_dtype, const vo
     if (M <= 0 || N <= 0 || K <= 0 || ldo < N || splits < 1 || act_parts < 1) return LLOGOS_BAD_ARGUMENT;
     if (out_dtype != DT_BF16 && out_dtype != DT_F32) return LLOGOS_BAD_ARGUMENT;
     if (mode < PRODUCE_PLAIN || mode > PRODUCE_SWIGLU_BF16) return LLOGOS_BAD_ARGUMENT;
-    if (M > 64 || (K % 8) || (lda % 8) || ((uintptr_t)act % 16) || ((uintptr_t)w % 16) || (act_part_stride % 4))
+    if (M > kLdsMaxRows || (K % 8) || (lda % 8) || ((uintptr_t)act % 16) || ((uintptr_t)w % 16) || (act_part_stride % 4))
         return LLOGOS_UNSUPPORTED;
+    if (M > 64 && mode != PRODUCE_PLAIN) return LLOGOS_UNSUPPORTED;
     if (mode == PRODUCE_PLAIN ? lda < K : lda < 2 * K) return LLOGOS_BAD_ARGUMENT;
     const int parts = llogos_gemm_skinny_lds_parts(K, splits);
     if (parts > 1 && (out_dtype != DT_F32 || bias != nullptr || part_stride < (long long)M * ldo))
@@ -243,6 +248,11 @@ LLOGOS_EXPORT int llogos_gemm_skinny_lds_bf16(void* out, int out_dtype, const vo
 #define BY_MODE(RB, MB) do { if (mode == PRODUCE_PLAIN) GO(RB, MB, PRODUCE_PLAIN); \
                              if (mode == PRODUCE_SWIGLU_F32) GO(RB, MB, PRODUCE_SWIGLU_F32); \
                              GO(RB, MB, PRODUCE_SWIGLU_BF16); } while (0)
+    // 65 to 128 rows: chunks of 128 values of k, so that two blocks' activations fit a compute unit's LDS
+    if (mb > 6) { if (row_blocks >= 2) return launch_lds<2, 8, PRODUCE_PLAIN, 128>(out, out_dtype, src, W, bias, M, N, K, ldo, (size_t)part_stride, kpb, parts, stream);
+                  return launch_lds<1, 8, PRODUCE_PLAIN, 128>(out, out_dtype, src, W, bias, M, N, K, ldo, (size_t)part_stride, kpb, parts, stream); }
+    if (mb > 4) { if (row_blocks >= 2) return launch_lds<2, 6, PRODUCE_PLAIN, 128>(out, out_dtype, src, W, bias, M, N, K, ldo, (size_t)part_stride, kpb, parts, stream);
+                  return launch_lds<1, 6, PRODUCE_PLAIN, 128>(out, out_dtype, src, W, bias, M, N, K, ldo, (size_t)part_stride, kpb, parts, stream); }
     if (mb == 1) { if (row_blocks >= 2) BY_MODE(2, 1); BY_MODE(1, 1); }
     if (mb == 2) { if (row_blocks >= 2) BY_MODE(2, 2); BY_MODE(1, 2); }
     if (row_blocks >= 2) BY_MODE(2, 4);

@@ -131,14 +131,44 @@ def test_gemm_few_rows_on_the_matrix_cores(M, N, K_):
     assert K.gemm_skinny_bf16(a[:, :K_ - 4], w[:, :K_ - 4].contiguous(), None, torch.float32) is None   # k % 8
 
 
+@pytest.mark.parametrize("M,N,K_", [(65, 257, 2048), (96, 4096, 14336), (97, 100, 1000), (128, 5120, 17408), (111, 333, 72)])
+def test_gemm_of_65_to_128_rows_on_the_matrix_cores(M, N, K_):
+    """The LDS few-row product at 65 to 128 rows: every number of blocks along k and both widths
+    of a wave's strip of w; a row's result is the same bit for bit for every batch of this class."""
+    rng = np.random.default_rng(8)
+    a = _t(rng.standard_normal((M, K_)), torch.bfloat16)
+    w = _t(rng.standard_normal((N, K_)) * 0.05, torch.bfloat16)
+    b = _t(rng.standard_normal(N))
+    want = pm.linear(_np(a), _np(w))
+    scale = np.abs(want).max()
+    for splits in (1, 3, 8):
+        for rb in (1, 2):
+            out = K.gemm_skinny_lds_bf16(a, w, None, torch.float32, splits, rb)
+            assert out is not None and out.dtype == torch.float32 and out.shape[1:] == (M, N)
+            assert np.abs(_np(out).sum(0) - want).max() <= 2e-6 * scale * math.sqrt(K_)
+    out = K.gemm_skinny_lds_bf16(a, w, b, torch.bfloat16, 1, 1)
+    assert np.abs(_np(out)[0] - (want + _np(b))).max() <= 1e-2 * scale
+    assert K.gemm_skinny_lds_bf16(torch.cat([a, a]), w, None, torch.float32, 1, 1) is None            # more than 128 rows
+    assert K.gemm_skinny_lds_bf16(a.float().repeat(1, 2), w, None, torch.float32, 1, 1, swiglu=True) is None  # fused producer: 64 rows
+    prod = K.gemm_product(a, w, torch.bfloat16, f32_ok=True)
+    assert (prod.dim() == 3) == (K.long_inner(w) and K.lds_splits(M, N, K_) > 1)
+    many = K.sum_parts(prod, None, torch.float32)
+    assert np.abs(_np(many) - want).max() <= (1e-5 if prod.dtype == torch.float32 else 1e-2) * scale
+    if K.long_inner(w):
+        few = K.sum_parts(K.gemm_product(a[:65], w, torch.bfloat16, f32_ok=True), None, torch.float32)
+        assert torch.equal(few, many[:65])
+
+
 def test_products_of_random_shapes_through_the_dispatch():
     """Whatever kernel and split of k the plan picks for a shape, the product is right: row
     counts up to 64 and beyond, widths and depths that are multiples of 8 and of nothing else."""
     rng = np.random.default_rng(21)
     for case in range(40):
-        M = int(rng.choice([1, 2, 5, 8, 13, 16, 17, 31, 33, 64, 70]))
+        M = int(rng.choice([1, 2, 5, 8, 13, 16, 17, 31, 33, 64, 70, 100, 128, 130]))
         K_ = 8 * int(rng.integers(1, 1100))                                # up to 8,792
         N = int(rng.integers(1, 40000)) if case % 4 else int(rng.integers(16384, 72000))
+        if case % 5 == 3:
+            N = int(rng.integers(1, K_ // 2 + 2))                           # few rows of w for its length
         a = _t(rng.standard_normal((M, K_)), torch.bfloat16)
         w = torch.randn((N, K_), device=DEV, dtype=torch.bfloat16, generator=torch.Generator(device=DEV).manual_seed(case)) * 0.05
         b = _t(rng.standard_normal(N))
