@@ -530,13 +530,11 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dty
                 out += bias.to(torch.bfloat16)
             return out
         elif out_dtype == torch.float32 and a.is_contiguous() and a.shape[1] % 8 == 0:
-            # float32 results for many rows: row blocks through the hand-written kernel
-            out = torch.empty((M, w.shape[0]), dtype=torch.float32, device=a.device)
-            for r in range(0, M, SKINNY_MAX_ROWS):
-                blk = gemm_skinny_lds_bf16(a[r:r + SKINNY_MAX_ROWS], w, bias, torch.float32, 1, 1)
-                if blk is None:
-                    return gemm_generic(a, w, bias, out_dtype)
-                out[r:r + SKINNY_MAX_ROWS] = blk[0]
+            # float32 results for many rows (the logits of many positions): the library's product
+            # with float32 accumulation and output, one pass over w
+            out = torch.mm(a, w.t(), out_dtype=torch.float32)
+            if bias is not None:
+                out += bias
             return out
     return gemm_generic(a, w, bias, out_dtype)
 
