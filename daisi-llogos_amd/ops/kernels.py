@@ -288,8 +288,8 @@ def lds_splits(M: int, N: int, K: int, n_cus: int = 256) -> int:
     how evenly the blocks fill the compute units (544 blocks on 256 units run as long as 768),
     whether there are enough of them to keep the memory system busy (about 1.5 a unit), and the
     float32 partial sums every further block along k writes and the consumer reads (they cost
-    about 6 M / K of the weights' time each).  64 rows of activations leave LDS for two blocks a
-    unit, so blocks come in rounds of twice the units there.  More blocks along k are taken only
+    about 6 M / K of the weights' time each).  64 and more rows of activations leave LDS for two
+    blocks a unit, so blocks come in rounds of twice the units there.  More blocks along k are taken only
     for a clear gain (8 %), since they also cost the consumer a fused form or a launch."""
     n_blocks = -(-N // 64)
     chunks = -(-K // 256)
