@@ -210,6 +210,31 @@ def test_layer_sizes_of_large_models(name, dtype):
     H.close(out, np.stack([pa[149], pb[67]]), dtype, f"{name}: a continued prompt beside a single token")
 
 
+@pytest.mark.parametrize("dtype", H.DTYPES)
+@pytest.mark.parametrize("name", ["tiny_c", "layer_8b"])
+def test_batches_of_more_than_64_sequences(name, dtype):
+    """100 sequences with prompts of 3 to 9 tokens in one step, then one token each while a third
+    of them ends early: beyond the batch sizes whose steps are captured, where the products take
+    other kernels (the library's, and the few-row product in its form for 65 to 128 rows)."""
+    n = 100
+    base = [H.tokens(name, 13, 40 + j) for j in range(5)]
+    plain = [H.plain_logits(name, b) for b in base]
+    eng = H.engine(name, dtype, max_tokens=64 * n, n_slots=n)
+    slots = [eng.alloc_slot() for _ in range(n)]
+    seq, plen = [i % 5 for i in range(n)], [3 + i % 7 for i in range(n)]
+    out = _np(eng.step([(slots[i], base[seq[i]][:plen[i]]) for i in range(n)], want="last"))
+    H.close(out, np.stack([plain[seq[i]][plen[i] - 1] for i in range(n)]), dtype, f"{name}: 100 prompts")
+    live = list(range(n))
+    for t in range(4):
+        out = _np(eng.step([(slots[i], [base[seq[i]][plen[i] + t]]) for i in live], want="last"))
+        H.close(out, np.stack([plain[seq[i]][plen[i] + t] for i in live]), dtype, f"{name}: token {t} of {len(live)} sequences")
+        if t == 0:
+            for i in live[::3]:
+                eng.free_slot(slots[i])
+            live = [i for i in live if i % 3]
+    assert len(live) == 66
+
+
 def test_step_errors():
     eng = H.engine("tiny_a", "float32", max_tokens=128, n_slots=2)
     s = eng.alloc_slot()
