@@ -1,0 +1,106 @@
+"""The whole Llama-3.1-8B configuration (32 layers, vocabulary 128256) with random weights
+against the plain implementation: requests whole, the last tokens one by one, and an unequal
+batch, in float32 (1e-4 absolute) and in bfloat16.  It writes a 16 GB model folder and holds
+the weights in float64 on the host (about 80 GB), so it runs only when LLOGOS_FULL_SIZE=1 is
+set; a minute on the GPU box.
+
+At this depth the bfloat16 engine's distance from float64 arithmetic is set by where values
+are rounded to bfloat16 (normed rows, rotated queries and keys, values, probabilities, the
+attention's output, the gate/up product, silu(gate) * up), not by how the engine computes:
+the plain implementation with the same roundings lies as far from the plain implementation
+without them (0.31 at logits of up to 6.6 when this was written).  The bound for bfloat16 is
+therefore that distance, measured in the same run, with a margin of a half."""
+import os
+import shutil
+import tempfile
+
+import numpy as np
+import pytest
+import torch
+
+import gpu_helpers as H
+import plain_model as pm
+
+pytestmark = [pytest.mark.gpu,
+              pytest.mark.skipif(os.environ.get("LLOGOS_FULL_SIZE") != "1",
+                                 reason="16 GB of weights and 80 GB of host memory: set LLOGOS_FULL_SIZE=1")]
+
+LLAMA31_8B = {
+    "architectures": ["LlamaForCausalLM"], "vocab_size": 128256, "hidden_size": 4096, "intermediate_size": 14336,
+    "num_hidden_layers": 32, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+    "rms_norm_eps": 1e-5, "rope_theta": 500000.0, "max_position_embeddings": 131072,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 8192},
+    "tie_word_embeddings": False, "torch_dtype": "bfloat16", "eos_token_id": 128001,
+}
+
+
+def _bf16(x):
+    return torch.from_numpy(np.ascontiguousarray(x)).to(torch.bfloat16).to(torch.float64).numpy()
+
+
+def _forward_with_roundings(cfg, w, tokens):
+    """pm.forward with the bfloat16 engine's roundings put in (causal, no window)."""
+    def attention(q, k, v, n_heads, n_kv_heads, head_dim, window=0, sinks=0, positions=None):
+        q, k, v = _bf16(q), _bf16(k), _bf16(v)
+        T, group = q.shape[0], n_heads // n_kv_heads
+        out = np.zeros((T, n_heads * head_dim))
+        seen = np.tril(np.ones((T, T), bool))
+        for h in range(n_heads):
+            g = h // group
+            qh, kh, vh = (m[:, i * head_dim:(i + 1) * head_dim] for m, i in ((q, h), (k, g), (v, g)))
+            s = np.where(seen, (qh @ kh.T) / np.sqrt(head_dim), -np.inf)
+            p = np.exp(s - s.max(1, keepdims=True))
+            out[:, h * head_dim:(h + 1) * head_dim] = (_bf16(p) @ vh) / p.sum(1, keepdims=True)
+        return _bf16(out)
+
+    def swiglu_mlp(x, wg, wu, wd):
+        g, u = _bf16(pm.linear(x, wg)), _bf16(pm.linear(x, wu))
+        return pm.linear(_bf16(pm.silu(g) * u), wd)
+
+    saved = pm.rms_norm, pm.attention, pm.swiglu_mlp
+    norm = pm.rms_norm
+    pm.rms_norm, pm.attention, pm.swiglu_mlp = (lambda x, w_, eps: _bf16(norm(x, w_, eps))), attention, swiglu_mlp
+    try:
+        return pm.forward(cfg, w, tokens)
+    finally:
+        pm.rms_norm, pm.attention, pm.swiglu_mlp = saved
+
+
+def test_the_whole_8b_configuration():
+    folder = tempfile.mkdtemp(prefix="llogos_full8b_")
+    try:
+        H.llogos.write_random_model(folder, LLAMA31_8B, seed=1)
+        cfg, w = pm.load_folder(folder)
+        rng = np.random.default_rng(5)
+        reqs = [rng.integers(0, LLAMA31_8B["vocab_size"], n).tolist() for n in (40, 9, 21)]
+        plain = [pm.forward(cfg, w, r) for r in reqs]
+        rounded = max(float(np.abs(_forward_with_roundings(cfg, w, r) - p).max()) for r, p in zip(reqs, plain))
+        del w
+        for dtype, bound in (("float32", 1e-4), ("bfloat16", 1.5 * rounded)):
+            eng = H.llogos.Engine.from_folder(folder, dtype=dtype, max_tokens=64 * 4, n_slots=3)
+            for r, p in zip(reqs, plain):                                   # whole, each alone
+                s = eng.alloc_slot()
+                got = eng.step([(s, r)], want="all").cpu().double().numpy()
+                eng.free_slot(s)
+                assert np.abs(got - p).max() <= bound, (dtype, "whole", np.abs(got - p).max(), bound)
+            s, r, p = eng.alloc_slot(), reqs[0], plain[0]                   # the last 8 tokens one by one
+            rows = [eng.step([(s, r[:-8])], want="all").cpu().double().numpy()]
+            rows += [eng.step([(s, [t])]).cpu().double().numpy() for t in r[-8:]]
+            eng.free_slot(s)
+            assert np.abs(np.concatenate(rows) - p).max() <= bound, (dtype, "token by token")
+            slots, cut = [eng.alloc_slot() for _ in reqs], (30, 5, 15)      # an unequal batch, one ends early
+            got = eng.step([(sl, r[:c]) for sl, r, c in zip(slots, reqs, cut)], want="all").cpu().double().numpy()
+            assert np.abs(got - np.concatenate([p[:c] for p, c in zip(plain, cut)])).max() <= bound, (dtype, "batch")
+            live = [0, 1, 2]
+            for t in range(4):
+                if t == 2:
+                    eng.free_slot(slots[1])
+                    live = [0, 2]
+                got = eng.step([(slots[i], [reqs[i][cut[i] + t]]) for i in live], want="last").cpu().double().numpy()
+                want = np.stack([plain[i][cut[i] + t] for i in live])
+                assert np.abs(got - want).max() <= bound, (dtype, "batch, token", t)
+            del eng
+            torch.cuda.empty_cache()
+    finally:
+        shutil.rmtree(folder, ignore_errors=True)
