@@ -1,8 +1,9 @@
-"""The whole Llama-3.1-8B configuration (32 layers, vocabulary 128256) with random weights
-against the plain implementation: requests whole, the last tokens one by one, and an unequal
-batch, in float32 (1e-4 absolute) and in bfloat16.  It writes a 16 GB model folder and holds
-the weights in float64 on the host (about 80 GB), so it runs only when LLOGOS_FULL_SIZE=1 is
-set; a minute on the GPU box.
+"""The whole Llama-3.1-8B configuration (32 layers, vocabulary 128256) and the whole Qwen3-14B
+configuration (40 layers, per-head norms, vocabulary 151936) with random weights against the
+plain implementation: requests whole, the last tokens one by one, and an unequal
+batch, in float32 (1e-4 absolute) and in bfloat16.  It writes model folders of 16 and 30 GB and
+holds the weights in float64 on the host (80 and 150 GB), so it runs only when
+LLOGOS_FULL_SIZE=1 is set; three minutes on the GPU box.
 
 At this depth the bfloat16 engine's distance from float64 arithmetic is set by where values
 are rounded to bfloat16 (normed rows, rotated queries and keys, values, probabilities, the
@@ -32,6 +33,14 @@ LLAMA31_8B = {
     "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
                      "original_max_position_embeddings": 8192},
     "tie_word_embeddings": False, "torch_dtype": "bfloat16", "eos_token_id": 128001,
+}
+
+
+QWEN3_14B = {
+    "architectures": ["Qwen3ForCausalLM"], "vocab_size": 151936, "hidden_size": 5120, "intermediate_size": 17408,
+    "num_hidden_layers": 40, "num_attention_heads": 40, "num_key_value_heads": 8, "head_dim": 128,
+    "rms_norm_eps": 1e-6, "rope_theta": 1000000.0, "max_position_embeddings": 40960,
+    "tie_word_embeddings": False, "torch_dtype": "bfloat16", "eos_token_id": 151645,
 }
 
 
@@ -67,13 +76,14 @@ def _forward_with_roundings(cfg, w, tokens):
         pm.rms_norm, pm.attention, pm.swiglu_mlp = saved
 
 
-def test_the_whole_8b_configuration():
-    folder = tempfile.mkdtemp(prefix="llogos_full8b_")
+@pytest.mark.parametrize("config", [LLAMA31_8B, QWEN3_14B], ids=["llama-3.1-8b", "qwen3-14b"])
+def test_a_whole_configuration(config):
+    folder = tempfile.mkdtemp(prefix="llogos_full_size_")
     try:
-        H.llogos.write_random_model(folder, LLAMA31_8B, seed=1)
+        H.llogos.write_random_model(folder, config, seed=1)
         cfg, w = pm.load_folder(folder)
         rng = np.random.default_rng(5)
-        reqs = [rng.integers(0, LLAMA31_8B["vocab_size"], n).tolist() for n in (40, 9, 21)]
+        reqs = [rng.integers(0, config["vocab_size"], n).tolist() for n in (40, 9, 21)]
         plain = [pm.forward(cfg, w, r) for r in reqs]
         rounded = max(float(np.abs(_forward_with_roundings(cfg, w, r) - p).max()) for r, p in zip(reqs, plain))
         del w
@@ -83,6 +93,7 @@ def test_the_whole_8b_configuration():
                 s = eng.alloc_slot()
                 got = eng.step([(s, r)], want="all").cpu().double().numpy()
                 eng.free_slot(s)
+                print(dtype, "whole:", float(np.abs(got - p).max()), "bound", bound, flush=True)
                 assert np.abs(got - p).max() <= bound, (dtype, "whole", np.abs(got - p).max(), bound)
             s, r, p = eng.alloc_slot(), reqs[0], plain[0]                   # the last 8 tokens one by one
             rows = [eng.step([(s, r[:-8])], want="all").cpu().double().numpy()]
