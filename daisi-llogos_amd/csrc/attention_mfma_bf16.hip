@@ -480,11 +480,12 @@ __global__ __launch_bounds__(kAttnWaves * kWave) void attn_prefill_kernel(
 // values are copied to LDS once per block (two buffers, the copy of the next page is in
 // flight while the current one is used), and every key fragment a wave reads serves both of
 // its column blocks.  Keys are visited in natural order here (operand row i of block rb is key
-// 16 rb + i, conflict-free in LDS with rows padded by 16 bytes), so lane group g owns keys
+// 16 rb + i, conflict-free in LDS with key rows padded by 32 bytes and the 8-byte reads of the
+// value rows padded by 16), so lane group g owns keys
 // 16 rb + 4 g .. + 3 of each block, and the value operand of a step of 32 keys is two runs of
 // four tokens.
 constexpr int kTileRows = 128;
-constexpr int kKPad = 8, kVPad = 8;
+constexpr int kKPad = 16, kVPad = 8;
 
 template <int HD>
 struct PageLds {
@@ -492,7 +493,7 @@ struct PageLds {
     bf16_t v[HD][kPageTokens + kVPad];
 };
 
-// two page buffers: 2 * 35.8 KB for head size 128, so that two blocks share a compute unit and
+// two page buffers: 2 * 36.9 KB for head size 128, so that two blocks share a compute unit and
 // one block's LDS and MFMA latencies are covered by the other
 template <int HD>
 struct TileLds {

@@ -8,7 +8,9 @@
 //  * the block copies the activations of that range, 256 values of k at a time, with full
 //    16-byte-per-lane loads into LDS (two buffers; the copy of the next chunk is in flight
 //    while the current one is multiplied), and the waves read their second MFMA operand
-//    from LDS (rows are padded by 16 bytes so that 16 lanes hit 64 different banks);
+//    from LDS (rows are padded by 32 bytes: with a row stride of 32 bytes modulo 64 a wave's
+//    16-byte reads of 16 rows take 4 clocks, free of bank conflicts by the hardware's counters;
+//    a stride of 16 modulo 32 takes 8);
 //  * each wave loads its weights straight from global memory into the MFMA operand layout,
 //    a whole chunk ahead;
 //  * an activation "producer" can be fused into the copy: SwiGLU of the (partial) gate/up
@@ -26,7 +28,7 @@ constexpr int kLdsWaves = 4;                 // waves per block (8 measured no f
 constexpr int kChunkK = 256;                 // values of k per LDS chunk (128 and 512 measured no faster)
 constexpr int kChunkSteps = kChunkK / 32;    // MFMA steps per chunk
 constexpr int kLdsMaxRows = 128;            // rows of activations (64 with a fused producer)
-constexpr int kRowPad = 8;                   // bf16 of padding per LDS row (16 bytes)
+constexpr int kRowPad = 16;                  // bf16 of padding per LDS row (32 bytes)
 
 enum { PRODUCE_PLAIN = 0, PRODUCE_SWIGLU_F32 = 1, PRODUCE_SWIGLU_BF16 = 2 };
 
