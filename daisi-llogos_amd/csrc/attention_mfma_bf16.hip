@@ -107,7 +107,9 @@ __device__ __forceinline__ void softmax_page(f32x4 (&s)[4], WaveState<HD>& st, f
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             if (MASKED) {
-                const int key = key0 + g * GS + rb * RS + r;
+                // GS < 0: eight consecutive keys per lane group and half page (the layout of the
+                // kernel whose pages go straight to LDS)
+                const int key = GS < 0 ? key0 + 32 * (rb >> 1) + 8 * g + 4 * (rb & 1) + r : key0 + g * GS + rb * RS + r;
                 if (!(q_pos >= 0 && key_visible(q_pos, key, window, sinks))) s[rb][r] = -INFINITY;
             }
             tile_max = fmaxf(tile_max, s[rb][r]);
@@ -717,6 +719,235 @@ void attn_prefill_lds_kernel(
     write_out(st1, 16 + c);
 }
 
+// ---------------------------------------------------------------- prefill, pages straight to LDS
+// The same tiles and the same order of blocks, for head size 128.  A page's keys and transposed
+// values go from global memory into LDS without passing through registers (16 bytes a lane, a
+// wave's 64 lanes to 1 KB of consecutive LDS), which frees the 32 registers of the copy and the
+// time of the stores.  Such a copy cannot pad rows, so the 16-byte pieces of a row are swizzled
+// instead: piece p of row r lies at p ^ f(r).  LDS serves a wave's 16-byte reads in four groups
+// of lanes {c, c + 16 : c = 8 h .. 8 h + 7} (+32), and a group is free of bank conflicts when its
+// 16 pieces cover the 64 banks once; with f(r) = 2 j(r), where j counts the rows that such a group
+// reads one after the other, that holds for the keys (256-byte rows) and for the values
+// (128-byte rows, two to a bank line: j over rows of equal parity).
+// Operand row i = 4 g' + r of key block rb is key 32 (rb >> 1) + 8 g' + 4 (rb & 1) + r, so the
+// lane of group g holds, after both blocks of a half page, the scores of the 8 consecutive keys
+// 32 t + 8 g .. + 7, and its value operand for that half page is one 16-byte read.
+template <int HD>
+struct DirectPageLds {
+    bf16_t k[kPageTokens][HD];
+    bf16_t v[HD][kPageTokens];
+};
+
+__device__ __forceinline__ int direct_key_row(int rb, int i) {
+    return 32 * (rb >> 1) + 8 * (i >> 2) + 4 * (rb & 1) + (i & 3);
+}
+__device__ __forceinline__ int direct_k_swizzle(int row) {                // rows read together: i = 0..7 of one block
+    return 2 * ((row & 3) | (((row >> 3) & 1) << 2));
+}
+__device__ __forceinline__ int direct_v_swizzle(int row) {                // rows of equal parity among 8 consecutive
+    return 2 * ((row >> 1) & 3);
+}
+
+__global__ __launch_bounds__(kAttnWaves * kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void attn_prefill_direct_kernel(
+        bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int q_stride,
+        const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
+        const int* __restrict__ table, int table_stride, const int* __restrict__ cu,
+        const int* __restrict__ tok_pos, int batch, int n_tiles, int n_heads, int n_kv_heads, int group,
+        float scale, int window, int sinks) {
+    constexpr int HD = 128;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    DirectPageLds<HD>* lds = reinterpret_cast<DirectPageLds<HD>*>(smem_raw);   // two buffers
+    int m_xcd = blockIdx.x / 8;
+    const int xcd = blockIdx.x % 8, per_xcd = gridDim.x / 8;
+    if (per_xcd > 32 && per_xcd <= 64 && m_xcd >= 32) m_xcd = per_xcd - 1 - (m_xcd - 32);   // see attn_prefill_lds_kernel
+    const int pair = (m_xcd / group) * 8 + xcd;
+    if (pair >= n_tiles * n_kv_heads) return;
+    const int kvh = pair % n_kv_heads, h = kvh * group + m_xcd % group;
+    int tile = n_tiles - 1 - pair / n_kv_heads, b = 0, first = 0;
+    for (; b < batch; ++b) {
+        const int len = cu[b + 1] - cu[b];
+        const int tiles = (len + kTileRows - 1) / kTileRows;
+        if (tile < tiles) { first = cu[b] + tile * kTileRows; break; }
+        tile -= tiles;
+    }
+    if (b >= batch) return;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int c = lane & 15, g = lane >> 4;
+    const int seq_end = cu[b + 1];
+    const int tile_rows = min(kTileRows, seq_end - first);
+    const int tile_last_pos = tok_pos[first + tile_rows - 1];
+    const int tile_first_pos = tok_pos[first];
+    const int written = tok_pos[seq_end - 1] + 1;
+    const int row0 = first + 32 * wave;
+    const int wave_rows = max(0, min(32, seq_end - row0));
+    const bool ok0 = c < wave_rows, ok1 = 16 + c < wave_rows;
+    const int q_pos0 = ok0 ? tok_pos[row0 + c] : -1, q_pos1 = ok1 ? tok_pos[row0 + 16 + c] : -1;
+    bf16x8 qf0[HD / 32], qf1[HD / 32];
+    {
+        const bf16_t* qrow0 = q + (size_t)(row0 + (ok0 ? c : 0)) * q_stride + (size_t)h * HD + 8 * g;
+        const bf16_t* qrow1 = q + (size_t)(row0 + (ok1 ? 16 + c : 0)) * q_stride + (size_t)h * HD + 8 * g;
+#pragma unroll
+        for (int sk = 0; sk < HD / 32; ++sk) {
+            qf0[sk] = ok0 ? ld_frag(qrow0 + 32 * sk) : zero_frag();
+            qf1[sk] = ok1 ? ld_frag(qrow1 + 32 * sk) : zero_frag();
+        }
+    }
+    WaveState<HD> st0, st1;
+    st0.init();
+    st1.init();
+    const int wave_first_pos = wave_rows > 0 ? tok_pos[row0] : 0;
+    const int wave_last_pos = wave_rows > 0 ? tok_pos[row0 + wave_rows - 1] : -1;
+    const float scale_log2 = scale * kLog2e;
+
+    const int n_pages = tile_last_pos / kPageTokens + 1;
+    auto page_needed = [&](int pi) {
+        return page_may_be_visible_to_range(tile_first_pos, tile_last_pos, pi * kPageTokens, window, sinks);
+    };
+    auto next_needed = [&](int pi) {
+        ++pi;
+        while (pi < n_pages && !page_needed(pi)) ++pi;
+        return pi;
+    };
+    auto page_id = [&](int pi) { return table[(size_t)b * table_stride + pi]; };
+    auto page_base = [&](int id) { return ((size_t)id * n_kv_heads + kvh) * kPageTokens * HD; };
+    // This wave's share of a page's copy: 4 + 4 instructions of 1 KB.  Instruction j of the keys
+    // covers rows 16 j + 4 wave .. + 3 (lane: row + lane / 16, piece lane % 16), of the values
+    // rows 32 j + 8 wave .. + 7 (lane: row + lane / 8, piece lane % 8).
+    auto copy_page = [&](int id, DirectPageLds<HD>& pg) {
+        const bf16_t* kpage = k_pool + page_base(id);
+        const bf16_t* vpage = v_pool + page_base(id);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int krow0 = 16 * j + 4 * wave, krow = krow0 + (lane >> 4);
+            const bf16_t* ksrc = kpage + (size_t)krow * HD + 8 * ((lane & 15) ^ direct_k_swizzle(krow));
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ksrc,
+                                             (__attribute__((address_space(3))) void*)&pg.k[krow0][0], 16, 0, 0);
+            const int vrow0 = 32 * j + 8 * wave, vrow = vrow0 + (lane >> 3);
+            const bf16_t* vsrc = vpage + (size_t)vrow * kPageTokens + 8 * ((lane & 7) ^ direct_v_swizzle(vrow));
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vsrc,
+                                             (__attribute__((address_space(3))) void*)&pg.v[vrow0][0], 16, 0, 0);
+        }
+    };
+    // The values of tokens that have not been written may be anything, also NaN, and 0 * NaN is
+    // NaN: in the one page of a sequence that is not full they are zeroed in LDS after the copy.
+    auto zero_unwritten = [&](DirectPageLds<HD>& pg, int valid_keys) {
+        const int row = threadIdx.x >> 1, half = threadIdx.x & 1;          // 128 rows, 4 pieces each
+#pragma unroll
+        for (int pp = 0; pp < 4; ++pp) {
+            const int piece = 4 * half + pp, keep = valid_keys - 8 * piece;
+            if (keep >= 8) continue;
+            uint4* at = reinterpret_cast<uint4*>(&pg.v[row][8 * (piece ^ direct_v_swizzle(row))]);
+            *at = __builtin_bit_cast(uint4, keep_first(__builtin_bit_cast(bf16x8, *at), keep));
+        }
+    };
+    auto land = [&](int pi, DirectPageLds<HD>& pg) {                        // the copy of page pi is complete and visible
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        const int valid_keys = written - pi * kPageTokens;
+        if (pi < n_pages && valid_keys < kPageTokens) {
+            zero_unwritten(pg, valid_keys);
+            __syncthreads();
+        }
+    };
+    int cur = next_needed(-1);
+    if (cur >= n_pages) return;                                          // cannot happen: a row sees itself
+    int nxt = next_needed(cur);
+    int nxt_id = nxt < n_pages ? page_id(nxt) : 0;
+    copy_page(page_id(cur), lds[0]);
+    land(cur, lds[0]);
+    int buf = 0;
+    while (cur < n_pages) {
+        const int nxt2 = next_needed(nxt);
+        if (nxt < n_pages) copy_page(nxt_id, lds[buf ^ 1]);
+        const int nxt2_id = nxt2 < n_pages ? page_id(nxt2) : 0;
+        do {
+        const int key0 = cur * kPageTokens;
+        if (wave_rows <= 0 || key0 > wave_last_pos) break;                // nothing of this page for this wave
+        if (!page_may_be_visible_to_range(wave_first_pos, wave_last_pos, key0, window, sinks)) break;
+        const DirectPageLds<HD>& pg = lds[buf];
+        f32x4 s0[4], s1[4];
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb) {
+            s0[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+            s1[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int sk = 0; sk < HD / 32; ++sk) {
+#pragma unroll
+            for (int rb = 0; rb < 4; ++rb) {
+                const int row = direct_key_row(rb, c);
+                const bf16x8 kf = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(
+                    &pg.k[row][8 * ((4 * sk + g) ^ direct_k_swizzle(row))]));
+                s0[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf0[sk], s0[rb], 0, 0, 0);
+                s1[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf1[sk], s1[rb], 0, 0, 0);
+            }
+        }
+        auto read_v = [&](int db, int t) {
+            const int row = 16 * db + c;
+            return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(
+                &pg.v[row][8 * ((4 * t + g) ^ direct_v_swizzle(row))]));
+        };
+        constexpr int kEarly = 2;
+        bf16x8 vf[HD / 16][2];
+#pragma unroll
+        for (int db = 0; db < kEarly; ++db) { vf[db][0] = read_v(db, 0); vf[db][1] = read_v(db, 1); }
+        bf16x8 pf0[2], pf1[2];
+        float corr0, corr1;
+        const bool all_visible = wave_rows == 32 &&
+                                 page_fully_visible(wave_first_pos, wave_last_pos, key0, window, sinks);
+        if (all_visible) {
+            softmax_page<false, -1, 0, HD>(s0, st0, scale_log2, q_pos0, key0, window, sinks, pf0, corr0);
+            softmax_page<false, -1, 0, HD>(s1, st1, scale_log2, q_pos1, key0, window, sinks, pf1, corr1);
+        } else {
+            softmax_page<true, -1, 0, HD>(s0, st0, scale_log2, q_pos0, key0, window, sinks, pf0, corr0);
+            softmax_page<true, -1, 0, HD>(s1, st1, scale_log2, q_pos1, key0, window, sinks, pf1, corr1);
+        }
+        const bool rescale = __ballot(corr0 != 1.0f || corr1 != 1.0f) != 0;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int db = 0; db < HD / 16; ++db) {
+            if (db + kEarly < HD / 16) {
+                vf[db + kEarly][0] = read_v(db + kEarly, 0);
+                vf[db + kEarly][1] = read_v(db + kEarly, 1);
+            }
+            f32x4 a0 = st0.acc[db], a1 = st1.acc[db];
+            if (rescale) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) { a0[r] *= corr0; a1[r] *= corr1; }
+            }
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[db][t], pf0[t], a0, 0, 0, 0);
+                a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[db][t], pf1[t], a1, 0, 0, 0);
+            }
+            st0.acc[db] = a0;
+            st1.acc[db] = a1;
+        }
+        } while (0);
+        land(nxt, lds[buf ^ 1]);
+        cur = nxt;
+        nxt = nxt2;
+        nxt_id = nxt2_id;
+        buf ^= 1;
+    }
+    auto write_out = [&](const WaveState<HD>& st, int rr) {
+        if (rr >= wave_rows) return;
+        const float inv = st.l > 0.f ? 1.0f / st.l : 0.f;
+        bf16_t* orow = out + ((size_t)(row0 + rr) * n_heads + h) * HD;
+#pragma unroll
+        for (int db = 0; db < HD / 16; ++db) {
+            uint2 u;
+            u.x = pack_bf16(st.acc[db][0] * inv, st.acc[db][1] * inv);
+            u.y = pack_bf16(st.acc[db][2] * inv, st.acc[db][3] * inv);
+            *reinterpret_cast<uint2*>(orow + 16 * db + 4 * g) = u;
+        }
+    };
+    write_out(st0, c);
+    write_out(st1, 16 + c);
+}
+
 // ---------------------------------------------------------------- entry points
 static bool mfma_shape_ok(int n_heads, int n_kv_heads, int head_dim) {
     if (n_kv_heads <= 0 || n_heads % n_kv_heads) return false;
@@ -806,12 +1037,13 @@ LLOGOS_EXPORT int llogos_attn_decode_fused_bf16(void* out, const float* qkv, int
                          n_heads, n_kv_heads, head_dim, scale, window, sinks, workspace, workspace_floats, stream);
 }
 
-// tile_rows: 64 for the kernel whose waves read pages from global memory, 128 for the kernel
-// that shares pages through LDS (n_tiles counts tiles of that many tokens per sequence).
+// tile_rows: 64 for the kernel whose waves read pages from global memory, 128 for the kernels
+// that share pages through LDS (n_tiles counts tiles of that many tokens per sequence); direct:
+// with 128-row tiles and head size 128, the kernel whose pages go straight to LDS.
 LLOGOS_EXPORT int llogos_attn_prefill_bf16(void* out, const void* q, int q_stride, const void* k_pool,
                                            const void* v_pool, const int* table, int table_stride,
                                            const int* cu, const int* tok_pos, int batch, int n_tiles, int tile_rows,
-                                           int n_heads, int n_kv_heads, int head_dim,
+                                           int direct, int n_heads, int n_kv_heads, int head_dim,
                                            float scale, int window, int sinks, hipStream_t stream) {
     if (batch <= 0 || n_tiles <= 0 || window < 0 || sinks < 0) return LLOGOS_BAD_ARGUMENT;
     if (tile_rows != 64 && tile_rows != kTileRows) return LLOGOS_BAD_ARGUMENT;
@@ -829,6 +1061,16 @@ LLOGOS_EXPORT int llogos_attn_prefill_bf16(void* out, const void* q, int q_strid
         attn_prefill_lds_kernel<HD><<<lgrid, kAttnWaves * kWave, smem, stream>>>( \
             (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride, \
             cu, tok_pos, batch, n_tiles, n_heads, n_kv_heads, group, scale, window, sinks); } while (0)
+        if (direct && head_dim == 128) {
+            const size_t smem = 2 * sizeof(DirectPageLds<128>);
+            hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_direct_kernel,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+            if (e != hipSuccess) return (int)e;
+            attn_prefill_direct_kernel<<<lgrid, kAttnWaves * kWave, smem, stream>>>(
+                (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride,
+                cu, tok_pos, batch, n_tiles, n_heads, n_kv_heads, group, scale, window, sinks);
+            return LLOGOS_LAUNCH_CHECK();
+        }
         if (head_dim == 64) GOL(64); else GOL(128);
 #undef GOL
         return LLOGOS_LAUNCH_CHECK();
