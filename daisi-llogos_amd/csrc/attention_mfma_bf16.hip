@@ -475,260 +475,23 @@ __global__ __launch_bounds__(kAttnWaves * kWave) void attn_prefill_kernel(
     }
 }
 
+constexpr int kTileRows = 128;
+
 // ---------------------------------------------------------------- prefill, pages shared through LDS
 // grid: one block per (tile of 128 tokens over all sequences, head), in the order given in the
-// kernel; the 4 waves of a block take 32 rows
-// each (two blocks of 16 columns) and walk the same pages: a page's keys and transposed
-// values are copied to LDS once per block (two buffers, the copy of the next page is in
-// flight while the current one is used), and every key fragment a wave reads serves both of
-// its column blocks.  Keys are visited in natural order here (operand row i of block rb is key
-// 16 rb + i, conflict-free in LDS with key rows padded by 32 bytes and the 8-byte reads of the
-// value rows padded by 16), so lane group g owns keys
-// 16 rb + 4 g .. + 3 of each block, and the value operand of a step of 32 keys is two runs of
-// four tokens.
-constexpr int kTileRows = 128;
-constexpr int kKPad = 16, kVPad = 8;
-
-template <int HD>
-struct PageLds {
-    bf16_t k[kPageTokens][HD + kKPad];
-    bf16_t v[HD][kPageTokens + kVPad];
-};
-
-// two page buffers: 2 * 36.9 KB for head size 128, so that two blocks share a compute unit and
-// one block's LDS and MFMA latencies are covered by the other
-template <int HD>
-struct TileLds {
-    PageLds<HD> page[2];
-};
-
-template <int HD, int N>
-__device__ __forceinline__ void fetch_page(uint4 (&kreg)[N], uint4 (&vreg)[N], const bf16_t* __restrict__ kpage,
-                                           const bf16_t* __restrict__ vpage) {
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-        const int piece = i * (kAttnWaves * kWave) + threadIdx.x;
-        kreg[i] = *reinterpret_cast<const uint4*>(kpage + (size_t)piece * 8);
-        vreg[i] = *reinterpret_cast<const uint4*>(vpage + (size_t)piece * 8);
-    }
-}
-
-// valid_keys: how many of the page's tokens have been written; the values of the others go to
-// LDS as zeros (their probabilities are zero, and 0 * NaN would be NaN).
-template <int HD, int N>
-__device__ __forceinline__ void stash_page(PageLds<HD>& pg, const uint4 (&kreg)[N], const uint4 (&vreg)[N],
-                                           int valid_keys) {
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-        const int piece = i * (kAttnWaves * kWave) + threadIdx.x;
-        *reinterpret_cast<uint4*>(&pg.k[piece / (HD / 8)][(piece % (HD / 8)) * 8]) = kreg[i];
-        const int tok0 = (piece % (kPageTokens / 8)) * 8;
-        uint4 v = vreg[i];
-        if (valid_keys < kPageTokens)
-            v = __builtin_bit_cast(uint4, keep_first(__builtin_bit_cast(bf16x8, v), valid_keys - tok0));
-        *reinterpret_cast<uint4*>(&pg.v[piece / (kPageTokens / 8)][tok0]) = v;
-    }
-}
-
-template <int HD>
-__global__ __launch_bounds__(kAttnWaves * kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void attn_prefill_lds_kernel(
-        bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int q_stride,
-        const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
-        const int* __restrict__ table, int table_stride, const int* __restrict__ cu,
-        const int* __restrict__ tok_pos, int batch, int n_tiles, int n_heads, int n_kv_heads, int group,
-        float scale, int window, int sinks) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    TileLds<HD>& tl = *reinterpret_cast<TileLds<HD>*>(smem_raw);
-    PageLds<HD>* lds = tl.page;                                       // two buffers
-    // Blocks start in the order of their index, round-robin over the 8 XCDs.  Block L is the
-    // m-th block of XCD x (L = 8 m + x); an XCD takes the `group` query heads of one (tile, kv
-    // head) pair one after the other, so that the pair's pages stay in its L2, and the pairs go
-    // from the last tile to the first: late tiles of a causal prompt see the most keys, and
-    // starting with them keeps the compute units evenly busy to the end.
-    // A grid of at most two blocks per compute unit starts all at once, and the m-th and the
-    // (m + 32)-th block of an XCD share a compute unit: the second half runs in rising order
-    // then, so that the longest block shares with the shortest.
-    int m_xcd = blockIdx.x / 8;
-    const int xcd = blockIdx.x % 8, per_xcd = gridDim.x / 8;
-    if (per_xcd > 32 && per_xcd <= 64 && m_xcd >= 32) m_xcd = per_xcd - 1 - (m_xcd - 32);
-    const int pair = (m_xcd / group) * 8 + xcd;
-    if (pair >= n_tiles * n_kv_heads) return;
-    const int kvh = pair % n_kv_heads, h = kvh * group + m_xcd % group;
-    int tile = n_tiles - 1 - pair / n_kv_heads, b = 0, first = 0;
-    for (; b < batch; ++b) {
-        const int len = cu[b + 1] - cu[b];
-        const int tiles = (len + kTileRows - 1) / kTileRows;
-        if (tile < tiles) { first = cu[b] + tile * kTileRows; break; }
-        tile -= tiles;
-    }
-    if (b >= batch) return;
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-    const int c = lane & 15, g = lane >> 4;
-    const int seq_end = cu[b + 1];
-    const int tile_rows = min(kTileRows, seq_end - first);
-    const int tile_last_pos = tok_pos[first + tile_rows - 1];
-    const int tile_first_pos = tok_pos[first];
-    const int written = tok_pos[seq_end - 1] + 1;
-    // this wave: rows first + 32 wave .. + 31, column block cb holds rows + 16 cb
-    const int row0 = first + 32 * wave;
-    const int wave_rows = max(0, min(32, seq_end - row0));
-    const bool ok0 = c < wave_rows, ok1 = 16 + c < wave_rows;
-    const int q_pos0 = ok0 ? tok_pos[row0 + c] : -1, q_pos1 = ok1 ? tok_pos[row0 + 16 + c] : -1;
-    // the wave's 32 query rows as second operands (rows past the sequence as zeros)
-    bf16x8 qf0[HD / 32], qf1[HD / 32];
-    {
-        const bf16_t* qrow0 = q + (size_t)(row0 + (ok0 ? c : 0)) * q_stride + (size_t)h * HD + 8 * g;
-        const bf16_t* qrow1 = q + (size_t)(row0 + (ok1 ? 16 + c : 0)) * q_stride + (size_t)h * HD + 8 * g;
-#pragma unroll
-        for (int sk = 0; sk < HD / 32; ++sk) {
-            qf0[sk] = ok0 ? ld_frag(qrow0 + 32 * sk) : zero_frag();
-            qf1[sk] = ok1 ? ld_frag(qrow1 + 32 * sk) : zero_frag();
-        }
-    }
-    WaveState<HD> st0, st1;
-    st0.init();
-    st1.init();
-    const int wave_first_pos = wave_rows > 0 ? tok_pos[row0] : 0;
-    const int wave_last_pos = wave_rows > 0 ? tok_pos[row0 + wave_rows - 1] : -1;
-    const float scale_log2 = scale * kLog2e;
-
-    // the pages the tile needs, in order
-    const int n_pages = tile_last_pos / kPageTokens + 1;
-    auto page_needed = [&](int pi) {
-        return page_may_be_visible_to_range(tile_first_pos, tile_last_pos, pi * kPageTokens, window, sinks);
-    };
-    constexpr int kPerThread = kPageTokens * HD / 8 / (kAttnWaves * kWave);   // 16-byte pieces of a page per thread
-    uint4 kreg[kPerThread], vreg[kPerThread];
-    // walk the needed pages with one page of look-ahead; the page id of the page after next is
-    // read one iteration early, so that no iteration waits for the table and then for the page
-    auto next_needed = [&](int pi) {
-        ++pi;
-        while (pi < n_pages && !page_needed(pi)) ++pi;
-        return pi;
-    };
-    auto page_id = [&](int pi) { return table[(size_t)b * table_stride + pi]; };
-    auto page_base = [&](int id) { return ((size_t)id * n_kv_heads + kvh) * kPageTokens * HD; };
-    int cur = next_needed(-1);
-    if (cur >= n_pages) return;                                          // cannot happen: a row sees itself
-    int nxt = next_needed(cur);
-    int cur_id = page_id(cur);
-    int nxt_id = nxt < n_pages ? page_id(nxt) : cur_id;
-    {
-        const size_t base = page_base(cur_id);
-        fetch_page<HD, kPerThread>(kreg, vreg, k_pool + base, v_pool + base);
-        stash_page<HD, kPerThread>(lds[0], kreg, vreg, min(kPageTokens, written - cur * kPageTokens));
-    }
-    __syncthreads();
-    int buf = 0;
-    while (cur < n_pages) {
-        const int nxt2 = next_needed(nxt);
-        {   // always fetched and stashed (past the end: the current page once more, never used)
-            const size_t base = page_base(nxt_id);
-            fetch_page<HD, kPerThread>(kreg, vreg, k_pool + base, v_pool + base);
-        }
-        const int nxt2_id = nxt2 < n_pages ? page_id(nxt2) : nxt_id;
-        const int pi = cur;
-        do {
-        const int key0 = pi * kPageTokens;
-        if (wave_rows <= 0 || key0 > wave_last_pos) break;                // nothing of this page for this wave
-        if (!page_may_be_visible_to_range(wave_first_pos, wave_last_pos, key0, window, sinks)) break;
-        const PageLds<HD>& pg = lds[buf];
-        // S^T for both column blocks; operand row c of block rb is key 16 rb + c
-        f32x4 s0[4], s1[4];
-#pragma unroll
-        for (int rb = 0; rb < 4; ++rb) {
-            s0[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
-            s1[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
-#pragma unroll
-        for (int sk = 0; sk < HD / 32; ++sk) {
-#pragma unroll
-            for (int rb = 0; rb < 4; ++rb) {
-                const bf16x8 kf = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&pg.k[16 * rb + c][32 * sk + 8 * g]));
-                s0[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf0[sk], s0[rb], 0, 0, 0);
-                s1[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf1[sk], s1[rb], 0, 0, 0);
-            }
-        }
-        // the value fragments are read now, so that their way from LDS is covered by the softmax.
-        // lane (c, g) of block cb: column c, keys key0 + 16 rb + 4 g + r; step t of the value
-        // product covers blocks 2 t and 2 t + 1: slots 0..3 keys 32 t + 4 g + e, slots 4..7 keys
-        // 32 t + 16 + 4 g + e
-        auto read_v = [&](int db, int t) {
-            const bf16_t* vrow = &pg.v[16 * db + c][32 * t + 4 * g];
-            const uint2 lo = *reinterpret_cast<const uint2*>(vrow), hi = *reinterpret_cast<const uint2*>(vrow + 16);
-            return __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
-        };
-        constexpr int kEarly = 2;                                         // the others two steps ahead of their use
-        bf16x8 vf[HD / 16][2];
-#pragma unroll
-        for (int db = 0; db < kEarly; ++db) { vf[db][0] = read_v(db, 0); vf[db][1] = read_v(db, 1); }
-        bf16x8 pf0[2], pf1[2];
-        float corr0, corr1;
-        const bool all_visible = wave_rows == 32 &&
-                                 page_fully_visible(wave_first_pos, wave_last_pos, key0, window, sinks);
-        if (all_visible) {
-            softmax_page<false, 4, 16, HD>(s0, st0, scale_log2, q_pos0, key0, window, sinks, pf0, corr0);
-            softmax_page<false, 4, 16, HD>(s1, st1, scale_log2, q_pos1, key0, window, sinks, pf1, corr1);
-        } else {
-            softmax_page<true, 4, 16, HD>(s0, st0, scale_log2, q_pos0, key0, window, sinks, pf0, corr0);
-            softmax_page<true, 4, 16, HD>(s1, st1, scale_log2, q_pos1, key0, window, sinks, pf1, corr1);
-        }
-        const bool rescale = __ballot(corr0 != 1.0f || corr1 != 1.0f) != 0;
-        __builtin_amdgcn_sched_barrier(0);                                // the late reads stay behind the softmax
-#pragma unroll
-        for (int db = 0; db < HD / 16; ++db) {
-            if (db + kEarly < HD / 16) {
-                vf[db + kEarly][0] = read_v(db + kEarly, 0);
-                vf[db + kEarly][1] = read_v(db + kEarly, 1);
-            }
-            f32x4 a0 = st0.acc[db], a1 = st1.acc[db];
-            if (rescale) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) { a0[r] *= corr0; a1[r] *= corr1; }
-            }
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[db][t], pf0[t], a0, 0, 0, 0);
-                a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[db][t], pf1[t], a1, 0, 0, 0);
-            }
-            st0.acc[db] = a0;
-            st1.acc[db] = a1;
-        }
-        } while (0);
-        stash_page<HD, kPerThread>(lds[buf ^ 1], kreg, vreg, min(kPageTokens, written - min(nxt, n_pages - 1) * kPageTokens));
-        __syncthreads();
-        cur = nxt;
-        nxt = nxt2;
-        nxt_id = nxt2_id;
-        buf ^= 1;
-    }
-    auto write_out = [&](const WaveState<HD>& st, int rr) {
-        if (rr >= wave_rows) return;
-        const float inv = st.l > 0.f ? 1.0f / st.l : 0.f;
-        bf16_t* orow = out + ((size_t)(row0 + rr) * n_heads + h) * HD;
-#pragma unroll
-        for (int db = 0; db < HD / 16; ++db) {
-            uint2 u;
-            u.x = pack_bf16(st.acc[db][0] * inv, st.acc[db][1] * inv);
-            u.y = pack_bf16(st.acc[db][2] * inv, st.acc[db][3] * inv);
-            *reinterpret_cast<uint2*>(orow + 16 * db + 4 * g) = u;
-        }
-    };
-    write_out(st0, c);
-    write_out(st1, 16 + c);
-}
-
-// ---------------------------------------------------------------- prefill, pages straight to LDS
-// The same tiles and the same order of blocks, for head size 128.  A page's keys and transposed
+// kernel; the 4 waves of a block take 32 rows each (two blocks of 16 columns) and walk the same
+// pages: a page is copied to LDS once per block (two buffers, the copy of the next page is in
+// flight while the current one is used), and every key and value fragment a wave reads serves
+// both of its column blocks.  A page's keys and transposed
 // values go from global memory into LDS without passing through registers (16 bytes a lane, a
 // wave's 64 lanes to 1 KB of consecutive LDS), which frees the 32 registers of the copy and the
 // time of the stores.  Such a copy cannot pad rows, so the 16-byte pieces of a row are swizzled
 // instead: piece p of row r lies at p ^ f(r).  LDS serves a wave's 16-byte reads in four groups
 // of lanes {c, c + 16 : c = 8 h .. 8 h + 7} (+32), and a group is free of bank conflicts when its
 // 16 pieces cover the 64 banks once; with f(r) = 2 j(r), where j counts the rows that such a group
-// reads one after the other, that holds for the keys (256-byte rows) and for the values
-// (128-byte rows, two to a bank line: j over rows of equal parity).
+// reads one after the other, that holds for rows of 256 bytes (the keys at head size 128); rows
+// of 128 bytes (the values, and the keys at head size 64) lie two to a bank line, and j counts
+// the rows of equal parity.
 // Operand row i = 4 g' + r of key block rb is key 32 (rb >> 1) + 8 g' + 4 (rb & 1) + r, so the
 // lane of group g holds, after both blocks of a half page, the scores of the 8 consecutive keys
 // 32 t + 8 g .. + 7, and its value operand for that half page is one 16-byte read.
@@ -741,13 +504,16 @@ struct DirectPageLds {
 __device__ __forceinline__ int direct_key_row(int rb, int i) {
     return 32 * (rb >> 1) + 8 * (i >> 2) + 4 * (rb & 1) + (i & 3);
 }
+template <int HD>
 __device__ __forceinline__ int direct_k_swizzle(int row) {                // rows read together: i = 0..7 of one block
-    return 2 * ((row & 3) | (((row >> 3) & 1) << 2));
+    return HD == 128 ? 2 * ((row & 3) | (((row >> 3) & 1) << 2))
+                     : 2 * (((row >> 1) & 1) | (((row >> 3) & 1) << 1));
 }
 __device__ __forceinline__ int direct_v_swizzle(int row) {                // rows of equal parity among 8 consecutive
     return 2 * ((row >> 1) & 3);
 }
 
+template <int HD>
 __global__ __launch_bounds__(kAttnWaves * kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attn_prefill_direct_kernel(
         bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int q_stride,
@@ -755,12 +521,19 @@ void attn_prefill_direct_kernel(
         const int* __restrict__ table, int table_stride, const int* __restrict__ cu,
         const int* __restrict__ tok_pos, int batch, int n_tiles, int n_heads, int n_kv_heads, int group,
         float scale, int window, int sinks) {
-    constexpr int HD = 128;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     DirectPageLds<HD>* lds = reinterpret_cast<DirectPageLds<HD>*>(smem_raw);   // two buffers
+    // Blocks start in the order of their index, round-robin over the 8 XCDs.  Block L is the
+    // m-th block of XCD x (L = 8 m + x); an XCD takes the `group` query heads of one (tile, kv
+    // head) pair one after the other, so that the pair's pages stay in its L2, and the pairs go
+    // from the last tile to the first: late tiles of a causal prompt see the most keys, and
+    // starting with them keeps the compute units evenly busy to the end.
+    // A grid of at most two blocks per compute unit starts all at once, and the m-th and the
+    // (m + 32)-th block of an XCD share a compute unit: the second half runs in rising order
+    // then, so that the longest block shares with the shortest.
     int m_xcd = blockIdx.x / 8;
     const int xcd = blockIdx.x % 8, per_xcd = gridDim.x / 8;
-    if (per_xcd > 32 && per_xcd <= 64 && m_xcd >= 32) m_xcd = per_xcd - 1 - (m_xcd - 32);   // see attn_prefill_lds_kernel
+    if (per_xcd > 32 && per_xcd <= 64 && m_xcd >= 32) m_xcd = per_xcd - 1 - (m_xcd - 32);
     const int pair = (m_xcd / group) * 8 + xcd;
     if (pair >= n_tiles * n_kv_heads) return;
     const int kvh = pair % n_kv_heads, h = kvh * group + m_xcd % group;
@@ -812,19 +585,22 @@ void attn_prefill_direct_kernel(
     };
     auto page_id = [&](int pi) { return table[(size_t)b * table_stride + pi]; };
     auto page_base = [&](int id) { return ((size_t)id * n_kv_heads + kvh) * kPageTokens * HD; };
-    // This wave's share of a page's copy: 4 + 4 instructions of 1 KB.  Instruction j of the keys
-    // covers rows 16 j + 4 wave .. + 3 (lane: row + lane / 16, piece lane % 16), of the values
-    // rows 32 j + 8 wave .. + 7 (lane: row + lane / 8, piece lane % 8).
+    // This wave's share of a page's copy, in instructions of 1 KB (64 lanes x 16 bytes): a row of
+    // keys has HD / 8 pieces, a row of values 8; the block's instructions go to its waves in turn.
     auto copy_page = [&](int id, DirectPageLds<HD>& pg) {
         const bf16_t* kpage = k_pool + page_base(id);
         const bf16_t* vpage = v_pool + page_base(id);
+        constexpr int kKeyPieces = HD / 8, kKeyRows = kWave / kKeyPieces;    // pieces a row, rows an instruction
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int krow0 = 16 * j + 4 * wave, krow = krow0 + (lane >> 4);
-            const bf16_t* ksrc = kpage + (size_t)krow * HD + 8 * ((lane & 15) ^ direct_k_swizzle(krow));
+        for (int j = 0; j < kPageTokens / kKeyRows / kAttnWaves; ++j) {
+            const int krow0 = kKeyRows * (kAttnWaves * j + wave), krow = krow0 + lane / kKeyPieces;
+            const bf16_t* ksrc = kpage + (size_t)krow * HD + 8 * ((lane % kKeyPieces) ^ direct_k_swizzle<HD>(krow));
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ksrc,
                                              (__attribute__((address_space(3))) void*)&pg.k[krow0][0], 16, 0, 0);
-            const int vrow0 = 32 * j + 8 * wave, vrow = vrow0 + (lane >> 3);
+        }
+#pragma unroll
+        for (int j = 0; j < HD / 8 / kAttnWaves; ++j) {
+            const int vrow0 = 8 * (kAttnWaves * j + wave), vrow = vrow0 + (lane >> 3);
             const bf16_t* vsrc = vpage + (size_t)vrow * kPageTokens + 8 * ((lane & 7) ^ direct_v_swizzle(vrow));
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vsrc,
                                              (__attribute__((address_space(3))) void*)&pg.v[vrow0][0], 16, 0, 0);
@@ -833,7 +609,8 @@ void attn_prefill_direct_kernel(
     // The values of tokens that have not been written may be anything, also NaN, and 0 * NaN is
     // NaN: in the one page of a sequence that is not full they are zeroed in LDS after the copy.
     auto zero_unwritten = [&](DirectPageLds<HD>& pg, int valid_keys) {
-        const int row = threadIdx.x >> 1, half = threadIdx.x & 1;          // 128 rows, 4 pieces each
+        const int row = threadIdx.x >> 1, half = threadIdx.x & 1;          // a row's 8 pieces to two threads
+        if (row >= HD) return;
 #pragma unroll
         for (int pp = 0; pp < 4; ++pp) {
             const int piece = 4 * half + pp, keep = valid_keys - 8 * piece;
@@ -879,7 +656,7 @@ void attn_prefill_direct_kernel(
             for (int rb = 0; rb < 4; ++rb) {
                 const int row = direct_key_row(rb, c);
                 const bf16x8 kf = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(
-                    &pg.k[row][8 * ((4 * sk + g) ^ direct_k_swizzle(row))]));
+                    &pg.k[row][8 * ((4 * sk + g) ^ direct_k_swizzle<HD>(row))]));
                 s0[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf0[sk], s0[rb], 0, 0, 0);
                 s1[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf1[sk], s1[rb], 0, 0, 0);
             }
@@ -1037,13 +814,12 @@ LLOGOS_EXPORT int llogos_attn_decode_fused_bf16(void* out, const float* qkv, int
                          n_heads, n_kv_heads, head_dim, scale, window, sinks, workspace, workspace_floats, stream);
 }
 
-// tile_rows: 64 for the kernel whose waves read pages from global memory, 128 for the kernels
-// that share pages through LDS (n_tiles counts tiles of that many tokens per sequence); direct:
-// with 128-row tiles and head size 128, the kernel whose pages go straight to LDS.
+// tile_rows: 64 for the kernel whose waves read pages from global memory, 128 for the kernel
+// that shares pages through LDS (n_tiles counts tiles of that many tokens per sequence).
 LLOGOS_EXPORT int llogos_attn_prefill_bf16(void* out, const void* q, int q_stride, const void* k_pool,
                                            const void* v_pool, const int* table, int table_stride,
                                            const int* cu, const int* tok_pos, int batch, int n_tiles, int tile_rows,
-                                           int direct, int n_heads, int n_kv_heads, int head_dim,
+                                           int n_heads, int n_kv_heads, int head_dim,
                                            float scale, int window, int sinks, hipStream_t stream) {
     if (batch <= 0 || n_tiles <= 0 || window < 0 || sinks < 0) return LLOGOS_BAD_ARGUMENT;
     if (tile_rows != 64 && tile_rows != kTileRows) return LLOGOS_BAD_ARGUMENT;
@@ -1053,27 +829,17 @@ LLOGOS_EXPORT int llogos_attn_prefill_bf16(void* out, const void* q, int q_strid
     if (tile_rows == kTileRows) {
         const long long pairs = (long long)n_tiles * n_kv_heads;
         const dim3 lgrid((unsigned)((pairs + 7) / 8 * 8 * group));
-#define GOL(HD) do { \
-        const size_t smem = sizeof(TileLds<HD>); \
-        hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<HD>, \
+#define GOD(HD) do { \
+        const size_t smem = 2 * sizeof(DirectPageLds<HD>); \
+        hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_direct_kernel<HD>, \
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
         if (e != hipSuccess) return (int)e; \
-        attn_prefill_lds_kernel<HD><<<lgrid, kAttnWaves * kWave, smem, stream>>>( \
+        attn_prefill_direct_kernel<HD><<<lgrid, kAttnWaves * kWave, smem, stream>>>( \
             (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride, \
-            cu, tok_pos, batch, n_tiles, n_heads, n_kv_heads, group, scale, window, sinks); } while (0)
-        if (direct && head_dim == 128) {
-            const size_t smem = 2 * sizeof(DirectPageLds<128>);
-            hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_direct_kernel,
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-            if (e != hipSuccess) return (int)e;
-            attn_prefill_direct_kernel<<<lgrid, kAttnWaves * kWave, smem, stream>>>(
-                (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride,
-                cu, tok_pos, batch, n_tiles, n_heads, n_kv_heads, group, scale, window, sinks);
-            return LLOGOS_LAUNCH_CHECK();
-        }
-        if (head_dim == 64) GOL(64); else GOL(128);
-#undef GOL
-        return LLOGOS_LAUNCH_CHECK();
+            cu, tok_pos, batch, n_tiles, n_heads, n_kv_heads, group, scale, window, sinks); \
+        return LLOGOS_LAUNCH_CHECK(); } while (0)
+        if (head_dim == 64) GOD(64); else GOD(128);
+#undef GOD
     }
 #define GO(HD) attn_prefill_kernel<HD><<<grid, kAttnWaves * kWave, 0, stream>>>( \
         (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride, \

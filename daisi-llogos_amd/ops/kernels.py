@@ -541,7 +541,6 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dty
 
 _attn_workspaces = {}
 PREFILL_TILE_ROWS = 0        # 0: chosen by the step; 64 or 128 force a prefill attention kernel (tests)
-PREFILL_DIRECT = 1           # 128-row tiles at head size 128: pages straight to LDS (1) or through registers (0)
 
 
 def _attn_workspace(device: torch.device, floats: int) -> torch.Tensor:
@@ -592,8 +591,8 @@ def attention_mfma_bf16(ctx, q: torch.Tensor, q_stride: int, k_pool: torch.Tenso
         n_tiles = sum(-(-n // tile_rows) for n in lens)
         code = lib.llogos_attn_prefill_bf16(
             _p(out), _p(q), q_stride, _p(k_pool), _p(v_pool), _p(table), table.stride(0), _p(cu), _p(ctx.tok_pos),
-            ctx.batch, n_tiles, tile_rows, PREFILL_DIRECT, n_heads, n_kv_heads, head_dim, ctypes.c_float(scale),
-            window, sinks, _stream())
+            ctx.batch, n_tiles, tile_rows, n_heads, n_kv_heads, head_dim, ctypes.c_float(scale), window, sinks,
+            _stream())
     if code == -2:
         return None
     _check(code, "attention_mfma_bf16")
