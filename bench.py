@@ -32,8 +32,12 @@ QWEN3_14B = {
     "attention_bias": False, "tie_word_embeddings": False, "torch_dtype": "bfloat16", "eos_token_id": 151645,
 }
 LLAMA31_70B = dict(LLAMA31_8B, hidden_size=8192, intermediate_size=28672, num_hidden_layers=80, num_attention_heads=64)
+# the size class of the reference's own published runs (Llama-3.2-1B: head size 64, tied head)
+LLAMA32_1B = dict(LLAMA31_8B, hidden_size=2048, intermediate_size=8192, num_hidden_layers=16, head_dim=64,
+                  tie_word_embeddings=True,
+                  rope_scaling=dict(LLAMA31_8B["rope_scaling"], factor=32.0))
 MODELS = {"llama-3.1-8b": ("Llama-3.1-8B", LLAMA31_8B), "qwen3-14b": ("Qwen3-14B", QWEN3_14B),
-          "llama-3.1-70b": ("Llama-3.1-70B", LLAMA31_70B)}
+          "llama-3.1-70b": ("Llama-3.1-70B", LLAMA31_70B), "llama-3.2-1b": ("Llama-3.2-1B", LLAMA32_1B)}
 CONTEXT, PROMPT, PREFILL_TOKENS = 4096, 512, 2048
 
 
@@ -157,7 +161,7 @@ def main(argv=None) -> int:
                    "layers_full": full_layers, "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
                    "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
                    "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
-                   "rope_theta": cfg["rope_theta"], "rope_scaling": "llama3 x8" if cfg.get("rope_scaling") else "none", "rms_eps": cfg["rms_norm_eps"],
+                   "rope_theta": cfg["rope_theta"], "rope_scaling": f"llama3 x{cfg['rope_scaling']['factor']:g}" if cfg.get("rope_scaling") else "none", "rms_eps": cfg["rms_norm_eps"],
                    "sampling": "greedy", "hip_graphs": eng.graphs is not None},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4)},
