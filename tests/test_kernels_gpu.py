@@ -201,10 +201,11 @@ def _pages(n_seqs, max_len, rng):
 @pytest.mark.parametrize("nh,nkv,hd,rot,pairing,norm", [
     (4, 2, 16, 16, 0, False), (6, 1, 32, 32, 0, True), (5, 5, 48, 24, 0, True), (8, 2, 80, 80, 1, False),
     (3, 3, 128, 64, 1, True), (2, 1, 256, 256, 0, False), (8, 2, 128, 128, 0, True), (5, 5, 128, 128, 0, False)])
-def test_qk_rope_cache(dtype, nh, nkv, hd, rot, pairing, norm):
+@pytest.mark.parametrize("lens,new", [([70, 3], [5, 3]), ([70, 30], [40, 27])])
+def test_qk_rope_cache(dtype, nh, nkv, hd, rot, pairing, norm, lens, new):
+    """Two sequences; this step brings the last `new` tokens of each: a few tokens, and runs
+    that cross a page's end and start in the middle of one."""
     rng = np.random.default_rng(3)
-    lens = [70, 3]                                      # two sequences; this step brings the last 5 and 3 tokens
-    new = [5, 3]
     T = sum(new)
     tok_seq = np.repeat(np.arange(2), new).astype(np.int32)
     tok_pos = np.concatenate([np.arange(l - n, l) for l, n in zip(lens, new)]).astype(np.int32)
