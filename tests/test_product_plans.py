@@ -1,0 +1,52 @@
+"""The plans of the few-row matrix products are host arithmetic: which kernel, how many blocks
+along k.  A plan may depend on the matrix and on the class of the row count (up to 16, 32, 64,
+128 rows) only, so that a row's sums come in the same order for every batch of its class; the
+consumers of partial sums take at most 8 parts."""
+import importlib
+
+import pytest
+
+K = importlib.import_module("daisi-llogos_amd.ops.kernels")
+
+SHAPES = [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336), (128256, 4096),      # Llama-3.1-8B
+          (7168, 5120), (5120, 5120), (34816, 5120), (5120, 17408), (151936, 5120),      # Qwen3-14B
+          (10240, 8192), (8192, 8192), (57344, 8192), (8192, 28672),                     # Llama-3.1-70B
+          (3072, 2048), (16384, 2048), (2048, 8192), (331, 80), (96, 1000), (17, 8)]
+
+
+@pytest.mark.parametrize("N,K_", SHAPES)
+def test_a_plan_depends_on_the_class_of_the_row_count_only(N, K_):
+    for lo, hi in ((1, 4), (5, 8), (9, 16), (17, 32), (33, 64)):
+        plans = {K.skinny_plan(M, N, K_) for M in range(lo, hi + 1)}
+        if hi <= 16:
+            # up to 16 rows the kernel may change with the row count (activations held in
+            # registers for the fewest rows), but not within 1..4, 5..8 and 9..16
+            assert len(plans) == 1, (N, K_, lo, hi, plans)
+        else:
+            assert len(plans) == 1 and next(iter(plans))[0] == "lds", (N, K_, lo, hi, plans)
+    assert len({K.lds_splits(M, N, K_) for M in range(65, 129)}) == 1
+
+
+@pytest.mark.parametrize("N,K_", SHAPES)
+def test_plans_are_within_what_the_kernels_and_their_consumers_take(N, K_):
+    for M in (1, 4, 8, 16, 32, 64, 128):
+        parts = K.lds_splits(M, N, K_)
+        assert 1 <= parts <= 8
+        assert parts == 1 or -(-K_ // 256) >= 2 * parts - 1        # every block along k has work
+        if M <= 64:
+            kernel, splits, third = K.skinny_plan(M, N, K_)
+            assert kernel in ("stationary", "regs", "lds") and 1 <= splits <= 8 and third >= 1
+            if kernel == "stationary":
+                assert M <= 16 and K_ <= 8192 and 2 <= third <= 16
+    assert 2 <= K.stationary_strips(N, K_) <= 16
+
+
+def test_known_choices():
+    """The choices measured to be best at the Llama-3.1-8B layer sizes (they are what the
+    scoring was fitted to; a change of the scoring that moves them should be a decision)."""
+    assert K.skinny_plan(8, 28672, 4096)[0] == "stationary"
+    assert K.skinny_plan(8, 4096, 14336) == ("lds", 8, 1)
+    assert K.skinny_plan(8, 4096, 4096) == ("lds", 8, 1)
+    assert K.skinny_plan(64, 28672, 4096) == ("lds", 1, 1)
+    assert K.skinny_plan(64, 6144, 4096) == ("lds", 4, 1)
+    assert K.lds_splits(128, 4096, 14336) == 8
