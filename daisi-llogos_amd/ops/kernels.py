@@ -330,8 +330,32 @@ def stationary_strips(N: int, K: int, n_cus: int = 256) -> int:
     return best
 
 
+def resident_strips(M: int, N: int, K: int, n_cus: int = 256) -> Optional[Tuple[int, int]]:
+    """(parts of k, strips per block) for the few-row product whose operands go straight into
+    LDS, or None where it is not the faster one.  It pays for 17 to 64 rows on a tall matrix
+    whose blocks, 7 to 9 strips high, are all resident at once (two to a compute unit) and fill
+    at least nine tenths of those places: then the activations are read once per 112 to 144
+    rows of w and nothing waits for a second round.  Elsewhere the LDS few-row product with
+    its 64-row blocks was measured level or faster."""
+    if not (16 < M <= 64 and N >= 32768 and K % 64 == 0):
+        return None
+    n_strips = -(-N // 16)
+    places = 2 * n_cus
+    best, best_fill = None, 0.9
+    for strips in (9, 8, 7):
+        for parts in (1, 2):
+            if parts > 1 and K < 512 * parts:
+                continue
+            blocks = -(-n_strips // strips) * parts
+            fill = blocks / places
+            if blocks <= places and fill > best_fill:
+                best, best_fill = (parts, strips), fill
+    return best
+
+
 def skinny_plan(M: int, N: int, K: int) -> Tuple[str, int, int]:
     """(kernel, blocks along k, 16-row blocks of w per wave) for the few-row product.
+    'strips': both operands straight into LDS, blocks of several strips (see resident_strips).
     'stationary': activations held in registers while strips of w stream past; best for few
     rows and very many rows of w (gate/up, the head).  'regs': every wave fetches its own
     activation fragments; for up to 4 rows where k is too long for 'stationary'.  'lds': the
@@ -345,6 +369,9 @@ def skinny_plan(M: int, N: int, K: int) -> Tuple[str, int, int]:
     if M <= 4 and N >= 16384:
         strips = -(-N // 16)
         return "regs", max(1, min(-(-1024 // strips), K // 1024, 8)), 1
+    resident = resident_strips(M, N, K)
+    if resident is not None:
+        return "strips", resident[0], resident[1]             # third value: strips per block
     return "lds", lds_splits(M, N, K), 1
 
 
@@ -457,6 +484,36 @@ def gemm_skinny_lds_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.
     return out
 
 
+def gemm_strips_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype,
+                     splits: int, strips: int) -> Optional[torch.Tensor]:
+    """The bfloat16 product for up to 128 rows whose operands go straight into LDS, several
+    stages ahead, with blocks of `strips` 16-row strips of w: [parts, M, N], the same parts of k
+    and the same sums as gemm_skinny_lds_bf16.  None for shapes it does not take."""
+    if a.dtype != torch.bfloat16 or a.dim() != 2 or w.dtype != torch.bfloat16 or w.dim() != 2:
+        return None
+    M, K = a.shape
+    N = w.shape[0]
+    if not (0 < M <= LDS_MAX_ROWS and K % 64 == 0 and a.stride(1) == 1 and a.stride(0) % 8 == 0 and w.shape[1] == K
+            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and w.is_contiguous() and 2 <= strips <= 9):
+        return None
+    _dev(w, bias)
+    _need(a.is_cuda and a.device == w.device, "gemm: a and w must be on the same GPU")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.shape == (N,), "gemm: bias must be float32 [N]")
+    lib = _lib()
+    parts = lib.llogos_gemm_skinny_lds_parts(K, int(splits))
+    if parts > 1:
+        _need(bias is None, "gemm: a product in parts leaves the bias to its consumer")
+        out_dtype = torch.float32
+    out = torch.empty((parts, M, N), dtype=out_dtype, device=a.device)
+    code = lib.llogos_gemm_strips_bf16(_p(out), _DT[out_dtype], _p(a), a.stride(0), _p(w), _p(bias), M, N, K, N,
+                                       ctypes.c_longlong(M * N), int(splits), int(strips), _stream())
+    if code == -2:
+        return None
+    _check(code, "gemm_strips_bf16")
+    return out
+
+
 def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swiglu_input: bool = False,
                  f32_ok: bool = False) -> torch.Tensor:
     """a [M, K] . w [N, K]^T without bias, as [M, N] of `out_dtype` or as float32 partial sums
@@ -480,6 +537,13 @@ def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swigl
             kernel, splits, row_blocks = "lds", 1, 1
         elif kernel == "stationary":
             kernel, splits, row_blocks = "lds", 1, 1
+        if kernel == "strips":
+            if swiglu_input:
+                a, swiglu_input = swiglu(a, out_dtype), False
+            out = gemm_strips_bf16(a, w, None, few_dtype, splits, row_blocks) if a.dim() == 2 else None
+            if out is not None:
+                return out
+            kernel, splits, row_blocks = "lds", lds_splits(M, w.shape[0], w.shape[1]), 1
         # silu(gate) * up inside the product costs every block of rows of w a second read of the
         # gate/up row: worth it for few rows in bfloat16, not for partial sums or many rows
         if swiglu_input and not (M <= 16 and a.dtype == torch.bfloat16 and (a.dim() == 2 or a.shape[0] == 1)):
@@ -516,6 +580,9 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dty
             kernel, _, row_blocks = skinny_plan(M, w.shape[0], w.shape[1])
             if kernel == "stationary":
                 out = gemm_skinny_stationary_bf16(a, w, bias, out_dtype, row_blocks)
+                kernel, row_blocks = "lds", 1
+            elif kernel == "strips":
+                out = gemm_strips_bf16(a, w, bias, out_dtype, 1, row_blocks)
                 kernel, row_blocks = "lds", 1
             else:
                 out = None

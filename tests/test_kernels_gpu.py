@@ -159,6 +159,50 @@ def test_gemm_of_65_to_128_rows_on_the_matrix_cores(M, N, K_):
         assert torch.equal(few, many[:65])
 
 
+@pytest.mark.parametrize("M,N,K_", [(17, 3000, 1024), (33, 16 * 9 * 5 + 7, 2048), (64, 4096, 4096), (100, 777, 512), (128, 2048, 640)])
+def test_gemm_with_operands_straight_into_lds(M, N, K_):
+    """The third form of the few-row product: every height of its blocks and several numbers
+    of blocks along k; its results equal the LDS few-row product's bit for bit for the same
+    parts of k, whatever the height."""
+    rng = np.random.default_rng(9)
+    a = _t(rng.standard_normal((M, K_)), torch.bfloat16)
+    w = _t(rng.standard_normal((N, K_)) * 0.05, torch.bfloat16)
+    b = _t(rng.standard_normal(N))
+    want = pm.linear(_np(a), _np(w))
+    scale = np.abs(want).max()
+    for splits in (1, 2, 5):
+        same = K.gemm_skinny_lds_bf16(a, w, None, torch.float32, splits, 1)
+        for strips in (2, 3, 4, 7, 9):
+            out = K.gemm_strips_bf16(a, w, None, torch.float32, splits, strips)
+            assert out is not None and out.shape == same.shape
+            assert np.abs(_np(out).sum(0) - want).max() <= 2e-6 * scale * math.sqrt(K_)
+            assert torch.equal(out, same), (splits, strips)
+    out = K.gemm_strips_bf16(a, w, b, torch.bfloat16, 1, 7)
+    assert np.abs(_np(out)[0] - (want + _np(b))).max() <= 1e-2 * scale
+    wide = _t(rng.standard_normal((M, K_ + 24)), torch.bfloat16)              # a view with a row stride
+    out = K.gemm_strips_bf16(wide[:, :K_], w, None, torch.float32, 1, 8)
+    assert np.abs(_np(out)[0] - pm.linear(_np(wide)[:, :K_], _np(w))).max() <= 2e-6 * scale * math.sqrt(K_)
+    assert K.gemm_strips_bf16(a[:, :K_ - 8], w[:, :K_ - 8].contiguous(), None, torch.float32, 1, 7) is None   # k % 64
+    assert K.gemm_strips_bf16(a, w, None, torch.float32, 1, 10) is None                                       # too high
+
+
+def test_tall_products_through_the_dispatch_take_the_third_form():
+    """A matrix as tall as the Qwen3-14B gate/up projection, few columns: the plan for 17 to 64
+    rows is the third form, and a row's result is the same for every batch of such a class."""
+    rng = np.random.default_rng(10)
+    N, K_ = 34816, 1024
+    w = torch.randn((N, K_), device=DEV, dtype=torch.bfloat16, generator=torch.Generator(device=DEV).manual_seed(3)) * 0.05
+    a = _t(rng.standard_normal((64, K_)), torch.bfloat16)
+    assert K.skinny_plan(33, N, K_)[0] == "strips" and K.skinny_plan(64, N, K_) == K.skinny_plan(33, N, K_)
+    many = K.sum_parts(K.gemm_product(a, w, torch.bfloat16, f32_ok=True), None, torch.float32)
+    few = K.sum_parts(K.gemm_product(a[:33], w, torch.bfloat16, f32_ok=True), None, torch.float32)
+    assert torch.equal(few, many[:33])
+    want = _np(a.float() @ w.float().t())
+    assert np.abs(_np(many) - want).max() <= 2e-5 * max(1.0, np.abs(want).max())
+    plain = K.gemm(a, w, None, torch.float32)
+    assert np.abs(_np(plain) - want).max() <= 2e-5 * max(1.0, np.abs(want).max())
+
+
 def test_products_of_random_shapes_through_the_dispatch():
     """Whatever kernel and split of k the plan picks for a shape, the product is right: row
     counts up to 64 and beyond, widths and depths that are multiples of 8 and of nothing else."""

@@ -23,7 +23,7 @@ def test_a_plan_depends_on_the_class_of_the_row_count_only(N, K_):
             # registers for the fewest rows), but not within 1..4, 5..8 and 9..16
             assert len(plans) == 1, (N, K_, lo, hi, plans)
         else:
-            assert len(plans) == 1 and next(iter(plans))[0] == "lds", (N, K_, lo, hi, plans)
+            assert len(plans) == 1 and next(iter(plans))[0] in ("lds", "strips"), (N, K_, lo, hi, plans)
     assert len({K.lds_splits(M, N, K_) for M in range(65, 129)}) == 1
 
 
@@ -35,7 +35,10 @@ def test_plans_are_within_what_the_kernels_and_their_consumers_take(N, K_):
         assert parts == 1 or -(-K_ // 256) >= 2 * parts - 1        # every block along k has work
         if M <= 64:
             kernel, splits, third = K.skinny_plan(M, N, K_)
-            assert kernel in ("stationary", "regs", "lds") and 1 <= splits <= 8 and third >= 1
+            assert kernel in ("stationary", "regs", "lds", "strips") and 1 <= splits <= 8 and third >= 1
+            if kernel == "strips":
+                blocks = -(-(-(-N // 16)) // third) * splits
+                assert 16 < M and 7 <= third <= 9 and K_ % 64 == 0 and 0.9 * 512 < blocks <= 512
             if kernel == "stationary":
                 assert M <= 16 and K_ <= 8192 and 2 <= third <= 16
     assert 2 <= K.stationary_strips(N, K_) <= 16
@@ -50,3 +53,7 @@ def test_known_choices():
     assert K.skinny_plan(64, 28672, 4096) == ("lds", 1, 1)
     assert K.skinny_plan(64, 6144, 4096) == ("lds", 4, 1)
     assert K.lds_splits(128, 4096, 14336) == 8
+    # tall matrices whose blocks of 7 to 9 strips are all resident at once: operands straight into LDS
+    assert K.skinny_plan(32, 34816, 5120) == ("strips", 2, 9) and K.skinny_plan(64, 34816, 5120) == ("strips", 2, 9)
+    assert K.skinny_plan(64, 57344, 8192) == ("strips", 1, 7)
+    assert K.skinny_plan(16, 57344, 8192)[0] == "stationary" and K.skinny_plan(64, 128256, 4096)[0] == "lds"
