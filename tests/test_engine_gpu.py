@@ -12,6 +12,8 @@ import gpu_helpers as H
 import plain_model as pm
 import tiny_configs as tc
 
+K = importlib.import_module("daisi-llogos_amd.ops.kernels")
+
 pytestmark = pytest.mark.gpu
 CONFIGS = ["tiny_a", "tiny_b", "tiny_c", "tiny_w", "tiny_d"]
 
@@ -285,6 +287,35 @@ def test_replayed_steps_equal_steps_launched_kernel_by_kernel(name, dtype):
         if outs:
             assert torch.equal(outs[0], outs[1]), (what, arg)
     assert len(engines[0].graphs.graphs) >= 2
+
+
+def test_replayed_steps_of_twenty_sequences():
+    """The same with 20 sequences at the Qwen3-14B layer sizes, where the gate/up product takes
+    the kernel whose operands go straight into LDS: its launches replay like the others'."""
+    name, dtype, n = "layer_14b", "bfloat16", 20
+    assert K.skinny_plan(n, 2 * tc.ALL[name]["intermediate_size"], tc.ALL[name]["hidden_size"])[0] == "strips"
+    engines = [H.engine(name, dtype, max_tokens=64 * (n + 2), n_slots=n + 1, use_graphs=g) for g in (True, False)]
+    rng = np.random.default_rng(4)
+    vocab = tc.ALL[name]["vocab_size"]
+    new = lambda k: [int(t) for t in rng.integers(0, vocab, k)]
+    prompts = [new(3 + i % 4) for i in range(n)]
+    slots = [[eng.alloc_slot() for _ in range(n)] for eng in engines]
+    outs = [eng.step(list(zip(sl, prompts)), want="last") for eng, sl in zip(engines, slots)]
+    assert torch.equal(outs[0], outs[1])
+    extra = [None, None]
+    for t in range(5):
+        toks = new(n)
+        outs = [eng.step([(s, [tok]) for s, tok in zip(sl, toks)], want="last") for eng, sl in zip(engines, slots)]
+        assert torch.equal(outs[0], outs[1]), t
+        if t == 1:                                       # other work between the replays
+            p = new(40)
+            for e, eng in enumerate(engines):
+                extra[e] = eng.alloc_slot()
+                eng.step([(extra[e], p)], want=None)
+        if t == 2:
+            for e, eng in enumerate(engines):
+                eng.free_slot(extra[e])
+    assert len(engines[0].graphs.graphs) >= 1
 
 
 def test_captured_steps_are_dropped_and_made_again(monkeypatch):
