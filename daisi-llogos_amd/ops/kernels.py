@@ -332,24 +332,29 @@ def stationary_strips(N: int, K: int, n_cus: int = 256) -> int:
 
 def resident_strips(M: int, N: int, K: int, n_cus: int = 256) -> Optional[Tuple[int, int]]:
     """(parts of k, strips per block) for the few-row product whose operands go straight into
-    LDS, or None where it is not the faster one.  It pays for 17 to 64 rows on a tall matrix
-    whose blocks, 7 to 9 strips high, are all resident at once (two to a compute unit) and fill
-    at least nine tenths of those places: then the activations are read once per 112 to 144
-    rows of w and nothing waits for a second round.  Elsewhere the LDS few-row product with
-    its 64-row blocks was measured level or faster."""
-    if not (16 < M <= 64 and N >= 32768 and K % 64 == 0):
+    LDS, or None where it is not the faster one.  It pays for 17 to 64 rows on a tall, large
+    matrix when its blocks, 5 to 9 strips high, are all resident at once (two to a compute
+    unit) and fill most of those places, while the LDS few-row product's 64-row blocks either
+    need a second round or leave a fifth more of the places empty: then the activations are
+    read once per 80 to 144 rows of w and nothing waits for a second round (measured on the
+    gate/up matrices of eight model sizes: 6 to 20 % faster where this says so, level or
+    slower where it does not, among them everything below 24576 rows)."""
+    if not (16 < M <= 64 and N >= 24576 and K % 64 == 0):
         return None
-    n_strips = -(-N // 16)
     places = 2 * n_cus
-    best, best_fill = None, 0.9
-    for strips in (9, 8, 7):
+    other = -(-N // 64) * lds_splits(M, N, K)
+    other_fill = other / places if other <= places else 0.0
+    n_strips = -(-N // 16)
+    best, best_fill = None, 0.0
+    for strips in (9, 8, 7, 6, 5):
         for parts in (1, 2):
             if parts > 1 and K < 512 * parts:
                 continue
             blocks = -(-n_strips // strips) * parts
-            fill = blocks / places
-            if blocks <= places and fill > best_fill:
-                best, best_fill = (parts, strips), fill
+            if blocks <= places and blocks / places > best_fill:
+                best, best_fill = (parts, strips), blocks / places
+    if best is None or best_fill < 0.75 or best_fill - other_fill < 0.2:
+        return None
     return best
 
 

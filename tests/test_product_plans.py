@@ -8,7 +8,8 @@ import pytest
 
 K = importlib.import_module("daisi-llogos_amd.ops.kernels")
 
-SHAPES = [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336), (128256, 4096),      # Llama-3.1-8B
+SHAPES = [(24576, 4096), (37888, 3584), (51200, 5120), (59136, 8192),                     # other models' gate/up
+          (6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336), (128256, 4096),      # Llama-3.1-8B
           (7168, 5120), (5120, 5120), (34816, 5120), (5120, 17408), (151936, 5120),      # Qwen3-14B
           (10240, 8192), (8192, 8192), (57344, 8192), (8192, 28672),                     # Llama-3.1-70B
           (3072, 2048), (16384, 2048), (2048, 8192), (331, 80), (96, 1000), (17, 8)]
@@ -38,7 +39,7 @@ def test_plans_are_within_what_the_kernels_and_their_consumers_take(N, K_):
             assert kernel in ("stationary", "regs", "lds", "strips") and 1 <= splits <= 8 and third >= 1
             if kernel == "strips":
                 blocks = -(-(-(-N // 16)) // third) * splits
-                assert 16 < M and 7 <= third <= 9 and K_ % 64 == 0 and 0.9 * 512 < blocks <= 512
+                assert 16 < M and 5 <= third <= 9 and K_ % 64 == 0 and 0.75 * 512 <= blocks <= 512
             if kernel == "stationary":
                 assert M <= 16 and K_ <= 8192 and 2 <= third <= 16
     assert 2 <= K.stationary_strips(N, K_) <= 16
@@ -53,7 +54,12 @@ def test_known_choices():
     assert K.skinny_plan(64, 28672, 4096) == ("lds", 1, 1)
     assert K.skinny_plan(64, 6144, 4096) == ("lds", 4, 1)
     assert K.lds_splits(128, 4096, 14336) == 8
-    # tall matrices whose blocks of 7 to 9 strips are all resident at once: operands straight into LDS
+    # tall matrices whose blocks of 5 to 9 strips are all resident at once: operands straight into LDS
     assert K.skinny_plan(32, 34816, 5120) == ("strips", 2, 9) and K.skinny_plan(64, 34816, 5120) == ("strips", 2, 9)
     assert K.skinny_plan(64, 57344, 8192) == ("strips", 1, 7)
     assert K.skinny_plan(16, 57344, 8192)[0] == "stationary" and K.skinny_plan(64, 128256, 4096)[0] == "lds"
+    assert K.skinny_plan(64, 24576, 4096) == ("strips", 2, 6) and K.skinny_plan(32, 37888, 3584) == ("strips", 1, 5)
+    assert K.skinny_plan(64, 51200, 5120) == ("strips", 1, 7) and K.skinny_plan(64, 59136, 8192) == ("strips", 1, 8)
+    # ... and not where the LDS few-row product's own blocks fill one round well, or the matrix is small
+    assert K.skinny_plan(64, 28672, 4096)[0] == "lds" and K.skinny_plan(32, 28672, 4096)[0] == "lds"
+    assert K.skinny_plan(64, 16384, 3072)[0] == "lds" and K.skinny_plan(64, 19456, 2560)[0] == "lds"
