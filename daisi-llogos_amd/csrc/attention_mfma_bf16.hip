@@ -389,26 +389,47 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_decode_kernel(
     }
 }
 
-// grid (batch, heads); HD threads.  Adds the partial results of the blocks along the context,
-// each of which covered pages_per_block pages.  (Letting the last block to finish add them,
-// behind a device-wide fence and a ticket counter, was measured: the fence writes back whatever
-// earlier kernels left dirty in the L2 and cost 20 us a layer at batch 8; this kernel costs 4.6.)
+// grid (batch, heads); kMergeLanes x HD threads.  Adds the partial results of the blocks along
+// the context, each of which covered pages_per_block pages: thread (j, d) takes blocks j,
+// j + kMergeLanes, ... of dimension d, and LDS adds the kMergeLanes sums in ascending j, so the
+// order depends on the sequence's own length alone.  (One thread per dimension walking all
+// blocks took 17 us at 33 blocks: a chain of dependent L2 latencies.  Letting the last block
+// to finish add them, behind a device-wide fence and a ticket counter, was measured too: the
+// fence writes back whatever earlier kernels left dirty in the L2 and cost 20 us a layer at
+// batch 8; this kernel costs 4.6.)
+constexpr int kMergeLanes = 4;
+
 template <int HD>
-__global__ void attn_decode_merge_kernel(bf16_t* __restrict__ out, const float* __restrict__ partial,
-                                         const int* __restrict__ tok_pos, int n_heads, int n_z, int pages_per_block) {
-    const int b = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
+__global__ __launch_bounds__(kMergeLanes * HD) void attn_decode_merge_kernel(
+        bf16_t* __restrict__ out, const float* __restrict__ partial, const int* __restrict__ tok_pos,
+        int n_heads, int n_z, int pages_per_block) {
+    __shared__ float lds_m[kMergeLanes], lds_l[kMergeLanes], lds_o[kMergeLanes][HD];
+    const int b = blockIdx.x, h = blockIdx.y, d = threadIdx.x % HD, j = threadIdx.x / HD;
     const int n_pages = tok_pos[b] / kPageTokens + 1;
     const int used = min(n_z, (n_pages + pages_per_block - 1) / pages_per_block);
     const float* src = partial + ((size_t)b * n_heads + h) * n_z * (HD + 2);
     float m = -INFINITY;
-    for (int z = 0; z < used; ++z) m = fmaxf(m, src[(size_t)z * (HD + 2)]);
+#pragma unroll 4
+    for (int z = j; z < used; z += kMergeLanes) m = fmaxf(m, src[(size_t)z * (HD + 2)]);
+    if (d == 0) lds_m[j] = m;
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kMergeLanes; ++i) m = fmaxf(m, lds_m[i]);
     float l = 0.f, o = 0.f;
-    for (int z = 0; z < used; ++z) {
+#pragma unroll 4
+    for (int z = j; z < used; z += kMergeLanes) {
         const float* p = src + (size_t)z * (HD + 2);
         const float f = (p[0] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(p[0] - m);
         l += p[1] * f;
         o += p[2 + d] * f;
     }
+    lds_o[j][d] = o;
+    if (d == 0) lds_l[j] = l;
+    __syncthreads();
+    if (j != 0) return;
+    l = lds_l[0]; o = lds_o[0][d];
+#pragma unroll
+    for (int i = 1; i < kMergeLanes; ++i) { l += lds_l[i]; o += lds_o[i][d]; }
     out[((size_t)b * n_heads + h) * HD + d] = f32_to_bf16(l > 0.f ? o / l : 0.f);
 }
 
@@ -772,7 +793,7 @@ static int launch_decode(void* out, const void* q, int q_stride, const QkvSource
     attn_decode_kernel<HD, W, FUSED><<<grid, W * kWave, smem, stream>>>( \
         (bf16_t*)out, workspace, (const bf16_t*)q, q_stride, FUSED ? *src : none, (const bf16_t*)k_pool, \
         (const bf16_t*)v_pool, table, table_stride, tok_pos, n_heads, n_kv_heads, group, scale, window, sinks); \
-    if (n_z > 1) attn_decode_merge_kernel<HD><<<mgrid, HD, 0, stream>>>((bf16_t*)out, workspace, tok_pos, n_heads, \
+    if (n_z > 1) attn_decode_merge_kernel<HD><<<mgrid, kMergeLanes * HD, 0, stream>>>((bf16_t*)out, workspace, tok_pos, n_heads, \
                                                                         n_z, W); } while (0)
 #define BY_WAVES(HD, FUSED) do { if (waves == 16) GO(HD, 16, FUSED); else if (waves == 8) GO(HD, 8, FUSED); \
                                  else GO(HD, 4, FUSED); } while (0)

@@ -301,9 +301,10 @@ def _attention_case(dtype, nh, nkv, hd, lens, new, window=0, sinks=0, seed=4, sc
     for b in range(B):
         kb, vb = _t(ks[b], DT[dtype]), _t(vs[b], DT[dtype])
         ks[b], vs[b] = _np(kb), _np(vb)
-        for p in range(lens[b]):
-            kp[table[b, p // 64], :, p % 64, :] = kb[p].view(nkv, hd)
-            vp[table[b, p // 64], :, :, p % 64] = vb[p].view(nkv, hd)
+        for p0 in range(0, lens[b], 64):                                # page by page
+            n = min(64, lens[b] - p0)
+            kp[table[b, p0 // 64], :, :n, :] = kb[p0:p0 + n].view(n, nkv, hd).permute(1, 0, 2)
+            vp[table[b, p0 // 64], :, :, :n] = vb[p0:p0 + n].view(n, nkv, hd).permute(1, 2, 0)
     stride = nh * hd + 24                                               # queries sit in a wider row
     qbuf = _t(rng.standard_normal((T, stride)) * scale_q, DT[dtype])
     tok_seq = np.repeat(np.arange(B), new).astype(np.int32)
@@ -348,7 +349,8 @@ def test_attention_whole_prompts_and_single_tokens(dtype, nh, nkv, hd):
 @pytest.mark.parametrize("nh,nkv,hd,batch,longest", [(8, 4, 128, 64, 700),      # 16 pages a block, no merge
                                                      (8, 4, 64, 70, 1500),       # 16 pages a block, merged
                                                      (16, 2, 64, 128, 700),      # 8 pages a block, merged
-                                                     (8, 4, 128, 3, 1500)])      # 4 pages a block
+                                                     (8, 4, 128, 4, 1500),       # 4 pages a block, 6 blocks merged
+                                                     (4, 1, 128, 4, 3300)])      # 13 blocks merged
 def test_single_token_attention_with_blocks_of_every_size(nh, nkv, hd, batch, longest):
     """The decode kernel gives a block more pages when there are many blocks; every form must
     agree with the plain attention, whatever the lengths of the other sequences."""
