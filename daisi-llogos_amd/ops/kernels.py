@@ -754,20 +754,30 @@ def sample_prepare(logits: torch.Tensor, history: Optional[torch.Tensor], histor
     return work
 
 
+SAMPLE_ORDERS = {"single": 0, "head": 1, "whole": 2}
+
+
 def sample_pipeline(work: torch.Tensor, uniforms: torch.Tensor, top_k: int, top_p: float, min_p: float,
-                    typical_p: float, min_keep: int) -> torch.Tensor:
-    """Token ids int32 [R] drawn from prepared rows `work` (overwritten) with one uniform
-    number per row: top-k, min-p, softmax, typical-p, top-p, draw."""
+                    typical_p: float, min_keep: int, order: str = "head") -> torch.Tensor:
+    """Token ids int32 [R] drawn from prepared rows `work` with one uniform number per row:
+    top-k, min-p, softmax, typical-p, top-p, draw.  order "head": a row is first tried with
+    the head of its descending order alone (a histogram finds it; no sort of the vocabulary),
+    and rows that this cannot decide are sorted whole by many blocks; "whole": every row is
+    sorted so; "single": every row is sorted by its own block (slow, the plain form).  Rows
+    sorted whole are overwritten with probabilities."""
     _dev(work, uniforms)
     _need(work.dtype == torch.float32 and work.dim() == 2, "sample_pipeline: work must be float32 [R, V]")
+    _need(order in SAMPLE_ORDERS, f"sample_pipeline: order must be one of {sorted(SAMPLE_ORDERS)}")
     R, V = work.shape
     _need(uniforms.dtype == torch.float32 and uniforms.numel() == R, "sample_pipeline: one float32 uniform per row")
     n_pad = 1
     while n_pad < V:
         n_pad <<= 1
     scratch = torch.empty((R, n_pad), dtype=torch.int64, device=work.device)
+    prob = torch.empty_like(work) if order == "head" else None
     out = torch.empty((R,), dtype=torch.int32, device=work.device)
     _check(_lib().llogos_sample_pipeline(
-        _p(out), _p(work), R, V, _p(scratch), n_pad, _p(uniforms), int(top_k), ctypes.c_float(top_p),
-        ctypes.c_float(min_p), ctypes.c_float(typical_p), int(min_keep), _stream()), "sample_pipeline")
+        _p(out), _p(work), _p(prob), R, V, _p(scratch), n_pad, _p(uniforms), int(top_k), ctypes.c_float(top_p),
+        ctypes.c_float(min_p), ctypes.c_float(typical_p), int(min_keep), SAMPLE_ORDERS[order], _stream()),
+        "sample_pipeline")
     return out

@@ -137,3 +137,134 @@ def test_sampled_generation_draws_what_the_plain_sampler_draws():
             want = pm.sample(logits[len(p) + i - 1], u, history=p + toks[:i], **opts)
             differ += int(want != t)
     assert differ == 0
+
+
+def _every_way(rows, us, **opts):
+    """Tokens drawn with the head of the order alone where that decides, with every row sorted
+    whole by many blocks, and with every row sorted by its own block."""
+    K = importlib.import_module("daisi-llogos_amd.ops.kernels")
+    p = S.GenerationParams(**opts)
+    out = []
+    for order in ("head", "whole", "single"):
+        work = K.sample_prepare(rows, None, None, 1.0, 0.0, 0.0, p.temperature, True)
+        u = torch.tensor(np.asarray(us, dtype=np.float32), device=DEV)
+        out.append(K.sample_pipeline(work, u, p.top_k, p.top_p, p.min_p, p.typical_p, p.min_keep, order=order).cpu().tolist())
+    return out
+
+
+def _peaked_rows(rng, R, V, spread):
+    """Rows like a language model's: a few likely tokens, a long tail `spread` units wide."""
+    rows = rng.standard_normal((R, V)).astype(np.float32) * spread
+    for r in range(R):
+        rows[r, rng.integers(0, V, 30)] += rng.random(30).astype(np.float32) * 4 * spread
+    return rows
+
+
+def _intervals(row, u_count, temperature, top_k, top_p, min_p=0.0, min_keep=1, **_):
+    """The pipeline without typical-p in float64, vectorised for a large vocabulary: for every
+    token the interval of uniform numbers that draws it (empty for tokens that are cut)."""
+    work = row.astype(np.float64) / temperature
+    order = np.lexsort((np.arange(len(work)), -work))
+    n = top_k if 0 < top_k < len(work) else len(work)
+    keep = max(min_keep, 1)
+    if 0 < min_p < 1 and n > keep:
+        n = max(keep, int((work[order[:n]] >= work[order[0]] + np.log(min_p)).sum()))
+    cand = order[:n]
+    p = np.exp(work[cand] - work[cand[0]])
+    p /= p.sum()
+    if 0 < top_p < 1:
+        cut = np.nonzero((np.cumsum(p) > top_p) & (np.arange(n) + 1 >= keep))[0]
+        if len(cut):
+            cand, p = cand[:cut[0] + 1], p[:cut[0] + 1] / p[:cut[0] + 1].sum()
+    hi = np.cumsum(p)
+    lo_all, hi_all = np.ones(len(work)), np.zeros(len(work))
+    lo_all[cand], hi_all[cand] = hi - p, hi
+    return lo_all, hi_all
+
+
+HEAD_OPTS = [
+    dict(temperature=0.7, top_k=40, top_p=0.9),
+    dict(temperature=0.7, top_k=0, top_p=0.9),
+    dict(temperature=1.0, top_k=0, top_p=1.0),
+    dict(temperature=1.0, top_k=0, top_p=0.98, min_p=0.001),
+    dict(temperature=0.9, top_k=2048, top_p=1.0, min_keep=100),
+    dict(temperature=0.9, top_k=3000, top_p=0.95),                      # more than the head holds: sorted whole
+    dict(temperature=0.8, top_k=500, top_p=0.9, typical_p=0.8),
+    dict(temperature=0.8, top_k=0, top_p=0.9, typical_p=0.8),           # typical-p over the vocabulary: sorted whole
+]
+
+
+@pytest.mark.parametrize("opts", HEAD_OPTS)
+@pytest.mark.parametrize("V,spread", [(128256, 2.0), (151936, 0.5), (5000, 3.0)])
+def test_the_head_of_the_order_decides_as_the_whole_order_does(opts, V, spread):
+    """Rows like a language model's, with equal values, banned halves and the ends of the range
+    of uniform numbers.  Both ways must draw the same tokens; a small vocabulary is compared with
+    the plain sampler, a large one with the intervals of the cumulative distribution in float64:
+    the uniform number lies in the drawn token's interval, within what float32 sums of 10^5 terms
+    can be off (1e-5)."""
+    rng = np.random.default_rng(V + int(opts["top_k"]))
+    R = 12
+    rows = _peaked_rows(rng, R, V, spread)
+    rows[1, 7] = rows[1, 9] = rows[1].max() + 1.0                       # equal values at the top
+    rows[2, rng.integers(0, V, V // 2)] = -np.inf                       # half of the row banned
+    rows[3] = np.round(rows[3] * 2) / 2                                 # many equal values everywhere
+    us = rng.random(R).astype(np.float32)
+    us[4], us[5] = 0.0, np.float32(1.0 - 2 ** -24)                      # the ends of the range
+    head, whole, single = _every_way(torch.tensor(rows, device=DEV), us, repetition_penalty=1.0, **opts)
+    assert whole == single                                              # the same order, the same sums
+    # a draw within float rounding of a boundary of the cumulative sum may fall either way
+    assert sum(a != b for a, b in zip(head, whole)) <= 1, (head, whole)
+    if V <= 5000:
+        p = S.GenerationParams(repetition_penalty=1.0, **opts)
+        want = [_plain(rows[r], p, [us[r]])[0] for r in range(R)]
+        assert sum(a != b for a, b in zip(head, want)) <= 1, (head, want)
+    elif "typical_p" not in opts:
+        off = 0
+        for r in range(R):
+            lo, hi = _intervals(rows[r], us[r], **opts)
+            off += not (lo[head[r]] - 1e-5 <= us[r] <= hi[head[r]] + 1e-5)
+        assert off <= 1, (opts, head)
+
+
+def test_rows_the_head_cannot_hold():
+    """Every logit equal (one bin holds the row), a flat row of which top-p needs nine tenths, a
+    row whose largest is infinite: the whole order decides, and gives what the plain sampler gives."""
+    V = 20000
+    us = [0.0, 0.3, 0.77, 0.999]
+    for row, opts in ((np.ones(V, np.float32), dict(temperature=1.0, top_k=0, top_p=0.9)),
+                      (np.ones(V, np.float32), dict(temperature=1.0, top_k=50, top_p=1.0)),
+                      (np.linspace(0, 0.01, V).astype(np.float32), dict(temperature=1.0, top_k=0, top_p=0.9)),
+                      (np.linspace(0, 100, V).astype(np.float32), dict(temperature=1.0, top_k=0, top_p=1.0))):
+        rows = torch.tensor(np.tile(row, (len(us), 1)), device=DEV)
+        head, whole, single = _every_way(rows, us, repetition_penalty=1.0, **opts)
+        p = S.GenerationParams(repetition_penalty=1.0, **opts)
+        assert head == whole == single == _plain(row, p, us), opts
+    inf_row = np.zeros(V, np.float32)
+    inf_row[5] = np.inf
+    rows = torch.tensor(np.tile(inf_row, (2, 1)), device=DEV)
+    head, whole, single = _every_way(rows, [0.2, 0.8], temperature=1.0, top_k=40, top_p=0.9, repetition_penalty=1.0)
+    assert head == whole == single
+
+
+def test_candidates_far_below_the_largest():
+    """A low temperature spreads the candidates over a hundred units (coarse bins), and a row
+    may have fewer tokens of probability above 0 than top-k or min_keep ask for: the head then
+    holds every token that can be drawn."""
+    rng = np.random.default_rng(11)
+    V = 50000
+    us = [0.0, 0.41, 0.93, 0.9999]
+    wide = (rng.standard_normal(V) * 3).astype(np.float32)
+    few = np.full(V, -np.inf, np.float32)
+    few[[3, 77, 4000, 9, 12]] = [1.0, 0.5, 0.2, -200.0, -90.0]
+    steep = (-np.arange(V) * 0.5).astype(np.float32)                    # one token per coarse bin, then exact zeros
+    for row, opts in ((wide, dict(temperature=0.1, top_k=40, top_p=0.95)),
+                      (wide, dict(temperature=0.05, top_k=0, top_p=1.0)),
+                      (wide, dict(temperature=0.1, top_k=1000, top_p=1.0, min_p=1e-30)),
+                      (few, dict(temperature=1.0, top_k=40, top_p=0.9)),
+                      (few, dict(temperature=1.0, top_k=0, top_p=1.0, min_keep=20)),
+                      (steep, dict(temperature=1.0, top_k=0, top_p=0.999)),
+                      (steep, dict(temperature=1.0, top_k=500, top_p=1.0, typical_p=0.9))):
+        rows = torch.tensor(np.tile(row, (len(us), 1)), device=DEV)
+        head, whole, single = _every_way(rows, us, repetition_penalty=1.0, **opts)
+        p = S.GenerationParams(repetition_penalty=1.0, **opts)
+        assert head == whole == single == _plain(row, p, us), opts
