@@ -26,8 +26,9 @@ class KVGroup:
         self.pages = GroupPages(n_pages, spec.window, spec.sinks)
         self.k = self.v = None
         if rt is not None:
-            # keys [.., token in page, head size]; values transposed [.., head size, token in page]
-            shape = (len(entries), n_pages, spec.n_kv_heads, PAGE_TOKENS, spec.head_dim)
+            # keys [.., token in page, head size]; values transposed [.., head size, token in page];
+            # one page more than the pool hands out: the page of padding rows (Cache.pad_page)
+            shape = (len(entries), n_pages + 1, spec.n_kv_heads, PAGE_TOKENS, spec.head_dim)
             self.k = torch.zeros(shape, dtype=rt.dtype, device=rt.device)
             self.v = torch.zeros(shape[:3] + (spec.head_dim, PAGE_TOKENS), dtype=rt.dtype, device=rt.device)
 
@@ -67,7 +68,8 @@ class Cache:
         if rt is not None:
             for e, st in enumerate(self.state_specs):
                 if st is not None:
-                    self.states[e] = torch.zeros((n_slots,) + tuple(st.shape), dtype=st.dtype, device=rt.device)
+                    # one row more than there are slots: the state of padding rows (pad_slot)
+                    self.states[e] = torch.zeros((n_slots + 1,) + tuple(st.shape), dtype=st.dtype, device=rt.device)
 
     # ---- slots ------------------------------------------------------------------
     def alloc_slot(self) -> int:
@@ -93,9 +95,20 @@ class Cache:
         self.slots.grow(n_slots)
         for e, st in enumerate(self.states):
             if st is not None:
-                bigger = torch.zeros((n_slots,) + tuple(st.shape[1:]), dtype=st.dtype, device=st.device)
-                bigger[:old].copy_(st)
+                bigger = torch.zeros((n_slots + 1,) + tuple(st.shape[1:]), dtype=st.dtype, device=st.device)
+                bigger[:old].copy_(st[:old])
                 self.states[e] = bigger
+
+    # A step that is replayed from a captured graph may carry rows that belong to no sequence, so
+    # that a few captured batch sizes serve every batch.  Such a row writes its key, value and
+    # state somewhere nobody reads: a page and a state row that are never handed out.
+    @property
+    def pad_slot(self) -> int:
+        return self.slots.n_slots
+
+    @property
+    def pad_page(self) -> int:
+        return self.n_pages
 
     def length(self, slot: int) -> int:
         self.slots.check(slot)

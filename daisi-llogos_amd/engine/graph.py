@@ -20,11 +20,25 @@ from ..ops import kernels as K
 from ..parts.base import StepContext
 
 TABLE_BUCKET = 16          # page-table widths are rounded up to this many pages (1024 positions)
-MAX_GRAPHS = 32
+MAX_GRAPHS = 64
+# Batch sizes that are captured.  A batch between two of them runs as the next larger one with
+# padding rows (token 0 at position 0 of a page and a state row that belong to no sequence),
+# so that a batch whose sequences end one after the other does not capture a graph for every
+# size on its way down (a capture costs about three replays).  Up to 8 every size is its own;
+# above, a size and its bucket are in the same class of row counts of the few-row products
+# (16, 32, 64), so a sequence's logits are the same bits with and without the padding.
+BATCH_BUCKETS = (1, 2, 3, 4, 5, 6, 7, 8, 12, 16, 24, 32, 48, 64)
 
 
 def bucket_width(width: int) -> int:
     return -(-max(1, width) // TABLE_BUCKET) * TABLE_BUCKET
+
+
+def bucket_batch(batch: int) -> int:
+    for b in BATCH_BUCKETS:
+        if batch <= b:
+            return b
+    return batch
 
 
 class DecodeGraph:
@@ -117,7 +131,18 @@ class GraphCache:
         self.graphs.clear()
 
     def step(self, ids, tok_pos, slot_ids, tables: List[np.ndarray], device_ids=None) -> torch.Tensor:
-        key = (len(slot_ids), tuple(bucket_width(t.shape[1]) for t in tables))
+        B = len(slot_ids)
+        pad = bucket_batch(B) - B
+        if pad:
+            cache = self._engine().cache
+            zeros = np.zeros(pad, dtype=np.int32)
+            ids, tok_pos = np.concatenate([ids, zeros]), np.concatenate([tok_pos, zeros])
+            slot_ids = np.concatenate([slot_ids, np.full(pad, cache.pad_slot, dtype=np.int32)])
+            rows = np.full((pad, 1), cache.pad_page, dtype=np.int32)
+            tables = [np.concatenate([t, np.pad(rows, ((0, 0), (0, t.shape[1] - 1)), constant_values=-1)]) for t in tables]
+            if device_ids is not None:
+                device_ids = (device_ids[0], list(device_ids[1]) + [0] * pad)
+        key = (B + pad, tuple(bucket_width(t.shape[1]) for t in tables))
         g = self.graphs.get(key)
         if g is None:
             while len(self.graphs) >= MAX_GRAPHS:
@@ -126,4 +151,5 @@ class GraphCache:
             self.graphs[key] = g
         else:
             self.graphs.move_to_end(key)
-        return g.run(ids, tok_pos, slot_ids, tables, device_ids)
+        logits = g.run(ids, tok_pos, slot_ids, tables, device_ids)
+        return logits[:B] if pad else logits

@@ -336,6 +336,43 @@ def test_captured_steps_are_dropped_and_made_again(monkeypatch):
         assert len(engines[0].graphs.graphs) <= 2
 
 
+@pytest.mark.parametrize("dtype", H.DTYPES)
+def test_a_batch_that_shrinks_replays_a_few_captured_sizes(dtype):
+    """19 sequences that end one after the other: the steps between two captured batch sizes
+    run as the larger one with padding rows, which belong to no sequence; every sequence's
+    logits are, bit for bit, those of uncaptured steps without padding, also for sequences that
+    start in the slots and pages the ended ones gave back."""
+    graph_mod = importlib.import_module("daisi-llogos_amd.engine.graph")
+    name, n = "tiny_a", 19
+    engines = [H.engine(name, dtype, max_tokens=64 * (n + 4), n_slots=n, use_graphs=g) for g in (True, False)]
+    rng = np.random.default_rng(12)
+    vocab = tc.ALL[name]["vocab_size"]
+    new = lambda k: [int(t) for t in rng.integers(0, vocab, k)]
+    prompts = [new(1 + (7 * i) % 11) for i in range(n)]
+    slots = [[eng.alloc_slot() for _ in range(n)] for eng in engines]
+    outs = [eng.step(list(zip(sl, prompts)), want="last") for eng, sl in zip(engines, slots)]
+    assert torch.equal(outs[0], outs[1])
+    live = list(range(n))
+    while live:
+        toks = new(len(live))
+        outs = [eng.step([(sl[r], [t]) for r, t in zip(live, toks)], want="last") for eng, sl in zip(engines, slots)]
+        assert torch.equal(outs[0], outs[1]), len(live)
+        gone = live.pop(int(rng.integers(0, len(live))))
+        for eng, sl in zip(engines, slots):
+            eng.free_slot(sl[gone])
+    sizes = {key[0] for key in engines[0].graphs.graphs}
+    assert sizes <= set(graph_mod.BATCH_BUCKETS) and sizes == {graph_mod.bucket_batch(b) for b in range(1, n + 1)}
+    # the slots and pages that came back, used again at a size with padding
+    for eng in engines:
+        assert eng.cache.live_slots == [] and len(set(eng.cache.free_pages())) == 1
+    slots = [[eng.alloc_slot() for _ in range(10)] for eng in engines]
+    prompts = [new(2 + i) for i in range(10)]
+    for _ in range(3):
+        outs = [eng.step(list(zip(sl, prompts)), want="last") for eng, sl in zip(engines, slots)]
+        assert torch.equal(outs[0], outs[1])
+        prompts = [[int(t)] for t in rng.integers(0, vocab, 10)]
+
+
 @pytest.mark.parametrize("graphs", [True, False])
 @pytest.mark.parametrize("dtype", H.DTYPES)
 def test_a_step_can_take_its_tokens_from_the_device(dtype, graphs):
