@@ -4,7 +4,8 @@ from the cache; logits come back for the wanted places.
 The reference has two step shapes for one sequence: a whole prompt
 (ForwardBatchedPrefill, Daisi.Llogos/Inference/ForwardPass.cs:630-697) and one token
 (Forward, :174-184).  Here a step takes any number of sequences with unequal token
-counts; no padding token enters any kernel."""
+counts; sequences are not padded to a common length.  (A replayed single-token step may
+carry whole rows that belong to no sequence, see graph.py; no kernel mixes rows.)"""
 from __future__ import annotations
 
 import os
