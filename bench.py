@@ -78,6 +78,9 @@ def main(argv=None) -> int:
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration has (0 = all)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--only-prefill", action="store_true", help="time the 2,048-token prompt alone (for profiling)")
+    ap.add_argument("--temperature", type=float, default=0.0, help="0 = greedy (the default run); above 0 the sampler draws")
+    ap.add_argument("--top-k", type=int, default=40)
+    ap.add_argument("--top-p", type=float, default=0.9)
     args = ap.parse_args(argv)
     prefill_tokens = args.prefill_tokens
     if args.gpus != 1:
@@ -103,15 +106,30 @@ def main(argv=None) -> int:
     print(f"[bench] model ready in {time.time() - t0:.1f} s; weights {weight_bytes(cfg) / 1e9:.2f} GB, "
           f"cache {eng.cache.bytes() / 1e9:.2f} GB", file=sys.stderr, flush=True)
     rng = np.random.default_rng(0)
+    if args.temperature > 0:
+        S = importlib.import_module("daisi-llogos_amd.sampling")
+        sampler = S.Sampler(S.GenerationParams(temperature=args.temperature, top_k=args.top_k, top_p=args.top_p,
+                                               repetition_penalty=1.0, seed=0))
+        sampling = f"temperature {args.temperature:g}, top-k {args.top_k}, top-p {args.top_p:g}"
+    else:
+        sampler, sampling = None, "greedy"
+
+    def pick(logits, step):
+        """The step's tokens on the device: the first maximum, or the sampler's draw."""
+        if sampler is None:
+            return K.argmax(logits)
+        n = logits.shape[0]
+        return sampler.sample(logits, list(range(n)), [step] * n, None)
 
     def decode_run(batch, steps, warmup):
         """Prompts in one step, then greedy single-token steps: `warmup` untimed, `steps` timed."""
         slots = [eng.alloc_slot() for _ in range(batch)]
         prompts = [rng.integers(0, cfg["vocab_size"], size=args.prompt_len).tolist() for _ in range(batch)]
         logits = eng.step(list(zip(slots, prompts)), want="last")
-        ids = K.argmax(logits)
+        ids = pick(logits, 0)
         rows = list(range(batch))
         placeholders = [(s, [0]) for s in slots]
+        done = [0]
 
         def run(n):
             """Greedy single-token steps as the generation loop runs them: a step takes its
@@ -121,7 +139,8 @@ def main(argv=None) -> int:
             for _ in range(n):
                 tokens = fetch_tokens(ids)
                 logits = eng.step(placeholders, want="last", device_ids=(ids, rows))
-                ids = K.argmax(logits)
+                done[0] += 1
+                ids = pick(logits, done[0])
                 tokens()
         run(warmup)
         torch.cuda.synchronize()
@@ -162,7 +181,7 @@ def main(argv=None) -> int:
                    "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
                    "intermediate": cfg["intermediate_size"], "vocab": cfg["vocab_size"],
                    "rope_theta": cfg["rope_theta"], "rope_scaling": f"llama3 x{cfg['rope_scaling']['factor']:g}" if cfg.get("rope_scaling") else "none", "rms_eps": cfg["rms_norm_eps"],
-                   "sampling": "greedy", "hip_graphs": eng.graphs is not None},
+                   "sampling": sampling, "hip_graphs": eng.graphs is not None},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4)},
     }

@@ -50,5 +50,25 @@ class Sampler:
                                 p.presence_penalty, p.temperature, p.penalize_newline, banned)
         if p.temperature == 0:
             return K.argmax(work)
-        u = torch.tensor(self.uniforms(requests, indices), dtype=torch.float32, device=logits.device)
+        u = self._to_device(self.uniforms(requests, indices), logits.device)
         return K.sample_pipeline(work, u, p.top_k, p.top_p, p.min_p, p.typical_p, p.min_keep)
+
+    def _to_device(self, us: Sequence[float], device) -> torch.Tensor:
+        """The step's uniform numbers on the device without the host waiting for the work already
+        queued there (a copy from ordinary host memory would): through one of a few pinned
+        staging buffers, each free again once its last copy has run."""
+        n = len(us)
+        ring = getattr(self, "_staging", None)
+        if ring is None or ring[0][0].numel() < n:
+            size = max(64, 2 * n)
+            ring = self._staging = [(torch.empty(size, dtype=torch.float32, pin_memory=True), torch.cuda.Event())
+                                    for _ in range(4)]
+            self._staging_next = 0
+        host, copied = ring[self._staging_next]
+        self._staging_next = (self._staging_next + 1) % len(ring)
+        copied.synchronize()
+        host[:n] = torch.tensor(us, dtype=torch.float32)
+        dev = torch.empty(n, dtype=torch.float32, device=device)
+        dev.copy_(host[:n], non_blocking=True)
+        copied.record()
+        return dev
