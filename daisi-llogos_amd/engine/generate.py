@@ -96,7 +96,7 @@ class Generator:
         try:
             if params.max_tokens == 0:
                 return
-            if self.look_ahead and getattr(eng, "takes_device_ids", False) and not params.has_penalties:
+            if self.look_ahead and getattr(eng, "takes_device_ids", False):
                 self._decode_ahead(batch, slots, prompts, params, sampler, stops, result, on_token)
             else:
                 self._decode_in_step(batch, slots, prompts, params, sampler, stops, result, on_token)
@@ -105,8 +105,8 @@ class Generator:
                 eng.free_slot(slots.pop(r))
 
     def _decode_in_step(self, batch, slots, prompts, params, sampler, stops, result, on_token) -> None:
-        """Every step waits for its tokens on the host before the next one starts (needed when
-        the sampler wants each row's token history for penalties)."""
+        """Every step waits for its tokens on the host before the next one starts (engines that
+        take their tokens from the host only)."""
         eng = self.engine
         live = list(batch)
         need_history = params.has_penalties
@@ -151,17 +151,22 @@ class Generator:
         """The same loop with the host one step behind the device: step t + 1 takes its tokens
         from the device memory that step t's sampler wrote and is started before the host has
         seen them, so the host's work per step (bookkeeping, page tables, the launch) runs while
-        the device computes.  The host reads step t's tokens while step t + 1 runs.  A request
-        whose token turns out to be a stop token has then run one step too many: its result is
-        dropped, and its slot is given back as usual (later work on the device comes after that
-        step in stream order).  Requests never take more steps than their share of the cache
-        allows: one that has its last permitted token coming is not stepped ahead."""
+        the device computes.  The host reads step t's tokens while step t + 1 runs, and only then
+        queues step t + 1's sampler, which can so be given every row's tokens up to t (penalties
+        look at them).  A request whose token turns out to be a stop token has then run one step
+        too many: its result is dropped, and its slot is given back as usual (later work on the
+        device comes after that step in stream order).  Requests never take more steps than
+        their share of the cache allows: one that has its last permitted token coming is not
+        stepped ahead."""
         eng = self.engine
         live = list(batch)
+        need_history = params.has_penalties
+        history = (lambda rs: [recent_tokens(prompts[r], result.tokens[r], params.penalty_count) for r in rs]) \
+            if need_history else (lambda rs: None)
         self._sync()
         t0 = time.perf_counter()
         logits = eng.step([(slots[r], prompts[r]) for r in live], want="last")
-        ids = sampler.sample(logits, live, [0] * len(live), None)
+        ids = sampler.sample(logits, live, [0] * len(live), history(live))
         # rows: (request, its row in ids); fetch: the tokens on their way to the host
         rows, fetch = [(r, i) for i, r in enumerate(live)], fetch_tokens(ids)
         fetch_first = fetch
@@ -170,13 +175,10 @@ class Generator:
         while rows:
             # requests that go on if their pending token is no stop token: step them now
             ahead = [(r, i) for r, i in rows if len(result.tokens[r]) + 1 < params.max_tokens]
-            nxt_ids = nxt_fetch = None
+            logits = None
             if ahead:
                 logits = eng.step([(slots[r], [0]) for r, _ in ahead], want="last",
                                   device_ids=(ids, [i for _, i in ahead]))
-                nxt_ids = sampler.sample(logits, [r for r, _ in ahead],
-                                         [len(result.tokens[r]) + 1 for r, _ in ahead], None)
-                nxt_fetch = fetch_tokens(nxt_ids)
             toks = fetch()
             if t1 is None and fetch is fetch_first:                       # the prompt step has ended
                 t1 = time.perf_counter()
@@ -185,17 +187,36 @@ class Generator:
             for r, i in rows:
                 if self._take_token(r, int(toks[i]), slots, params, stops, result, on_token):
                     went_on.add(r)
+            ids = fetch = None
+            if ahead and went_on:
+                # (the rows of requests that have just ended are drawn too, and dropped)
+                stepped = [r for r, _ in ahead]
+                ids = sampler.sample(logits, stepped, [len(result.tokens[r]) for r in stepped], history(stepped))
+                fetch = fetch_tokens(ids)
             rows = [(r, j) for j, (r, _) in enumerate(ahead) if r in went_on]
-            ids, fetch = nxt_ids, nxt_fetch
         self._sync()
         result.decode_seconds += time.perf_counter() - (t1 if t1 is not None else t0)
 
     @staticmethod
     def _sample(sampler, logits, live, prompts, result, need_history) -> List[int]:
         indices = [len(result.tokens[r]) for r in live]
-        histories = [prompts[r] + result.tokens[r] for r in live] if need_history else None
+        histories = None
+        if need_history:
+            count = getattr(sampler, "params", None)
+            count = count.penalty_count if count is not None else 0
+            histories = [recent_tokens(prompts[r], result.tokens[r], count) for r in live]
         ids = sampler.sample(logits, live, indices, histories)
         return [int(t) for t in (ids.tolist() if hasattr(ids, "tolist") else ids)]
+
+
+def recent_tokens(prompt: List[int], generated: List[int], count: int) -> List[int]:
+    """The last `count` tokens of prompt + generated (all of them for count <= 0) without
+    joining the two lists whole at every step."""
+    if count <= 0:
+        return prompt + generated
+    if len(generated) >= count:
+        return generated[-count:]
+    return prompt[max(0, len(prompt) - (count - len(generated))):] + generated
 
 
 def fetch_tokens(ids):

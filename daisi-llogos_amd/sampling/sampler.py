@@ -34,7 +34,7 @@ class Sampler:
         p = self.params
         if p.is_greedy:
             return K.argmax(logits)
-        hist = hist_len = None
+        arrays = []
         if p.has_penalties:
             if histories is None:
                 raise ValueError("penalties need each row's token history")
@@ -43,32 +43,45 @@ class Sampler:
             arr = np.zeros((len(win), width), dtype=np.int32)
             for i, w in enumerate(win):
                 arr[i, :len(w)] = w
-            hist = torch.from_numpy(arr).to(logits.device)
-            hist_len = torch.tensor([len(w) for w in win], dtype=torch.int32, device=logits.device)
+            arrays = [arr, np.asarray([len(w) for w in win], dtype=np.int32)]
+        if p.temperature > 0:
+            arrays.append(np.asarray(self.uniforms(requests, indices), dtype=np.float32))
+        staged = self._to_device(arrays, logits.device)
+        hist, hist_len = (staged[0], staged[1]) if p.has_penalties else (None, None)
         banned = self.stop_tokens[:8] if p.prevent_eos else ()
         work = K.sample_prepare(logits, hist, hist_len, p.repetition_penalty, p.frequency_penalty,
                                 p.presence_penalty, p.temperature, p.penalize_newline, banned)
         if p.temperature == 0:
             return K.argmax(work)
-        u = self._to_device(self.uniforms(requests, indices), logits.device)
-        return K.sample_pipeline(work, u, p.top_k, p.top_p, p.min_p, p.typical_p, p.min_keep)
+        return K.sample_pipeline(work, staged[-1], p.top_k, p.top_p, p.min_p, p.typical_p, p.min_keep)
 
-    def _to_device(self, us: Sequence[float], device) -> torch.Tensor:
-        """The step's uniform numbers on the device without the host waiting for the work already
-        queued there (a copy from ordinary host memory would): through one of a few pinned
-        staging buffers, each free again once its last copy has run."""
-        n = len(us)
+    def _to_device(self, arrays, device) -> List[torch.Tensor]:
+        """The step's small host arrays (int32 or float32) on the device with one copy, without
+        the host waiting for the work already queued there (a copy from ordinary host memory
+        would): through one of a few pinned staging buffers, each free again once its last copy
+        has run."""
+        if not arrays:
+            return []
+        n = sum(a.size for a in arrays)
         ring = getattr(self, "_staging", None)
         if ring is None or ring[0][0].numel() < n:
-            size = max(64, 2 * n)
-            ring = self._staging = [(torch.empty(size, dtype=torch.float32, pin_memory=True), torch.cuda.Event())
-                                    for _ in range(4)]
+            ring = self._staging = [(torch.empty(max(1024, 2 * n), dtype=torch.int32, pin_memory=True),
+                                     torch.cuda.Event()) for _ in range(4)]
             self._staging_next = 0
         host, copied = ring[self._staging_next]
         self._staging_next = (self._staging_next + 1) % len(ring)
         copied.synchronize()
-        host[:n] = torch.tensor(us, dtype=torch.float32)
-        dev = torch.empty(n, dtype=torch.float32, device=device)
+        flat = host.numpy()
+        o = 0
+        for a in arrays:
+            flat[o:o + a.size] = a.reshape(-1).view(np.int32)          # float32 goes as its bits
+            o += a.size
+        dev = torch.empty(n, dtype=torch.int32, device=device)
         dev.copy_(host[:n], non_blocking=True)
         copied.record()
-        return dev
+        out, o = [], 0
+        for a in arrays:
+            t = dev[o:o + a.size]
+            out.append((t.view(torch.float32) if a.dtype == np.float32 else t).view(a.shape))
+            o += a.size
+        return out

@@ -200,3 +200,10 @@ def test_looking_ahead_changes_no_result(max_tokens):
         n = len(toks)
         want_single += n - 1 if why == "length" else n + (1 if n + 1 < max_tokens else 0)
     assert single == want_single
+
+
+def test_recent_tokens_are_the_tail_of_prompt_and_generated():
+    for prompt, generated, count in (([1, 2, 3], [4, 5], 2), ([1, 2, 3], [4, 5], 4), ([1, 2, 3], [4, 5], 10),
+                                     ([1, 2, 3], [], 0), ([], [7], 3), ([1, 2, 3], [4, 5], 5), ([1, 2, 3], [4, 5], -1)):
+        whole = prompt + generated
+        assert gen.recent_tokens(prompt, generated, count) == (whole[-count:] if count > 0 else whole)
