@@ -167,7 +167,8 @@ LLOGOS_EXPORT int llogos_sample_prepare(float* work, const float* logits, int R,
 // ---------------------------------------------------------------- the candidate pipeline
 // Order-preserving map of a float onto an unsigned integer (larger float, larger integer).
 __device__ __forceinline__ uint32_t ordered_bits(float f) {
-    const uint32_t u = __float_as_uint(f);
+    uint32_t u = __float_as_uint(f);
+    if (u == 0x80000000u) u = 0;          // -0 equals +0: the lower id decides between them, as between other equals
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 // ascending sort of these puts the larger value first and, among equals, the lower id

@@ -268,3 +268,16 @@ def test_candidates_far_below_the_largest():
         head, whole, single = _every_way(rows, us, repetition_penalty=1.0, **opts)
         p = S.GenerationParams(repetition_penalty=1.0, **opts)
         assert head == whole == single == _plain(row, p, us), opts
+
+
+def test_zeros_of_either_sign_are_equal_logits():
+    """-0.0 and +0.0 compare equal, so among them the lower id comes first, as among other equal
+    logits (rounded or penalised logits can hold both)."""
+    row = np.array([0.0, -0.0, 0.0, -0.0, -0.0, 0.0, -3.0, 1.0] * 40, np.float32)
+    us = [0.02, 0.2, 0.4, 0.6, 0.8, 0.97]
+    rows = torch.tensor(np.tile(row, (len(us), 1)), device=DEV)
+    for opts in (dict(temperature=1.5, top_k=0, top_p=1.0), dict(temperature=1.0, top_k=100, top_p=0.9),
+                 dict(temperature=0.7, top_k=0, top_p=0.8, min_p=0.2)):
+        head, whole, single = _every_way(rows, us, repetition_penalty=1.0, **opts)
+        p = S.GenerationParams(repetition_penalty=1.0, **opts)
+        assert head == whole == single == _plain(row, p, us), opts
