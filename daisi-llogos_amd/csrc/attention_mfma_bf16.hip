@@ -534,8 +534,14 @@ __device__ __forceinline__ int direct_v_swizzle(int row) {                // row
     return 2 * ((row >> 1) & 3);
 }
 
-template <int HD>
-__global__ __launch_bounds__(kAttnWaves * kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
+// HALVES = 2: a block of 8 waves, two sets of 4 with page buffers of their own, takes the same
+// 128 rows; the sets take the tile's pages in turn and add their results through LDS at the end.
+// One such block fills a compute unit (two waves a SIMD, as two blocks of 4 do), and a tile's
+// pages take half as long: with HALVES = 1 a block left alone on its unit goes no faster (one
+// wave a SIMD cannot overlap its matrix and its vector instructions), so a prompt of few tiles
+// took as long as the pages of its last tile, one after the other.
+template <int HD, int HALVES>
+__global__ __launch_bounds__(HALVES * kAttnWaves * kWave) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attn_prefill_direct_kernel(
         bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int q_stride,
         const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
@@ -543,7 +549,8 @@ void attn_prefill_direct_kernel(
         const int* __restrict__ tok_pos, int batch, int n_tiles, int n_heads, int n_kv_heads, int group,
         float scale, int window, int sinks) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    DirectPageLds<HD>* lds = reinterpret_cast<DirectPageLds<HD>*>(smem_raw);   // two buffers
+    const int set = HALVES == 2 ? __builtin_amdgcn_readfirstlane(threadIdx.x / (kAttnWaves * kWave)) : 0;
+    DirectPageLds<HD>* lds = reinterpret_cast<DirectPageLds<HD>*>(smem_raw) + 2 * set;   // two buffers a set
     // Blocks start in the order of their index, round-robin over the 8 XCDs.  Block L is the
     // m-th block of XCD x (L = 8 m + x); an XCD takes the `group` query heads of one (tile, kv
     // head) pair one after the other, so that the pair's pages stay in its L2, and the pairs go
@@ -554,7 +561,7 @@ void attn_prefill_direct_kernel(
     // then, so that the longest block shares with the shortest.
     int m_xcd = blockIdx.x / 8;
     const int xcd = blockIdx.x % 8, per_xcd = gridDim.x / 8;
-    if (per_xcd > 32 && per_xcd <= 64 && m_xcd >= 32) m_xcd = per_xcd - 1 - (m_xcd - 32);
+    if (HALVES == 1 && per_xcd > 32 && per_xcd <= 64 && m_xcd >= 32) m_xcd = per_xcd - 1 - (m_xcd - 32);
     const int pair = (m_xcd / group) * 8 + xcd;
     if (pair >= n_tiles * n_kv_heads) return;
     const int kvh = pair % n_kv_heads, h = kvh * group + m_xcd % group;
@@ -567,7 +574,7 @@ void attn_prefill_direct_kernel(
     }
     if (b >= batch) return;
     const int lane = threadIdx.x & (kWave - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave) % kAttnWaves;   // within its set
     const int c = lane & 15, g = lane >> 4;
     const int seq_end = cu[b + 1];
     const int tile_rows = min(kTileRows, seq_end - first);
@@ -629,39 +636,46 @@ void attn_prefill_direct_kernel(
     };
     // The values of tokens that have not been written may be anything, also NaN, and 0 * NaN is
     // NaN: in the one page of a sequence that is not full they are zeroed in LDS after the copy.
+    // Every lane does so with the pieces it copied itself, once they have arrived and before the
+    // block's barrier (one barrier a page, whatever the page: the two sets of HALVES = 2 are at
+    // different pages and must meet the same barriers).
     auto zero_unwritten = [&](DirectPageLds<HD>& pg, int valid_keys) {
-        const int row = threadIdx.x >> 1, half = threadIdx.x & 1;          // a row's 8 pieces to two threads
-        if (row >= HD) return;
 #pragma unroll
-        for (int pp = 0; pp < 4; ++pp) {
-            const int piece = 4 * half + pp, keep = valid_keys - 8 * piece;
+        for (int j = 0; j < HD / 8 / kAttnWaves; ++j) {
+            const int vrow = 8 * (kAttnWaves * j + wave) + (lane >> 3);
+            const int keep = valid_keys - 8 * ((lane & 7) ^ direct_v_swizzle(vrow));   // of the tokens this piece holds
             if (keep >= 8) continue;
-            uint4* at = reinterpret_cast<uint4*>(&pg.v[row][8 * (piece ^ direct_v_swizzle(row))]);
+            uint4* at = reinterpret_cast<uint4*>(&pg.v[vrow][8 * (lane & 7)]);
             *at = __builtin_bit_cast(uint4, keep_first(__builtin_bit_cast(bf16x8, *at), keep));
         }
     };
     auto land = [&](int pi, DirectPageLds<HD>& pg) {                        // the copy of page pi is complete and visible
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
         const int valid_keys = written - pi * kPageTokens;
-        if (pi < n_pages && valid_keys < kPageTokens) {
-            zero_unwritten(pg, valid_keys);
-            __syncthreads();
-        }
+        if (pi < n_pages && valid_keys < kPageTokens) zero_unwritten(pg, valid_keys);
+        __syncthreads();
     };
-    int cur = next_needed(-1);
-    if (cur >= n_pages) return;                                          // cannot happen: a row sees itself
-    int nxt = next_needed(cur);
+    // The pages that are needed go to the sets in turn.  `lead` is the first set's page: every
+    // wave follows it, so that both sets go round the loop, and through its barriers, equally often.
+    auto advance = [&](int pi) {
+        pi = next_needed(pi);
+        return HALVES == 2 ? next_needed(pi) : pi;
+    };
+    int lead = next_needed(-1);
+    if (lead >= n_pages) return;                                         // cannot happen: a row sees itself
+    int cur = set ? next_needed(lead) : lead;
+    int nxt = advance(cur);
     int nxt_id = nxt < n_pages ? page_id(nxt) : 0;
-    copy_page(page_id(cur), lds[0]);
+    if (cur < n_pages) copy_page(page_id(cur), lds[0]);
     land(cur, lds[0]);
     int buf = 0;
-    while (cur < n_pages) {
-        const int nxt2 = next_needed(nxt);
+    while (lead < n_pages) {
+        const int nxt2 = advance(nxt);
         if (nxt < n_pages) copy_page(nxt_id, lds[buf ^ 1]);
         const int nxt2_id = nxt2 < n_pages ? page_id(nxt2) : 0;
         do {
         const int key0 = cur * kPageTokens;
+        if (cur >= n_pages) break;                                        // the second set, after an odd number of pages
         if (wave_rows <= 0 || key0 > wave_last_pos) break;                // nothing of this page for this wave
         if (!page_may_be_visible_to_range(wave_first_pos, wave_last_pos, key0, window, sinks)) break;
         const DirectPageLds<HD>& pg = lds[buf];
@@ -729,6 +743,42 @@ void attn_prefill_direct_kernel(
         nxt = nxt2;
         nxt_id = nxt2_id;
         buf ^= 1;
+        lead = advance(lead);
+    }
+    if (HALVES == 2) {
+        // The second set's running maxima, sums and outputs go through LDS (lane by lane: the two
+        // sets hold the same rows in the same lanes) and are added to the first set's.  The loop's
+        // last barrier came after the last read of a page.
+        constexpr int kStateFloats = 2 + HD / 4;
+        float* state = reinterpret_cast<float*>(smem_raw) + (size_t)wave * (2 * kStateFloats * kWave) + lane;
+        auto put = [&](const WaveState<HD>& st, float* at) {
+            at[0] = st.m;
+            at[kWave] = st.l;
+#pragma unroll
+            for (int db = 0; db < HD / 16; ++db)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) at[(2 + 4 * db + r) * kWave] = st.acc[db][r];
+        };
+        auto add = [&](WaveState<HD>& st, const float* at) {
+            const float m_other = at[0], l_other = at[kWave];
+            const float m = fmaxf(st.m, m_other);
+            const float mine = st.m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(st.m - m);
+            const float theirs = m_other == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_other - m);
+            st.l = st.l * mine + l_other * theirs;
+            st.m = m;
+#pragma unroll
+            for (int db = 0; db < HD / 16; ++db)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) st.acc[db][r] = st.acc[db][r] * mine + at[(2 + 4 * db + r) * kWave] * theirs;
+        };
+        if (set == 1) {
+            put(st0, state);
+            put(st1, state + kStateFloats * kWave);
+        }
+        __syncthreads();
+        if (set == 1) return;
+        add(st0, state);
+        add(st1, state + kStateFloats * kWave);
     }
     auto write_out = [&](const WaveState<HD>& st, int rr) {
         if (rr >= wave_rows) return;
@@ -841,8 +891,8 @@ LLOGOS_EXPORT int llogos_attn_prefill_bf16(void* out, const void* q, int q_strid
                                            const void* v_pool, const int* table, int table_stride,
                                            const int* cu, const int* tok_pos, int batch, int n_tiles, int tile_rows,
                                            int n_heads, int n_kv_heads, int head_dim,
-                                           float scale, int window, int sinks, hipStream_t stream) {
-    if (batch <= 0 || n_tiles <= 0 || window < 0 || sinks < 0) return LLOGOS_BAD_ARGUMENT;
+                                           float scale, int window, int sinks, int halves, hipStream_t stream) {
+    if (batch <= 0 || n_tiles <= 0 || window < 0 || sinks < 0 || (halves != 1 && halves != 2)) return LLOGOS_BAD_ARGUMENT;
     if (tile_rows != 64 && tile_rows != kTileRows) return LLOGOS_BAD_ARGUMENT;
     if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || (q_stride % 8) || ((uintptr_t)q % 16)) return LLOGOS_UNSUPPORTED;
     const int group = n_heads / n_kv_heads;
@@ -850,16 +900,17 @@ LLOGOS_EXPORT int llogos_attn_prefill_bf16(void* out, const void* q, int q_strid
     if (tile_rows == kTileRows) {
         const long long pairs = (long long)n_tiles * n_kv_heads;
         const dim3 lgrid((unsigned)((pairs + 7) / 8 * 8 * group));
-#define GOD(HD) do { \
-        const size_t smem = 2 * sizeof(DirectPageLds<HD>); \
-        hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_direct_kernel<HD>, \
+#define GOD(HD, HALVES) do { \
+        const size_t smem = HALVES * 2 * sizeof(DirectPageLds<HD>); \
+        hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_direct_kernel<HD, HALVES>, \
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); \
         if (e != hipSuccess) return (int)e; \
-        attn_prefill_direct_kernel<HD><<<lgrid, kAttnWaves * kWave, smem, stream>>>( \
+        attn_prefill_direct_kernel<HD, HALVES><<<lgrid, HALVES * kAttnWaves * kWave, smem, stream>>>( \
             (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_stride, \
             cu, tok_pos, batch, n_tiles, n_heads, n_kv_heads, group, scale, window, sinks); \
         return LLOGOS_LAUNCH_CHECK(); } while (0)
-        if (head_dim == 64) GOD(64); else GOD(128);
+        if (halves == 2) { if (head_dim == 64) GOD(64, 2); else GOD(128, 2); }
+        if (head_dim == 64) GOD(64, 1); else GOD(128, 1);
 #undef GOD
     }
 #define GO(HD) attn_prefill_kernel<HD><<<grid, kAttnWaves * kWave, 0, stream>>>( \

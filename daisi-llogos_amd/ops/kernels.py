@@ -613,6 +613,24 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dty
 
 _attn_workspaces = {}
 PREFILL_TILE_ROWS = 0        # 0: chosen by the step; 64 or 128 force a prefill attention kernel (tests)
+PREFILL_HALVES = 0           # 0: chosen by the step; 1 or 2 sets of waves a block of the 128-row kernel (tests)
+
+
+def prefill_halves(lens: Sequence[int], starts: Optional[Sequence[int]], n_heads: int, n_cus: int = 256) -> int:
+    """Sets of waves a block of the 128-row prompt attention: 2 (the sets take a tile's pages in
+    turn) where the pages of the longest tile, one after the other, take longer than the chip
+    needs for all tiles; 1 (two independent blocks a compute unit, 15 % more throughput) where
+    the work of all tiles decides.  Measured at the 8B head shape: two sets win up to 2,048
+    tokens of one prompt (1,536: 45 us against 57) and lose from 2,560 on and for many short
+    prompts."""
+    longest = total = 0
+    for i, n in enumerate(lens):
+        start = starts[i] if starts else 0
+        for t in range(0, n, 128):
+            pages = (start + min(n, t + 128) + PAGE_TOKENS - 1) // PAGE_TOKENS
+            longest = max(longest, pages)
+            total += pages
+    return 2 if longest * 2 * n_cus > 1.7 * total * n_heads else 1
 
 
 def _attn_workspace(device: torch.device, floats: int) -> torch.Tensor:
@@ -661,10 +679,11 @@ def attention_mfma_bf16(ctx, q: torch.Tensor, q_stride: int, k_pool: torch.Tenso
         lens = [ctx.cu_seqlens[i + 1] - ctx.cu_seqlens[i] for i in range(ctx.batch)]
         tile_rows = PREFILL_TILE_ROWS or (128 if max(lens) > 64 else 64)
         n_tiles = sum(-(-n // tile_rows) for n in lens)
+        halves = PREFILL_HALVES or (prefill_halves(lens, getattr(ctx, "starts", None), n_heads) if tile_rows == 128 else 1)
         code = lib.llogos_attn_prefill_bf16(
             _p(out), _p(q), q_stride, _p(k_pool), _p(v_pool), _p(table), table.stride(0), _p(cu), _p(ctx.tok_pos),
             ctx.batch, n_tiles, tile_rows, n_heads, n_kv_heads, head_dim, ctypes.c_float(scale), window, sinks,
-            _stream())
+            halves, _stream())
     if code == -2:
         return None
     _check(code, "attention_mfma_bf16")

@@ -405,15 +405,17 @@ def test_attention_of_random_shapes(dtype):
         assert err <= RT[dtype] * max(1.0, np.abs(want).max()), (case, nh, nkv, hd, lens, new, window, sinks, err)
 
 
-@pytest.mark.parametrize("tile_rows", [64, 128])
+@pytest.mark.parametrize("tile_rows,halves", [(64, 1), (128, 1), (128, 2)])
 @pytest.mark.parametrize("nh,nkv,hd", [(6, 2, 64), (8, 2, 128), (3, 3, 128)])
 @pytest.mark.parametrize("window,sinks", [(0, 0), (100, 0), (70, 5)])
-def test_prompt_attention_on_the_matrix_cores(tile_rows, nh, nkv, hd, window, sinks):
-    """Both prompt kernels (pages read by each wave; pages shared through LDS) on long and
-    short sequences, whole and continued, with pages half written."""
-    K.PREFILL_TILE_ROWS = tile_rows
+def test_prompt_attention_on_the_matrix_cores(tile_rows, halves, nh, nkv, hd, window, sinks):
+    """The prompt kernels (pages read by each wave; pages shared through LDS by one set of waves
+    or by two that take the pages in turn) on long and short sequences, whole and continued,
+    with pages half written, and with odd and even numbers of pages a tile."""
+    K.PREFILL_TILE_ROWS, K.PREFILL_HALVES = tile_rows, halves
     try:
-        for lens, new in (([300, 129, 5, 64], [300, 129, 5, 64]), ([400, 90, 257], [200, 33, 129])):
+        for lens, new in (([300, 129, 5, 64], [300, 129, 5, 64]), ([400, 90, 257], [200, 33, 129]),
+                          ([1100, 700], [1100, 190])):
             c = _attention_case("bfloat16", nh, nkv, hd, lens, new, seed=11)
             ctx = type("Ctx", (), dict(tok_seq=_t(c["tok_seq"], torch.int32), tok_pos=_t(c["tok_pos"], torch.int32),
                                        is_decode=False, max_context=max(lens), batch=len(lens), n_tokens=sum(new),
@@ -431,7 +433,7 @@ def test_prompt_attention_on_the_matrix_cores(tile_rows, nh, nkv, hd, window, si
             assert out is not None
             _close(out, _plain_attention(c, nh, nkv, hd, window, sinks), "bfloat16")
     finally:
-        K.PREFILL_TILE_ROWS = 0
+        K.PREFILL_TILE_ROWS = K.PREFILL_HALVES = 0
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -63,3 +63,13 @@ def test_known_choices():
     # ... and not where the LDS few-row product's own blocks fill one round well, or the matrix is small
     assert K.skinny_plan(64, 28672, 4096)[0] == "lds" and K.skinny_plan(32, 28672, 4096)[0] == "lds"
     assert K.skinny_plan(64, 16384, 3072)[0] == "lds" and K.skinny_plan(64, 19456, 2560)[0] == "lds"
+
+
+def test_sets_of_waves_of_the_prompt_attention():
+    """Two sets of waves a block where one prompt's last tile would set the time, one where the
+    work of all tiles does (the measured cases at 32 heads)."""
+    for lens, want in (([512], 2), ([1536], 2), ([2048], 2), ([2560], 1), ([4096], 1), ([16384], 1),
+                       ([1024] * 2, 2), ([512] * 4, 1), ([256] * 4, 2), ([512] * 8, 1)):
+        assert K.prefill_halves(lens, None, 32) == want, lens
+    # a continued prompt counts the pages before it
+    assert K.prefill_halves([128], [4000], 32) == 2 and K.prefill_halves([128] * 64, [4000] * 64, 32) == 1
