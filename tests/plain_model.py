@@ -65,24 +65,22 @@ def rope_frequencies(rot_dim: int, theta: float) -> np.ndarray:
 
 def llama3_frequency_factors(freqs: np.ndarray, factor: float, low_freq_factor: float,
                              high_freq_factor: float, original_max_position: int) -> np.ndarray:
-    """Per-pair divisors in the manner of the reference's frequency-factor table
-    (f_i <- f_i / factor_i, Daisi.Llogos.Cpu/Rope.cs:42-63).  The Llama-3 rule for the
-    table is not in the reference; it is written from the rule's definition: pairs with
-    a wavelength below original/high keep their frequency, those above original/low
-    are slowed by `factor`, and the band between is interpolated in 1/factor."""
-    out = np.ones_like(freqs)
-    low_wavelen = original_max_position / low_freq_factor
-    high_wavelen = original_max_position / high_freq_factor
-    for i, f in enumerate(freqs):
-        wavelen = 2.0 * math.pi / f
-        if wavelen < high_wavelen:
-            out[i] = 1.0
-        elif wavelen > low_wavelen:
-            out[i] = factor
-        else:
-            smooth = (original_max_position / wavelen - low_freq_factor) / (high_freq_factor - low_freq_factor)
-            out[i] = 1.0 / ((1.0 - smooth) / factor + smooth)
-    return out
+    """Per-pair divisors for the reference's frequency-factor table (the effective frequency is
+    f_i / factor_i, Daisi.Llogos.Cpu/Rope.cs:42-63; the reference takes the table from the
+    checkpoint, here the Llama-3 rule fills it from the configuration).
+
+    The rule, stated by how often a pair turns within the original context, r_i =
+    original * f_i / (2 pi): pairs that turn more than `high` times keep their frequency;
+    pairs that turn less than `low` times run `factor` times slower; between the two the new
+    frequency is a mix of the slowed and the kept one, f_i * ((1 - s) / factor + s), with
+    s = (r_i - low) / (high - low) going from 0 to 1 across the band.  The mix is linear in the
+    *frequency* (that is in 1 / factor), not in the divisor."""
+    f = np.asarray(freqs, dtype=np.float64)
+    turns = float(original_max_position) * f / (2.0 * math.pi)
+    s = np.clip((turns - low_freq_factor) / (high_freq_factor - low_freq_factor), 0.0, 1.0)
+    kept_share = np.where(turns > high_freq_factor, 1.0, np.where(turns < low_freq_factor, 0.0, s))
+    new_f = f * ((1.0 - kept_share) / float(factor) + kept_share)
+    return f / new_f
 
 
 def rope_split_half(x: np.ndarray, positions, n_heads: int, head_dim: int, freqs: np.ndarray) -> np.ndarray:

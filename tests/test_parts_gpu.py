@@ -21,7 +21,7 @@ P = importlib.import_module("daisi-llogos_amd.parts")
 K = importlib.import_module("daisi-llogos_amd.ops.kernels")
 DEV = torch.device("cuda:0")
 DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
-TOL = {"float32": 2e-5, "bfloat16": 3e-2}
+TOL = {"float32": 2e-5, "bfloat16": 1e-2}
 
 
 def _np(t):
@@ -310,7 +310,7 @@ def test_a_layer_twice_and_a_layer_reading_anothers_cache(tmp_path, dtype):
     assert len(eng.cache.groups) == 1 and eng.cache.groups[0].k.shape[0] == 3      # three caches for four runs
     s = eng.alloc_slot()
     rows = [_np(eng.step([(s, toks[:66])], want="all"))] + [_np(eng.step([(s, [t])])) for t in toks[66:]]
-    H.close(np.concatenate(rows), want, dtype, "scheduled layers")
+    H.close(np.concatenate(rows), want, dtype, "scheduled layers", config="tiny_a")
     models = importlib.import_module("daisi-llogos_amd.models")
     spec = L.dense_decoder_spec(L.ARCHITECTURES["Qwen2ForCausalLM"].read_config(tc.TINY_A))
     spec.schedule = [models.ScheduleEntry(0), models.ScheduleEntry(1, cache_of=1)]

@@ -122,6 +122,50 @@ def test_llama3_factors():
     assert np.allclose(pm.llama3_frequency_factors(f, 1.0, 1.0, 4.0, 8192), 1.0)
 
 
+def test_llama3_band_mixes_frequencies_not_divisors():
+    """Numbers worked by hand.  original 8192, low 1, high 4, factor 8: a pair that turns 2.5
+    times in the original context is half way through the band, so its frequency becomes
+    f * (0.5 / 8 + 0.5) = 0.5625 f and its divisor 16 / 9.  Mixing the divisors (0.5 * 8 +
+    0.5 * 1 = 4.5), a band mixed the other way round (1 / (0.5 + 0.5 / 8) is the same at the
+    middle, so a second point at a quarter of the band separates that), or wavelength and
+    frequency taken for one another would all give other numbers."""
+    f_of = lambda turns: np.array([turns * 2.0 * math.pi / 8192.0])
+    assert pm.llama3_frequency_factors(f_of(2.5), 8.0, 1.0, 4.0, 8192)[0] == pytest.approx(16.0 / 9.0, rel=1e-12)
+    # a quarter of the way (1.75 turns): f * (0.75 / 8 + 0.25) = 0.34375 f -> divisor 32 / 11
+    assert pm.llama3_frequency_factors(f_of(1.75), 8.0, 1.0, 4.0, 8192)[0] == pytest.approx(32.0 / 11.0, rel=1e-12)
+    # the band's ends meet the flat parts: no jump
+    assert pm.llama3_frequency_factors(f_of(4.0), 8.0, 1.0, 4.0, 8192)[0] == pytest.approx(1.0, rel=1e-12)
+    assert pm.llama3_frequency_factors(f_of(1.0), 8.0, 1.0, 4.0, 8192)[0] == pytest.approx(8.0, rel=1e-12)
+    # other constants: original 64, low 2, high 6, factor 3; 3 turns are a quarter of the band:
+    # f * (0.75 / 3 + 0.25) = 0.5 f
+    f = np.array([3 * 2.0 * math.pi / 64.0])
+    assert pm.llama3_frequency_factors(f, 3.0, 2.0, 6.0, 64)[0] == pytest.approx(2.0, rel=1e-12)
+
+
+def test_per_head_norm_is_rms_norm_head_by_head_with_one_weight():
+    """Daisi.Llogos.Cpu/CpuBackend.cs:406-421: every head's head_dim values are normed on
+    their own, all heads with the same [head_dim] weight.  A norm over the whole row, a weight
+    per head, or eps taken per row would all fail one of these."""
+    rng = np.random.default_rng(5)
+    t, n_heads, hd, eps = 3, 4, 8, 1e-3
+    x = rng.standard_normal((t, n_heads * hd)) * np.repeat([0.01, 1.0, 30.0, 0.3], hd)   # heads of unlike size
+    w = rng.standard_normal(hd)
+    got = pm.per_head_rms_norm(x, w, n_heads, hd, eps)
+    for h in range(n_heads):
+        assert np.allclose(got[:, h * hd:(h + 1) * hd], pm.rms_norm(x[:, h * hd:(h + 1) * hd], w, eps), rtol=1e-13)
+    whole = pm.rms_norm(x, np.tile(w, n_heads), eps)
+    assert not np.allclose(got, whole, rtol=1e-2)
+    # eps counts per head: the small head is damped by it, the large ones are not
+    small = got[:, :hd] / w
+    assert np.all(np.abs((small * small).mean(-1) - 1.0) > 0.5)
+    big = got[:, 2 * hd:3 * hd] / w
+    assert np.allclose((big * big).mean(-1), 1.0, atol=1e-4)
+    # one head is the plain norm; one kv head (MQA) the same
+    assert np.allclose(pm.per_head_rms_norm(x[:, :hd], w, 1, hd, eps), pm.rms_norm(x[:, :hd], w, eps), rtol=1e-13)
+    # a row's result does not depend on the other rows
+    assert np.allclose(pm.per_head_rms_norm(x[1:2], w, n_heads, hd, eps), got[1:2], rtol=1e-13)
+
+
 def test_linear_scaling_stretches_positions():
     """rope_scaling 'linear' with factor s: position s * p of the scaled model is position p of
     the unscaled one; unknown kinds are refused."""

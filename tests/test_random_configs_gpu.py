@@ -58,16 +58,16 @@ def test_random_configuration(seed, dtype):
     eng = H.engine(name, dtype, max_tokens=64 * 12, n_slots=3)
     slots = [eng.alloc_slot() for _ in seqs]
     got = eng.step([(sl, s[:n]) for sl, s, n in zip(slots, seqs, lens)], want="all")
-    H.close(got.cpu().double().numpy(), np.concatenate([p[:n] for p, n in zip(plain, lens)]), dtype, f"{name}: prompts")
+    H.close(got.cpu().double().numpy(), np.concatenate([p[:n] for p, n in zip(plain, lens)]), dtype, f"{name}: prompts", config=name)
     live = [0, 1, 2]
     for t in range(4):
         if t == 2:                                      # the second sequence ends early; its slot takes a new prompt later
             eng.free_slot(slots[1])
             live = [0, 2]
         got = eng.step([(slots[i], [seqs[i][lens[i] + t]]) for i in live], want="last")
-        H.close(got.cpu().double().numpy(), np.stack([plain[i][lens[i] + t] for i in live]), dtype, f"{name}: token {t}")
+        H.close(got.cpu().double().numpy(), np.stack([plain[i][lens[i] + t] for i in live]), dtype, f"{name}: token {t}", config=name)
     # a continued prompt of two tokens beside a new prompt in the freed slot
     slots[1] = eng.alloc_slot()
     got = eng.step([(slots[0], seqs[0][lens[0] + 4:lens[0] + 6]), (slots[1], seqs[1][:lens[1]])], want=[[0, 1], [lens[1] - 1]])
     want = np.stack([plain[0][lens[0] + 4], plain[0][lens[0] + 5], plain[1][lens[1] - 1]])
-    H.close(got.cpu().double().numpy(), want, dtype, f"{name}: continued prompt beside a new one")
+    H.close(got.cpu().double().numpy(), want, dtype, f"{name}: continued prompt beside a new one", config=name)

@@ -44,10 +44,10 @@ def test_replay_of_two_batches(tmp_path, dtype):
     def read(step):
         return np.fromfile(os.path.join(out, f"{step}.f32"), dtype="<f4").reshape(-1, vocab)
     pa, pb, pc = H.plain_logits(name, a), H.plain_logits(name, b), H.plain_logits(name, c)
-    H.close(read(0), np.concatenate([pa[:66], pb[7:8]]), dtype, "step 0")
-    H.close(read(1), pa[66:67], dtype, "step 1")
-    H.close(read(3), pa[68:69], dtype, "step 3")
-    H.close(read(4), pc[[0, 39]], dtype, "step 4")
+    H.close(read(0), np.concatenate([pa[:66], pb[7:8]]), dtype, "step 0", config=name)
+    H.close(read(1), pa[66:67], dtype, "step 1", config=name)
+    H.close(read(3), pa[68:69], dtype, "step 3", config=name)
+    H.close(read(4), pc[[0, 39]], dtype, "step 4", config=name)
 
 
 @pytest.mark.parametrize("dtype", H.DTYPES)
@@ -103,11 +103,11 @@ def test_the_same_requests_whole_token_by_token_and_in_unequal_batches(tmp_path,
     steps.append({"step": n, "entries": [{"id": "c", "tokens": list(reqs["c"][:69]), "want": list(range(69))}], "end": []}); n += 1
     steps.append({"step": n, "entries": [{"id": "c", "tokens": [reqs["c"][69]], "want": [0]}], "end": ["c"]}); n += 1
     batched = replay(steps, 192, "batched")
-    tol = 2e-5 if dtype == "float32" else H.TOL[dtype]
+    tol = 2e-5 if dtype == "float32" else H.tol(dtype, name)
     for k in reqs:
         for way, got in (("whole", whole), ("token by token", single), ("batched", batched)):
             assert not np.isnan(got[k]).any(), (k, way)
-            H.close(got[k], plain[k], dtype, f"{name} {k} {way}")
+            H.close(got[k], plain[k], dtype, f"{name} {k} {way}", config=name)
         assert np.abs(whole[k] - single[k]).max() <= tol and np.abs(whole[k] - batched[k]).max() <= tol
 
 
