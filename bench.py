@@ -7,7 +7,13 @@ A step is one decode step of the whole batch.  The line printed at the end is th
 value = decoded tokens a second at the default batch of 8 (512-token random prompts, the
 context grows from there), "prefill" = one 2,048-token prompt, "roofline" = bytes the decode
 step has to read (every weight it uses once, the cache of the live requests) / its time
-against 8 TB/s, "points" = decoding at batch 1 and 64."""
+against 8 TB/s, "points" = decoding at batch 1 and 64.  Beside the published peaks the record
+holds what this GPU was measured to do at best in the same run ("measured_peak": a kernel that
+only reads the weights' bytes; v_mfma_f32_16x16x32_bf16 issued back to back) and the fractions
+of those; "generate_loop" is the same decode through the product's generation loop
+(Generator.generate: its batching, stop checks and bookkeeping inside the timed region).
+
+    python bench.py --ceilings      # the measured ceilings alone, at several buffer sizes"""
 import argparse
 import importlib
 import json
@@ -78,6 +84,7 @@ def main(argv=None) -> int:
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration has (0 = all)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
     ap.add_argument("--only-prefill", action="store_true", help="time the 2,048-token prompt alone (for profiling)")
+    ap.add_argument("--ceilings", action="store_true", help="measure the read bandwidth and the MFMA rate of this GPU and exit")
     ap.add_argument("--temperature", type=float, default=0.0, help="0 = greedy (the default run); above 0 the sampler draws")
     ap.add_argument("--top-k", type=int, default=40)
     ap.add_argument("--top-p", type=float, default=0.9)
@@ -92,6 +99,17 @@ def main(argv=None) -> int:
     llogos = importlib.import_module("daisi-llogos_amd")
     K = importlib.import_module("daisi-llogos_amd.ops.kernels")
     fetch_tokens = importlib.import_module("daisi-llogos_amd.engine.generate").fetch_tokens
+
+    if args.ceilings:
+        # the sizes are those of the 8B matrices a decode step streams: gate/up, down, qkv, o, and all weights of a layer
+        for label, n in (("gate/up 235 MB", 2 * 14336 * 4096 * 2), ("down 117 MB", 4096 * 14336 * 2), ("qkv 50 MB", 6144 * 4096 * 2),
+                         ("o 34 MB", 4096 * 4096 * 2), ("1 GiB", 1 << 30), ("4 GiB", 1 << 32)):
+            bw = K.measure_read_bandwidth(n)
+            print(f"[ceilings] read {label}: {bw / 1e12:.2f} TB/s ({bw / HBM_PEAK:.3f} of {HBM_PEAK / 1e12:g})", flush=True)
+        rate = K.measure_mfma_rate()
+        print(f"[ceilings] mfma 16x16x32 bf16: {rate / 1e15:.3f} PFLOP/s ({rate / MFMA_PEAK['bf16']:.3f} of "
+              f"{MFMA_PEAK['bf16'] / 1e15:g})", flush=True)
+        return 0
 
     model_name, cfg = MODELS[args.model]
     cfg = dict(cfg)
@@ -166,6 +184,11 @@ def main(argv=None) -> int:
             eng.free_slot(s)
         return 0
 
+    # what this GPU does at best: reading as many bytes as the model's weights, and the matrix cores' issue rate
+    read_peak = K.measure_read_bandwidth(min(weight_bytes(cfg), 4 << 30), repeats=5)
+    mfma_peak = K.measure_mfma_rate()
+    print(f"[bench] measured ceilings: read {read_peak / 1e12:.2f} TB/s, mfma bf16 {mfma_peak / 1e15:.3f} PFLOP/s",
+          file=sys.stderr, flush=True)
     dt, ctx_mid = decode_run(args.batch, args.steps, args.warmup)
     ms_per_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
@@ -183,11 +206,25 @@ def main(argv=None) -> int:
                    "rope_theta": cfg["rope_theta"], "rope_scaling": f"llama3 x{cfg['rope_scaling']['factor']:g}" if cfg.get("rope_scaling") else "none", "rms_eps": cfg["rms_norm_eps"],
                    "sampling": sampling, "hip_graphs": eng.graphs is not None},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK, 4)},
+                     "frac": round(achieved / HBM_PEAK, 4), "measured_peak": round(read_peak / 1e9, 1),
+                     "frac_of_measured": round(achieved / read_peak, 4)},
     }
     print(f"[bench] decode b{args.batch}: {value:.1f} tok/s, {ms_per_step:.3f} ms/step, "
           f"{achieved / 1e12:.2f} TB/s", file=sys.stderr, flush=True)
 
+    if not args.no_points and sampler is None:
+        # the same decode through the product's own loop: prompts in one step, then greedy tokens with
+        # the loop's batching, stop checks, slot bookkeeping and token fetches inside the timed region
+        S = importlib.import_module("daisi-llogos_amd.sampling")
+        generator = llogos.Generator(eng, max_batch=args.batch, synchronize=torch.cuda.synchronize)
+        prompts = [rng.integers(0, cfg["vocab_size"], size=args.prompt_len).tolist() for _ in range(args.batch)]
+        n_new = args.steps + args.warmup
+        res = generator.generate(prompts, S.GenerationParams.greedy(max_tokens=n_new, stop_tokens=()))
+        loop_steps = n_new - 1                                   # the first token comes from the prompt step
+        record["generate_loop"] = {"value": round(args.batch * loop_steps / res.decode_seconds, 1), "unit": "tok/s",
+                                   "ms_per_step": round(res.decode_seconds / loop_steps * 1e3, 4), "steps": loop_steps}
+        print(f"[bench] generation loop b{args.batch}: {record['generate_loop']['value']:.1f} tok/s, "
+              f"{record['generate_loop']['ms_per_step']:.3f} ms/step", file=sys.stderr, flush=True)
     if not args.no_points:
         points = {}
         for b in (1, 64):
@@ -210,7 +247,9 @@ def main(argv=None) -> int:
         pt = min(times[1:])
         flops = prefill_flops(cfg, prefill_tokens)
         record["prefill"] = {"value": round(prefill_tokens / pt, 1), "tokens": prefill_tokens, "ms": round(pt * 1e3, 3),
-                             "frac": round(flops / pt / MFMA_PEAK["bf16"], 4)}
+                             "frac": round(flops / pt / MFMA_PEAK["bf16"], 4),
+                             "measured_peak_tflops": round(mfma_peak / 1e12, 1),
+                             "frac_of_measured": round(flops / pt / mfma_peak, 4)}
         print(f"[bench] prefill {prefill_tokens}: {prefill_tokens / pt:.0f} tok/s, {pt * 1e3:.2f} ms", file=sys.stderr,
               flush=True)
     print(json.dumps(record), flush=True)

@@ -204,6 +204,11 @@ def main(argv=None) -> int:
               f"({r.decode_tokens_per_second:8.1f} tok/s)", file=sys.stderr)
         print(f"  Total:    {r.prompt_tokens + r.generated_tokens:6d} tokens in {total_ms:8.1f} ms", file=sys.stderr)
         print(f"  Load:     {load_ms:8.1f} ms", file=sys.stderr)
+        # against the MI355X's published peaks: the prompt step's flops, and the bytes the decode steps had to read
+        print(f"  Roofline: prefill {r.prefill_flops / max(r.prefill_seconds, 1e-12) / 1e12:7.1f} TFLOP/s "
+              f"({r.prefill_fraction_of_peak:.3f} of the {r.dtype} matrix peak)  "
+              f"decode {r.decode_bytes_per_second / 1e9:7.1f} GB/s ({r.decode_fraction_of_peak:.3f} of 8 TB/s)",
+              file=sys.stderr)
         return 0
 
     params = GenerationParams(max_tokens=args.max_tokens, temperature=args.temperature, top_k=args.top_k,

@@ -5,6 +5,7 @@ The reference's entry points are TextGenerator.Generate / Benchmark
 (Daisi.Llogos.Cli/Program.cs); option names and defaults follow them."""
 from __future__ import annotations
 
+import re
 import time
 from dataclasses import dataclass
 from typing import List, Optional, Sequence, Tuple, Union
@@ -17,26 +18,27 @@ from .engine.step import Engine
 from .sampling.params import GenerationParams
 
 
+_ATTENTION_FORMS = re.compile(r"^(?:(full)|window:(\d+)|sinks:(\d+),(\d+))$")
+
+
+HBM_PEAK_BYTES = 8.0e12                                                    # MI355X, bytes a second
+MFMA_PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}                       # dense, flops a second
+
+
 def parse_attention(value: str) -> Tuple[Optional[int], int]:
-    """'full', 'window:N' or 'sinks:S,W' (Daisi.Llogos/Inference/AttentionStrategy.cs:75-100)
-    -> (window or None for the configuration's own, sinks)."""
-    v = value.strip().lower()
-    if v == "full":
+    """The command line's --attention option: 'full' (the configuration's own attention),
+    'window:N' (the last N positions) or 'sinks:S,W' (the first S positions and the last W), the
+    reference's three strategies (Daisi.Llogos/Inference/AttentionStrategy.cs:75-100).
+    Returns (positions the cache keeps for a sequence, or None for 'full'; how many of them are sinks)."""
+    m = _ATTENTION_FORMS.match(value.strip().lower())
+    if m is None:
+        raise ValueError(f"--attention takes full, window:<N> or sinks:<S>,<W>, not '{value}'")
+    if m.group(1):
         return None, 0
-    if v.startswith("window:"):
-        n = int(v[7:])
-        if n <= 0:
-            raise ValueError("window size must be positive")
-        return n, 0
-    if v.startswith("sinks:"):
-        parts = v[6:].split(",")
-        if len(parts) != 2:
-            raise ValueError("sinks format: sinks:<sink_tokens>,<window_size>")
-        s, w = int(parts[0]), int(parts[1])
-        if s < 0 or w <= 0:
-            raise ValueError("sinks needs sink_tokens >= 0 and window_size > 0")
-        return s + w, s
-    raise ValueError(f"unknown attention strategy: {value}. Use full, window:<N>, or sinks:<S>,<W>")
+    sinks, window = (0, int(m.group(2))) if m.group(2) is not None else (int(m.group(3)), int(m.group(4)))
+    if window == 0:
+        raise ValueError(f"--attention {value}: the window must hold at least one position")
+    return sinks + window, sinks
 
 
 @dataclass
@@ -46,6 +48,9 @@ class BenchmarkResult:
     generated_tokens: int
     prefill_seconds: float
     decode_seconds: float
+    prefill_flops: float = 0.0            # of the timed prompt step
+    decode_bytes: float = 0.0             # every decode step's weights once + the cache of its live sequences
+    dtype: str = "bf16"
 
     @property
     def prefill_tokens_per_second(self) -> float:
@@ -54,6 +59,21 @@ class BenchmarkResult:
     @property
     def decode_tokens_per_second(self) -> float:
         return self.generated_tokens / self.decode_seconds if self.decode_seconds > 0 else 0.0
+
+    @property
+    def prefill_fraction_of_peak(self) -> float:
+        """Flops of the prompt step / its time / the MI355X's published dense matrix peak for the type."""
+        peak = MFMA_PEAK_FLOPS.get(self.dtype, 0.0)
+        return self.prefill_flops / self.prefill_seconds / peak if self.prefill_seconds > 0 and peak else 0.0
+
+    @property
+    def decode_bytes_per_second(self) -> float:
+        return self.decode_bytes / self.decode_seconds if self.decode_seconds > 0 else 0.0
+
+    @property
+    def decode_fraction_of_peak(self) -> float:
+        """Bytes the decode steps had to read / their time / the MI355X's published memory bandwidth."""
+        return self.decode_bytes_per_second / HBM_PEAK_BYTES
 
 
 class Llogos:
@@ -74,7 +94,7 @@ class Llogos:
         pool = max_tokens_in_cache or max_batch * pages_for(max_context) * PAGE_TOKENS
         self.max_context, self.max_batch = max_context, max_batch
         self.engine = Engine.from_folder(model, dtype=dtype, max_tokens=pool, n_slots=max(max_batch, 1),
-                                         device=device, **options)
+                                         device=device, max_seq=max_context, **options)
         self.config = self.engine.config
         self._generator = Generator(self.engine, max_batch=max_batch, synchronize=torch.cuda.synchronize)
 
@@ -105,4 +125,15 @@ class Llogos:
         self._generator.generate(prompts, warm)
         torch.cuda.synchronize()
         res = self._generator.generate(prompts, params)
-        return BenchmarkResult(res.prompt_tokens, res.generated_tokens, res.prefill_seconds, res.decode_seconds)
+        model, lens = self.engine.model, [len(p) for p in prompts]
+        weights, per_position = model.step_weight_bytes(), self.engine.cache.bytes_per_position()
+        # decode step t (the prompt step made token 0) reads the weights and, of each sequence, len + t positions
+        steps_by_batch = {}
+        for batch in res.batches:
+            steps_by_batch[len(batch)] = steps_by_batch.get(len(batch), 0) + max(0, max_tokens - 1)
+        decode_bytes = sum(n * weights for n in steps_by_batch.values()) + \
+            per_position * sum(n + t for n in lens for t in range(1, max_tokens))
+        flops = sum(model.step_flops([lens[r] for r in batch], wanted_rows=len(batch)) for batch in res.batches)
+        return BenchmarkResult(res.prompt_tokens, res.generated_tokens, res.prefill_seconds, res.decode_seconds,
+                               prefill_flops=flops, decode_bytes=decode_bytes,
+                               dtype="fp32" if self.engine.rt.is_f32 else "bf16")

@@ -22,7 +22,7 @@ from .pages import PAGE_TOKENS, CacheError, CacheFull, GroupPages, SlotAllocator
 class KVGroup:
     def __init__(self, spec: KVSpec, entries: List[int], n_pages: int, rt: Optional[Runtime]):
         self.spec = spec
-        self.entries = entries                       # schedule entries that own storage here
+        self.entries = entries                       # units that own storage here
         self.pages = GroupPages(n_pages, spec.window, spec.sinks)
         self.k = self.v = None
         if rt is not None:
@@ -37,8 +37,9 @@ class KVGroup:
 
 
 class Cache:
-    """needs: per schedule entry (KVSpec or None, StateSpec or None), as Model.cache_needs()
-    gives them; reads_from: per entry the entry whose storage it reads (itself when it owns).
+    """needs: per unit (one mixer of one scheduled run of a layer) a pair (KVSpec or None,
+    StateSpec or None), as Model.cache_needs() gives them; reads_from: per unit the unit whose
+    storage it reads (None or itself when it owns), as Model.cache_reads() gives them.
     With rt=None no device memory is made (bookkeeping only)."""
 
     def __init__(self, needs: Sequence[Tuple[Optional[KVSpec], Optional[StateSpec]]],
@@ -124,6 +125,13 @@ class Cache:
     def bytes(self) -> int:
         return sum(g.bytes() for g in self.groups)
 
+    def bytes_per_position(self) -> int:
+        """Bytes of keys and values that one position of one sequence takes in all groups."""
+        if self.rt is None:
+            return 0
+        elt = torch.empty((), dtype=self.rt.dtype).element_size()
+        return sum(2 * len(g.entries) * g.spec.n_kv_heads * g.spec.head_dim * elt for g in self.groups)
+
     # ---- a step's storage ----------------------------------------------------------
     def reserve(self, slot_ids: Sequence[int], new_lens: Sequence[int]) -> None:
         """Pages for every position below new_len of each sequence, in every group; either
@@ -174,7 +182,7 @@ class Cache:
         return out
 
     def layer_caches(self, tables: List[torch.Tensor]) -> List[LayerCache]:
-        """What each schedule entry sees in a step whose group tables are on the device."""
+        """What each unit sees in a step whose group tables are on the device."""
         out = []
         for e, loc in enumerate(self.entry_group):
             lc = LayerCache(state=self.states[e])

@@ -4,6 +4,8 @@ from __future__ import annotations
 
 from typing import Dict, List
 
+# Positions a page holds.  This is the definition; the kernel library has the same number
+# compiled in (kPageTokens) and loading it fails if the two differ.
 PAGE_TOKENS = 64
 
 

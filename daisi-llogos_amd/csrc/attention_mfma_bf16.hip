@@ -806,10 +806,34 @@ static bool mfma_shape_ok(int n_heads, int n_kv_heads, int head_dim) {
 // vector memory path, so few large blocks are slower than many small ones: blocks grow only
 // while there are enough of them for every CU (then the merge kernel falls away for contexts
 // of up to 1,024 positions), within the LDS that the waves' outputs need.
-static int decode_waves(int group, int table_width, int sequences_x_kv_heads) {
+// The choice must not depend on how many other sequences happen to be in the step beyond the
+// step's class of batch sizes (the sizes at which single-token steps are captured: a batch in
+// between runs padded to the next of them), or a sequence's sums would come in another order
+// alone than beside others of its class: `batch` is rounded up to its class first.
+LLOGOS_EXPORT int llogos_batch_class(int batch) {
+    static const int classes[] = {1, 2, 3, 4, 5, 6, 7, 8, 12, 16, 24, 32, 48, 64};
+    for (int c : classes) if (batch <= c) return c;
+    return (batch + 63) / 64 * 64;
+}
+
+// compute units of the current device, asked for once per device
+static int compute_units() {
+    static int cached[64];
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 256;
+    if (cached[device] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || n <= 0) n = 256;
+        cached[device] = n;
+    }
+    return cached[device];
+}
+
+static int decode_waves(int group, int table_width, int batch, int n_kv_heads) {
+    const long long pairs = (long long)llogos_batch_class(batch) * n_kv_heads;
+    const int units = compute_units();
     int waves = group <= 4 ? 16 : (group <= 8 ? 8 : 4);
-    while (waves > 4 && (waves / 2 >= table_width ||
-                         (long long)sequences_x_kv_heads * ((table_width + waves - 1) / waves) < 256))
+    while (waves > 4 && (waves / 2 >= table_width || pairs * ((table_width + waves - 1) / waves) < units))
         waves /= 2;
     return waves;
 }
@@ -818,7 +842,7 @@ static int decode_waves(int group, int table_width, int sequences_x_kv_heads) {
 LLOGOS_EXPORT long long llogos_attn_decode_workspace(int batch, int n_heads, int n_kv_heads, int head_dim,
                                                      int table_width) {
     if (n_kv_heads <= 0 || n_heads % n_kv_heads) return 0;
-    const int waves = decode_waves(n_heads / n_kv_heads, table_width, batch * n_kv_heads);
+    const int waves = decode_waves(n_heads / n_kv_heads, table_width, batch, n_kv_heads);
     const int n_z = (table_width + waves - 1) / waves;
     return n_z == 1 ? 0 : (long long)batch * n_heads * n_z * (head_dim + 2);
 }
@@ -833,7 +857,7 @@ static int launch_decode(void* out, const void* q, int q_stride, const QkvSource
     if (workspace_floats < llogos_attn_decode_workspace(batch, n_heads, n_kv_heads, head_dim, table_width))
         return LLOGOS_BAD_ARGUMENT;
     const int group = n_heads / n_kv_heads;
-    const int waves = decode_waves(group, table_width, batch * n_kv_heads);
+    const int waves = decode_waves(group, table_width, batch, n_kv_heads);
     const int n_z = (table_width + waves - 1) / waves;
     if (n_z > 1 && workspace == nullptr) return LLOGOS_BAD_ARGUMENT;
     dim3 grid(batch, n_kv_heads, n_z), mgrid(batch, n_heads);

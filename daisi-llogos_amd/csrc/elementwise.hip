@@ -4,27 +4,51 @@
 // is float or bfloat16.
 #include "common.h"
 
+// what the host side checks its own page size against when it loads the library
+LLOGOS_EXPORT int llogos_page_tokens(void) { return kPageTokens; }
+LLOGOS_EXPORT int llogos_wave_size(void) { return kWave; }
+
 // ---------------------------------------------------------------- embedding
 // out[t, :] = table[ids[t], :] as float.  One block per token.
 // (reference: Daisi.Llogos.Cuda/kernels/elementwise.cu:402-457, one row per call)
 template <typename T>
 __global__ void embed_kernel(float* __restrict__ out, const T* __restrict__ table,
-                             const int* __restrict__ ids, int H) {
+                             const int* __restrict__ ids, int H, float scale) {
     const int t = blockIdx.x;
     const T* row = table + (size_t)ids[t] * H;
     float* o = out + (size_t)t * H;
-    for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = load_f32(row + i);
+    if (scale == 1.0f) {
+        for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = load_f32(row + i);
+    } else {
+        for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = load_f32(row + i) * scale;
+    }
 }
 
+// out[t, :] = table[ids[t], :] * scale (scale 1: a row copy)
 LLOGOS_EXPORT int llogos_embed(float* out, const void* table, int table_dtype, const int* ids,
-                               int T, int H, hipStream_t stream) {
+                               int T, int H, float scale, hipStream_t stream) {
     if (T <= 0 || H <= 0) return LLOGOS_BAD_ARGUMENT;
     if (table_dtype == DT_F32)
-        embed_kernel<float><<<T, 256, 0, stream>>>(out, (const float*)table, ids, H);
+        embed_kernel<float><<<T, 256, 0, stream>>>(out, (const float*)table, ids, H, scale);
     else if (table_dtype == DT_BF16)
-        embed_kernel<bf16_t><<<T, 256, 0, stream>>>(out, (const bf16_t*)table, ids, H);
+        embed_kernel<bf16_t><<<T, 256, 0, stream>>>(out, (const bf16_t*)table, ids, H, scale);
     else
         return LLOGOS_BAD_ARGUMENT;
+    return LLOGOS_LAUNCH_CHECK();
+}
+
+// x = x * scale, then, with cap > 0, x = cap * tanh(x / cap): scaled and soft-capped logits
+__global__ void scale_softcap_kernel(float* __restrict__ x, long long n, float scale, float cap) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float v = x[i] * scale;
+    if (cap > 0.f) v = cap * tanhf(v / cap);
+    x[i] = v;
+}
+
+LLOGOS_EXPORT int llogos_scale_softcap(float* x, long long n, float scale, float cap, hipStream_t stream) {
+    if (n <= 0 || cap < 0.f) return LLOGOS_BAD_ARGUMENT;
+    scale_softcap_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(x, n, scale, cap);
     return LLOGOS_LAUNCH_CHECK();
 }
 

@@ -104,11 +104,12 @@ LLOGOS_EXPORT int llogos_argmax(int* out, const float* logits, int R, int V, hip
 // then - frequency * count - presence once per distinct token; tokens 10 and 13 are spared
 // unless penalize_newline), the given ids set to -inf (PreventEOS, :49-53), then times
 // 1 / temperature (:60-62).
+constexpr int kMaxBanned = 64;           // ids that a call can ban (a model's stop tokens)
 struct PenaltyParams {
     float repetition, frequency, presence, inv_temperature;
     int penalize_newline;
     int n_banned;
-    int banned[8];
+    int banned[kMaxBanned];
 };
 
 __global__ __launch_bounds__(kSampleThreads) void sample_prepare_kernel(
@@ -157,7 +158,7 @@ LLOGOS_EXPORT int llogos_sample_prepare(float* work, const float* logits, int R,
                                         const int* hist, const int* hist_len, int hist_stride,
                                         float repetition, float frequency, float presence, float inv_temperature,
                                         int penalize_newline, const int* banned, int n_banned, hipStream_t stream) {
-    if (R <= 0 || V <= 0 || n_banned < 0 || n_banned > 8) return LLOGOS_BAD_ARGUMENT;
+    if (R <= 0 || V <= 0 || n_banned < 0 || n_banned > kMaxBanned) return LLOGOS_BAD_ARGUMENT;
     PenaltyParams pp{repetition, frequency, presence, inv_temperature, penalize_newline, n_banned, {}};
     for (int i = 0; i < n_banned; ++i) pp.banned[i] = banned[i];
     sample_prepare_kernel<<<R, kSampleThreads, 0, stream>>>(work, logits, V, hist, hist_len, hist_stride, pp);

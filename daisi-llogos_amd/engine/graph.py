@@ -35,6 +35,8 @@ def bucket_width(width: int) -> int:
 
 
 def bucket_batch(batch: int) -> int:
+    """The captured batch size that serves `batch`.  (The kernel library rounds a batch up the
+    same way where a kernel's shape depends on the batch: llogos_batch_class.)"""
     for b in BATCH_BUCKETS:
         if batch <= b:
             return b
@@ -100,8 +102,17 @@ class DecodeGraph:
             K.gather_i32(self.views[0], device_ids[0], self.views[-1])
         if self.graph is None:
             # the longest context this graph may ever see: what its page tables can hold
-            cap = max(self.widths) * 64 if self.widths else 64
-            self._forward(cap)                          # warm up: lazy workspaces are made outside the capture
+            cap = max(self.widths) * K.PAGE_TOKENS if self.widths else K.PAGE_TOKENS
+            # Warm up: lazy workspaces are made outside the capture.  The warm-up is a real run of
+            # the step that the replay below runs again.  For keys and values that changes nothing
+            # (the same values go to the same places); fixed-size state would be advanced twice,
+            # so it is put back.
+            states = self._engine().cache.states
+            saved = [None if st is None else st.clone() for st in states]
+            self._forward(cap)
+            for st, keep in zip(states, saved):
+                if st is not None:
+                    st.copy_(keep)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             # freeing device memory or another graph is not allowed while a stream captures:

@@ -32,7 +32,8 @@ GRAPH_MAX_BATCH = 64
 
 
 class StepError(ValueError):
-    """A step that cannot run: empty token list, token out of range, slot used twice."""
+    """A step that cannot run: empty token list, token out of range, slot used twice, a sequence
+    longer than the engine's limit."""
 
 
 def resolve_dtype(dtype: Union[str, torch.dtype]) -> torch.dtype:
@@ -60,15 +61,19 @@ class Engine:
     """A bound model with its cache.  `step` is the only way tokens reach the model."""
 
     def __init__(self, model: Model, rt: Runtime, max_tokens: int, n_slots: int = 64, config=None,
-                 use_graphs: Optional[bool] = None):
+                 use_graphs: Optional[bool] = None, max_seq: Optional[int] = None):
         self.model, self.rt, self.config = model, rt, config
+        # The longest a sequence may become: the caller's limit (the reference's --max-context,
+        # Daisi.Llogos.Cli/Program.cs:194-197, 805) within the positions the model was made for
+        # (max_position_embeddings); a step that would go beyond is refused, nothing runs.
+        limits = [int(n) for n in (max_seq, model.spec.max_position) if n]
+        self.max_seq: Optional[int] = min(limits) if limits else None
         # single-token steps are replayed as HIP graphs when every mixer and feed-forward allows it
-        graph_ok = all(layer.mixer.graph_safe and getattr(layer.ffn, "graph_safe", False) for layer in model.layers)
+        graph_ok = model.graph_safe
         if use_graphs is None:
             use_graphs = os.environ.get("LLOGOS_GRAPHS", "1") != "0"
         self.graphs = GraphCache(self) if (use_graphs and graph_ok) else None
-        reads_from = [e.cache_of for e in model.schedule]
-        self.cache = Cache(model.cache_needs(), reads_from, max_tokens, rt, n_slots)
+        self.cache = Cache(model.cache_needs(), model.cache_reads(), max_tokens, rt, n_slots)
         self.vocab_size = model.spec.vocab_size
         self.steps_run = 0
 
@@ -76,7 +81,7 @@ class Engine:
     @classmethod
     def from_folder(cls, folder: str, dtype: Union[str, torch.dtype] = "bfloat16", max_tokens: int = 4096,
                     n_slots: int = 64, device: Union[str, torch.device] = "cuda:0",
-                    use_graphs: Optional[bool] = None, **spec_options) -> "Engine":
+                    use_graphs: Optional[bool] = None, max_seq: Optional[int] = None, **spec_options) -> "Engine":
         """config.json chooses the model class through the registry; model.safetensors is
         checked against what the model needs before any tensor is read."""
         dev = require_gpu(device)
@@ -94,38 +99,33 @@ class Engine:
                 torch.cuda.synchronize()
         finally:
             ckpt.close()
-        return cls(model, rt, max_tokens, n_slots, config, use_graphs)
+        return cls(model, rt, max_tokens, n_slots, config, use_graphs, max_seq)
 
     @classmethod
     def from_config(cls, config: dict, seed: int = 0, dtype: Union[str, torch.dtype] = "bfloat16",
                     max_tokens: int = 4096, n_slots: int = 64, device: Union[str, torch.device] = "cuda:0",
-                    std: float = 0.02, use_graphs: Optional[bool] = None, **spec_options) -> "Engine":
-        """A model of the parsed config.json `config` with random weights made on the device
-        (matrices N(0, std), norm weights 1 + U(-0.1, 0.1)), without a model folder."""
-        import hashlib
+                    std: float = 0.02, use_graphs: Optional[bool] = None, max_seq: Optional[int] = None,
+                    **spec_options) -> "Engine":
+        """A model of the parsed config.json `config` with random weights made on the device,
+        without a model folder: the weights that write_random_model(folder, config, seed) writes
+        (matrices N(0, std), norm weights 1 + U(-0.1, 0.1)), stored in the configuration's
+        `torch_dtype` first, as a folder would hold them."""
+        from ..weights.random_init import random_tensor, storage_dtype
         dev = require_gpu(device)
         arch = architecture_of(config)
         typed = arch.read_config(config)
         model = Model(arch.model_spec(typed, **spec_options))
         specs = {s.name: s for s in model.tensor_specs()}
         rt = Runtime(dev, resolve_dtype(dtype))
-        gen = torch.Generator(device=dev)
+        store = storage_dtype(config)
 
         def get(name: str):
             spec = specs.get(name)
-            if spec is None:
-                return None
-            digest = hashlib.sha256(f"{seed}:{name}".encode()).digest()
-            gen.manual_seed(int.from_bytes(digest[:8], "little") & ((1 << 63) - 1))
-            if spec.kind == "norm":
-                return 1.0 + (torch.rand(spec.shape, generator=gen, device=dev) * 0.2 - 0.1)
-            t = torch.empty(spec.shape, dtype=rt.dtype if spec.kind in ("matrix", "table") else torch.float32,
-                            device=dev)
-            return t.normal_(0.0, std, generator=gen)
+            return None if spec is None else random_tensor(spec, seed, store, std, device=dev)
         with torch.cuda.device(dev):
             model.bind(get, rt)
             torch.cuda.synchronize()
-        return cls(model, rt, max_tokens, n_slots, typed, use_graphs)
+        return cls(model, rt, max_tokens, n_slots, typed, use_graphs, max_seq)
 
     # ---- slots ---------------------------------------------------------------------
     def _graph_slots(self) -> int:
@@ -181,6 +181,10 @@ class Engine:
                 raise StepError(f"device_ids rows outside 0..{src.numel() - 1}")
         starts = [self.cache.length(s) for s in slot_ids]
         new_lens = [s + c for s, c in zip(starts, counts)]
+        if self.max_seq is not None and max(new_lens) > self.max_seq:
+            i = int(np.argmax(new_lens))
+            raise StepError(f"sequence {i} (slot {slot_ids[i]}) would become {new_lens[i]} positions long; "
+                            f"the limit is {self.max_seq}")
         cu = np.zeros(len(entries) + 1, dtype=np.int64)
         np.cumsum(counts, out=cu[1:])
         rows = self._want_rows(want, counts, cu)

@@ -12,11 +12,12 @@ from typing import Optional, Sequence, Tuple
 import torch
 
 from . import library
+from ..cache.pages import PAGE_TOKENS      # the one definition; the library is checked against it when loaded
 
 F32, BF16 = 0, 1
 _DT = {torch.float32: F32, torch.bfloat16: BF16}
-PAGE_TOKENS = 64
 MAX_HEAD_DIM = 512
+MAX_BANNED = 64             # ids one sampling call can set to -inf (kMaxBanned in csrc/sampling.hip)
 
 
 class KernelError(RuntimeError):
@@ -92,15 +93,25 @@ def _check_pools(k_pool: torch.Tensor, v_pool: torch.Tensor, n_kv_heads: int, he
 
 
 # ----------------------------------------------------------------------------
-def embed(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
-    """float32 rows of `table` ([V, H], float32 or bfloat16) at int32 `ids`."""
+def embed(table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """float32 rows of `table` ([V, H], float32 or bfloat16) at int32 `ids`, times `scale`."""
     _dev(table, ids)
     _i32(ids, "ids")
     _need(table.dim() == 2 and ids.dim() == 1, "embed: table [V, H], ids [T]")
     T, H = ids.numel(), table.shape[1]
     out = torch.empty((T, H), dtype=torch.float32, device=table.device)
-    _check(_lib().llogos_embed(_p(out), _p(table), _dt(table), _p(ids), T, H, _stream()), "embed")
+    _check(_lib().llogos_embed(_p(out), _p(table), _dt(table), _p(ids), T, H, ctypes.c_float(scale), _stream()), "embed")
     return out
+
+
+def scale_softcap(x: torch.Tensor, scale: float = 1.0, cap: float = 0.0) -> torch.Tensor:
+    """In place on float32 `x`: x * scale, then with cap > 0 bent to cap * tanh(x / cap)."""
+    _dev(x)
+    _need(x.dtype == torch.float32 and cap >= 0, "scale_softcap: float32 values, cap >= 0")
+    if x.numel():
+        _check(_lib().llogos_scale_softcap(_p(x), ctypes.c_longlong(x.numel()), ctypes.c_float(scale),
+                                           ctypes.c_float(cap), _stream()), "scale_softcap")
+    return x
 
 
 def gather_i32(dst: torch.Tensor, src: torch.Tensor, rows: torch.Tensor) -> None:
@@ -279,11 +290,25 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
 # ----------------------------------------------------------------------------
 # dispatch: which kernel serves a call
 # ----------------------------------------------------------------------------
+_compute_units = {}
+
+
+def compute_units(device=None) -> int:
+    """Compute units of the GPU the products are planned for, read from the device once (256 on
+    an MI355X; that number also stands in where no GPU is visible, for planning on the host)."""
+    if not torch.cuda.is_available():
+        return 256
+    index = torch.cuda.current_device() if device is None else torch.device(device).index or 0
+    if index not in _compute_units:
+        _compute_units[index] = int(torch.cuda.get_device_properties(index).multi_processor_count)
+    return _compute_units[index]
+
+
 SKINNY_MAX_ROWS = 64
 LDS_MAX_ROWS = 128          # rows the LDS few-row product takes without a fused producer
 
 
-def lds_splits(M: int, N: int, K: int, n_cus: int = 256) -> int:
+def lds_splits(M: int, N: int, K: int, n_cus: Optional[int] = None) -> int:
     """Blocks along k for the LDS few-row product.  Measured on the MI355X, three things decide:
     how evenly the blocks fill the compute units (544 blocks on 256 units run as long as 768),
     whether there are enough of them to keep the memory system busy (about 1.5 a unit), and the
@@ -291,6 +316,7 @@ def lds_splits(M: int, N: int, K: int, n_cus: int = 256) -> int:
     about 6 M / K of the weights' time each).  64 and more rows of activations leave LDS for two
     blocks a unit, so blocks come in rounds of twice the units there.  More blocks along k are taken only
     for a clear gain (8 %), since they also cost the consumer a fused form or a launch."""
+    n_cus = n_cus or compute_units()
     n_blocks = -(-N // 64)
     chunks = -(-K // 256)
     rows = 16 if M <= 16 else (32 if M <= 32 else (64 if M <= 64 else 128))
@@ -312,11 +338,12 @@ def lds_splits(M: int, N: int, K: int, n_cus: int = 256) -> int:
     return best
 
 
-def stationary_strips(N: int, K: int, n_cus: int = 256) -> int:
+def stationary_strips(N: int, K: int, n_cus: Optional[int] = None) -> int:
     """Strips of 16 rows of w a block of the activation-stationary product streams.  More strips
     spread the activations' loads over more weights; the blocks must still fill the compute
     units evenly (598 blocks on 256 units were measured at 3.9 TB/s where 448 reach 5.5) and
     leave about seven waves a unit."""
+    n_cus = n_cus or compute_units()
     waves = 4 if K <= 4096 else 8
     n_strips = -(-N // 16)
     best, best_score = 2, -1.0
@@ -330,7 +357,7 @@ def stationary_strips(N: int, K: int, n_cus: int = 256) -> int:
     return best
 
 
-def resident_strips(M: int, N: int, K: int, n_cus: int = 256) -> Optional[Tuple[int, int]]:
+def resident_strips(M: int, N: int, K: int, n_cus: Optional[int] = None) -> Optional[Tuple[int, int]]:
     """(parts of k, strips per block) for the few-row product whose operands go straight into
     LDS, or None where it is not the faster one.  It pays for 17 to 64 rows on a tall, large
     matrix when its blocks, 5 to 9 strips high, are all resident at once (two to a compute
@@ -341,8 +368,9 @@ def resident_strips(M: int, N: int, K: int, n_cus: int = 256) -> Optional[Tuple[
     slower where it does not, among them everything below 24576 rows)."""
     if not (16 < M <= 64 and N >= 24576 and K % 64 == 0):
         return None
+    n_cus = n_cus or compute_units()
     places = 2 * n_cus
-    other = -(-N // 64) * lds_splits(M, N, K)
+    other = -(-N // 64) * lds_splits(M, N, K, n_cus)
     other_fill = other / places if other <= places else 0.0
     n_strips = -(-N // 16)
     best, best_fill = None, 0.0
@@ -616,13 +644,14 @@ PREFILL_TILE_ROWS = 0        # 0: chosen by the step; 64 or 128 force a prefill 
 PREFILL_HALVES = 0           # 0: chosen by the step; 1 or 2 sets of waves a block of the 128-row kernel (tests)
 
 
-def prefill_halves(lens: Sequence[int], starts: Optional[Sequence[int]], n_heads: int, n_cus: int = 256) -> int:
+def prefill_halves(lens: Sequence[int], starts: Optional[Sequence[int]], n_heads: int, n_cus: Optional[int] = None) -> int:
     """Sets of waves a block of the 128-row prompt attention: 2 (the sets take a tile's pages in
     turn) where the pages of the longest tile, one after the other, take longer than the chip
     needs for all tiles; 1 (two independent blocks a compute unit, 15 % more throughput) where
     the work of all tiles decides.  Measured at the 8B head shape: two sets win up to 2,048
     tokens of one prompt (1,536: 45 us against 57) and lose from 2,560 on and for many short
     prompts."""
+    n_cus = n_cus or compute_units()
     longest = total = 0
     for i, n in enumerate(lens):
         start = starts[i] if starts else 0
@@ -758,13 +787,13 @@ def sample_prepare(logits: torch.Tensor, history: Optional[torch.Tensor], histor
     _dev(logits, history, history_len)
     _i32(history, "history"); _i32(history_len, "history_len")
     _need(logits.dtype == torch.float32 and logits.dim() == 2, "sample_prepare: logits must be float32 [R, V]")
-    _need(len(banned) <= 8, "sample_prepare: at most 8 banned ids")
+    _need(len(banned) <= MAX_BANNED, f"sample_prepare: at most {MAX_BANNED} banned ids, got {len(banned)}")
     R, V = logits.shape
     if history is not None:
         _need(history.dim() == 2 and history.shape[0] == R and history_len is not None
               and history_len.numel() == R, "sample_prepare: history [R, W] with lengths [R]")
     work = torch.empty_like(logits)
-    ban = (ctypes.c_int * 8)(*list(banned))
+    ban = (ctypes.c_int * MAX_BANNED)(*list(banned))
     inv_t = 1.0 / temperature if temperature > 0 else 1.0
     _check(_lib().llogos_sample_prepare(
         _p(work), _p(logits), R, V, _p(history), _p(history_len), history.stride(0) if history is not None else 0,
@@ -800,3 +829,47 @@ def sample_pipeline(work: torch.Tensor, uniforms: torch.Tensor, top_k: int, top_
         ctypes.c_float(min_p), ctypes.c_float(typical_p), int(min_keep), SAMPLE_ORDERS[order], _stream()),
         "sample_pipeline")
     return out
+
+
+# ----------------------------------------------------------------------------
+# what the GPU does at best, measured
+# ----------------------------------------------------------------------------
+def measure_read_bandwidth(n_bytes: int, repeats: int = 20, blocks_per_unit: int = 8, device="cuda:0") -> float:
+    """Bytes a second at which a kernel that only reads streams `n_bytes` of device memory
+    (16-byte loads, four in flight per thread), best of `repeats` runs over a buffer that was
+    not the last thing read."""
+    dev = torch.device(device)
+    n_bytes = max(1 << 20, n_bytes // 16 * 16)
+    with torch.cuda.device(dev):
+        buf = torch.empty(n_bytes // 4, dtype=torch.int32, device=dev).fill_(1)
+        other = torch.empty(max(n_bytes // 4, 1 << 27), dtype=torch.int32, device=dev).fill_(2)   # evicts the caches
+        sink = torch.zeros(4, dtype=torch.int32, device=dev)
+        blocks = compute_units(dev) * blocks_per_unit
+        lib, best = _lib(), 0.0
+        for _ in range(repeats):
+            _check(lib.llogos_measure_read(_p(other), ctypes.c_longlong(other.numel() * 4), blocks, _p(sink), _stream()), "measure_read")
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            _check(lib.llogos_measure_read(_p(buf), ctypes.c_longlong(n_bytes), blocks, _p(sink), _stream()), "measure_read")
+            end.record()
+            end.synchronize()
+            best = max(best, n_bytes / (start.elapsed_time(end) * 1e-3))
+    return best
+
+
+def measure_mfma_rate(iters: int = 20000, blocks_per_unit: int = 2, device="cuda:0") -> float:
+    """bfloat16 flops a second of v_mfma_f32_16x16x32_bf16 issued back to back by eight waves
+    on every compute unit (eight independent accumulators a wave)."""
+    dev = torch.device(device)
+    with torch.cuda.device(dev):
+        blocks = compute_units(dev) * blocks_per_unit
+        out = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
+        lib, best = _lib(), 0.0
+        for _ in range(4):
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            _check(lib.llogos_measure_mfma(_p(out), blocks, iters, _stream()), "measure_mfma")
+            end.record()
+            end.synchronize()
+            best = max(best, blocks * 4 * iters * 8 * 16384.0 / (start.elapsed_time(end) * 1e-3))
+    return best

@@ -1,7 +1,8 @@
 """Builds and loads the HIP kernel library (gfx950) that every device op calls.
 
 `build()` always compiles; `load()` uses the library that is there and compiles only
-when none is.  There is no fallback: without the library the ops raise.
+when none is, or when the one that is there was built from other sources.  There is no
+fallback: without the library the ops raise.
 """
 from __future__ import annotations
 
@@ -55,9 +56,21 @@ def _source_hash() -> str:
     return h.hexdigest()
 
 
+def _private(path: str) -> bool:
+    """Whether a folder under the shared temporary directory is this user's alone (a library is
+    never built into or loaded from a folder that another user could have written)."""
+    try:
+        st = os.stat(path)
+    except OSError:
+        return False
+    return st.st_uid == os.getuid() and (st.st_mode & 0o077) == 0
+
+
 def _writable(path: str) -> bool:
     try:
-        os.makedirs(path, exist_ok=True)
+        os.makedirs(path, mode=0o700, exist_ok=True)
+        if not path.startswith(_PKG) and not _private(path):
+            return False
         probe = os.path.join(path, f".probe{os.getpid()}")
         with open(probe, "w"):
             pass
@@ -80,11 +93,14 @@ def find_library() -> str | None:
     env = os.environ.get("LLOGOS_KERNEL_LIBRARY")
     if env:
         return env if os.path.isfile(env) else None
+    stale = None
     for d in build_dirs():
         p = os.path.join(d, LIB_NAME)
-        if os.path.isfile(p):
-            return p
-    return None
+        if os.path.isfile(p) and (d.startswith(_PKG) or _private(d)):
+            if not is_stale(p):
+                return p
+            stale = stale or p          # one built from the present sources, in a later folder, goes first
+    return stale
 
 
 def _hipcc() -> str:
@@ -175,13 +191,24 @@ def load() -> ctypes.CDLL:
     path = find_library()
     if path is None:
         path = build()
-    elif is_stale(path):
-        _log(f"warning: {path} is older than the sources in {_CSRC}; run __graft_entry__.build() to refresh it")
+    elif not os.environ.get("LLOGOS_KERNEL_LIBRARY") and is_stale(path):
+        # Python's declarations of the entry points describe the present sources: a library built
+        # from other sources would take wrong pointers and strides.  (A library named by
+        # LLOGOS_KERNEL_LIBRARY is the user's word and is trusted.)
+        _log(f"{path} was built from other sources than those in {_CSRC}: building again")
+        try:
+            path = build()
+        except KernelLibraryError as e:
+            raise KernelLibraryError(f"{path} is stale and cannot be rebuilt: {e}") from e
     try:
         lib = ctypes.CDLL(path)
     except OSError as e:
         raise KernelLibraryError(f"cannot load {path}: {e}") from e
     lib.llogos_attn_decode_workspace.restype = ctypes.c_longlong       # every other entry returns an int code
+    from ..cache.pages import PAGE_TOKENS
+    if lib.llogos_page_tokens() != PAGE_TOKENS:
+        raise KernelLibraryError(f"{path} was built for pages of {lib.llogos_page_tokens()} positions, "
+                                 f"the cache uses {PAGE_TOKENS}")
     with _lock:
         _lib = lib
     return lib

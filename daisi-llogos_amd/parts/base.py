@@ -105,6 +105,28 @@ class Part:
         the kernels want."""
         self.rt = rt
 
+    def weight_bytes(self) -> int:
+        """Bytes of the device tensors this part and its sub-parts hold: what a step reads of it."""
+        total = 0
+        for v in vars(self).values():
+            if isinstance(v, torch.Tensor):
+                total += v.numel() * v.element_size()
+            elif isinstance(v, Part):
+                total += v.weight_bytes()
+            elif isinstance(v, (list, tuple)):
+                total += sum(x.weight_bytes() for x in v if isinstance(x, Part))
+        return total
+
+    def matrix_elements(self) -> int:
+        """Elements of the matrices this part multiplies every token with (two flops each)."""
+        total = 0
+        for v in vars(self).values():
+            if isinstance(v, Part):
+                total += v.matrix_elements()
+            elif isinstance(v, (list, tuple)):
+                total += sum(x.matrix_elements() for x in v if isinstance(x, Part))
+        return total
+
 
 class Mixer(Part):
     """Token mixer: forward(ctx, h [T, H] in the runtime's type, cache) -> [T, H], or float32
@@ -117,7 +139,10 @@ class Mixer(Part):
         return None
 
     # True when forward reads the step only through device tensors (ids, tok_seq, tok_pos, slots,
-    # page tables), so that a captured single-token step can be replayed with new contents.
+    # page tables, the state tensor at the rows of `slots`), so that a captured single-token step
+    # can be replayed with new contents.  A captured step is run once for real before its
+    # capture; the engine puts the fixed-size state back afterwards, so a mixer with state may
+    # set this too, as long as the state tensor is all it changes beside its cache pages.
     graph_safe = False
 
     def forward(self, ctx: StepContext, h: torch.Tensor, cache: LayerCache) -> torch.Tensor:
@@ -145,11 +170,44 @@ class Norm(Part):
         raise NotImplementedError
 
 
+class Block(Part):
+    """Arrangement of a layer's parts: which mixers and feed-forwards it holds, with which norms
+    around them, and how their outputs join the residual stream.
+
+    forward(ctx, x, pending, caches) -> (x, pending): `x` is the float32 residual stream
+    [T, H], `pending` a delta that is still to be added to it ([T, H] or partial sums
+    [parts, T, H], or None), `caches` one LayerCache for each of mixers(), in that order."""
+
+    def mixers(self) -> List["Mixer"]:
+        return []
+
+    def feed_forwards(self) -> List["FeedForward"]:
+        return []
+
+    def parts(self) -> List[Part]:
+        raise NotImplementedError
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [s for p in self.parts() for s in p.tensor_specs()]
+
+    def bind(self, get: Callable[[str], Optional[torch.Tensor]], rt: Runtime) -> None:
+        super().bind(get, rt)
+        for p in self.parts():
+            p.bind(get, rt)
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, pending: Optional[torch.Tensor],
+                caches: List[LayerCache]) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+        raise NotImplementedError
+
+
 class PositionEncoding(Part):
     """prepare(ctx) -> whatever the mixer's kernels need for this step's positions."""
 
     def prepare(self, ctx: StepContext):
         raise NotImplementedError
+
+    def weight_bytes(self) -> int:
+        return 0                   # its tables come from the configuration, not from the checkpoint
 
 
 # ---------------------------------------------------------------------------

@@ -11,27 +11,26 @@ from typing import Callable, List, Optional, Tuple
 
 import torch
 
-from .base import FeedForward, LayerCache, Mixer, Norm, Part, Runtime, StepContext, TensorSpec, register_block
+from .base import Block, FeedForward, LayerCache, Mixer, Norm, Part, Runtime, StepContext, TensorSpec, register_block
 
 
 @register_block("pre_norm")
-class PreNormBlock(Part):
+class PreNormBlock(Block):
     def __init__(self, mixer_norm: Norm, mixer: Mixer, ffn_norm: Norm, ffn: FeedForward):
         self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+
+    def mixers(self) -> List[Mixer]:
+        return [self.mixer]
+
+    def feed_forwards(self) -> List[FeedForward]:
+        return [self.ffn]
 
     def parts(self) -> List[Part]:
         return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn]
 
-    def tensor_specs(self) -> List[TensorSpec]:
-        return [s for p in self.parts() for s in p.tensor_specs()]
-
-    def bind(self, get: Callable[[str], Optional[torch.Tensor]], rt: Runtime) -> None:
-        super().bind(get, rt)
-        for p in self.parts():
-            p.bind(get, rt)
-
     def forward(self, ctx: StepContext, x: torch.Tensor, pending: Optional[torch.Tensor],
-                cache: LayerCache) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+                caches) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+        cache = caches[0] if isinstance(caches, (list, tuple)) else caches
         h = self.mixer_norm.forward(x, pending)
         a = self.mixer.forward(ctx, h, cache)
         h = self.ffn_norm.forward(x, a)

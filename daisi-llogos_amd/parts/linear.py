@@ -43,6 +43,9 @@ class Linear(Part):
         if self.has_bias:
             self.bias = _to_device([get(n + ".bias") for n in self.names], torch.float32, rt.device)
 
+    def matrix_elements(self) -> int:
+        return self.in_features * self.total_out
+
     def bind_shared(self, weight: torch.Tensor, rt: Runtime) -> None:
         """Use a matrix that another part already holds on the device (tied embeddings)."""
         self.rt = rt

@@ -18,6 +18,8 @@ class Sampler:
     def __init__(self, params: GenerationParams, stop_tokens: Sequence[int] = ()):
         self.params = params
         self.stop_tokens = tuple(stop_tokens)
+        if params.prevent_eos and len(self.stop_tokens) > K.MAX_BANNED:
+            raise ValueError(f"prevent_eos can ban at most {K.MAX_BANNED} stop tokens, got {len(self.stop_tokens)}")
         self._fresh_seed = None
         if params.seed is None and params.temperature > 0:
             self._fresh_seed = int(np.random.SeedSequence().generate_state(1)[0])
@@ -48,7 +50,7 @@ class Sampler:
             arrays.append(np.asarray(self.uniforms(requests, indices), dtype=np.float32))
         staged = self._to_device(arrays, logits.device)
         hist, hist_len = (staged[0], staged[1]) if p.has_penalties else (None, None)
-        banned = self.stop_tokens[:8] if p.prevent_eos else ()
+        banned = self.stop_tokens if p.prevent_eos else ()
         work = K.sample_prepare(logits, hist, hist_len, p.repetition_penalty, p.frequency_penalty,
                                 p.presence_penalty, p.temperature, p.penalize_newline, banned)
         if p.temperature == 0:

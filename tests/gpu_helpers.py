@@ -25,9 +25,31 @@ DTYPES = ["float32", "bfloat16"]
 _tmp = tempfile.TemporaryDirectory(prefix="llogos_test_models_")
 
 
+PEAKY = "_peaky"            # suffix of a configuration's name: the same model with sharp attention
+PEAKY_FACTOR = 12.0
+
+
 @functools.lru_cache(maxsize=None)
 def folder(name: str, seed: int = 11) -> str:
+    """The model folder of a tiny configuration.  `<name>_peaky` is the same model with its query
+    and key projections (and their biases) scaled up, so that scores spread over tens of units and
+    each query looks at a few keys: a key that is dropped, or one too many, then moves the logits
+    by far more than rounding does."""
     path = os.path.join(_tmp.name, f"{name}_{seed}")
+    if name.endswith(PEAKY):
+        import json
+        import shutil
+        from safetensors.torch import load_file, save_file
+        base = folder(name[:-len(PEAKY)], seed)
+        os.makedirs(path, exist_ok=True)
+        shutil.copy(os.path.join(base, "config.json"), os.path.join(path, "config.json"))
+        tensors = load_file(os.path.join(base, "model.safetensors"))
+        for k in tensors:
+            if ".q_proj." in k or ".k_proj." in k:
+                tensors[k] = (tensors[k].float() * PEAKY_FACTOR).to(tensors[k].dtype)
+        save_file(tensors, os.path.join(path, "model.safetensors"))
+        tc.ALL.setdefault(name, tc.ALL[name[:-len(PEAKY)]])
+        return path
     llogos.write_random_model(path, tc.ALL[name], seed=seed)
     return path
 
@@ -57,15 +79,19 @@ def _bf16(x):
     return torch.from_numpy(np.ascontiguousarray(x)).to(torch.bfloat16).to(torch.float64).numpy()
 
 
-def forward_with_roundings(cfg, w, tokens, window=None, sinks=0):
-    """pm.forward with the bfloat16 engine's roundings put in: normed rows, rotated queries and
-    keys, values, probabilities (not their sum), the attention's output, gate and up,
-    silu(gate) * up.  Sums, softmax, norms and the residual stream stay in float64."""
+def with_roundings(run):
+    """run() with the bfloat16 engine's roundings put into the plain implementation's parts:
+    normed rows, rotated queries and keys, values, probabilities (not their sum), the
+    attention's output, gate and up, silu(gate) * up.  Sums, softmax, norms and the residual
+    stream stay in float64."""
     def attention(q, k, v, n_heads, n_kv_heads, head_dim, scale=None, window=0, sinks=0, positions=None):
         q, k, v = _bf16(q), _bf16(k), _bf16(v)
         T, group = q.shape[0], n_heads // n_kv_heads
-        pos = list(range(T)) if positions is None else list(positions)
-        seen = np.array([[pm.visible(pos[i], pos[j], window, sinks) for j in range(T)] for i in range(T)])
+        pos = np.arange(T) if positions is None else np.asarray(list(positions))
+        seen = pos[None, :] <= pos[:, None]
+        if window > 0:
+            seen &= (pos[None, :] < sinks) | (pos[None, :] > pos[:, None] - window)
+        assert seen[3 % T, 0] == pm.visible(int(pos[3 % T]), int(pos[0]), window, sinks)
         out = np.zeros((T, n_heads * head_dim))
         for h in range(n_heads):
             g = h // group
@@ -83,9 +109,13 @@ def forward_with_roundings(cfg, w, tokens, window=None, sinks=0):
     norm = pm.rms_norm
     pm.rms_norm, pm.attention, pm.swiglu_mlp = (lambda x, w_, eps: _bf16(norm(x, w_, eps))), attention, swiglu_mlp
     try:
-        return pm.forward(cfg, w, list(tokens), window=window, sinks=sinks)
+        return run()
     finally:
         pm.rms_norm, pm.attention, pm.swiglu_mlp = saved
+
+
+def forward_with_roundings(cfg, w, tokens, window=None, sinks=0):
+    return with_roundings(lambda: pm.forward(cfg, w, list(tokens), window=window, sinks=sinks))
 
 
 BOUND_LENGTHS = (150, 40, 17, 96)

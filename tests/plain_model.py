@@ -283,6 +283,30 @@ def forward(cfg: PlainConfig, w: dict, tokens, window: int | None = None, sinks:
     return linear(n, head)
 
 
+def forward_many(cfg: PlainConfig, get, sequences) -> list:
+    """forward() for several sequences of a model too large to hold in float64: `get(name)`
+    reads one tensor (float64) when it is needed, and a layer's tensors are read once for all
+    sequences.  The same functions in the same order as forward()."""
+    freqs = cfg.frequencies()
+    table = get("model.embed_tokens.weight")
+    xs = [embedding(table, t) for t in sequences]
+    names = ["input_layernorm.weight", "post_attention_layernorm.weight", "self_attn.q_proj.weight",
+             "self_attn.k_proj.weight", "self_attn.v_proj.weight", "self_attn.o_proj.weight", "mlp.gate_proj.weight",
+             "mlp.up_proj.weight", "mlp.down_proj.weight"]
+    if cfg.bias:
+        names += ["self_attn.q_proj.bias", "self_attn.k_proj.bias", "self_attn.v_proj.bias"]
+    if cfg.qk_norm:
+        names += ["self_attn.q_norm.weight", "self_attn.k_norm.weight"]
+    for i in range(cfg.n_layers):
+        p = f"model.layers.{i}."
+        w = {p + n: get(p + n) for n in names}
+        xs = [decoder_layer(cfg, w, i, x, list(range(len(t))), freqs) for x, t in zip(xs, sequences)]
+        del w
+    head = table if cfg.tied else get("lm_head.weight")
+    norm_w = get("model.norm.weight")
+    return [linear(rms_norm(x, norm_w, cfg.eps), head) for x in xs]
+
+
 # --------------------------------------------------------------------------
 # sampling
 # --------------------------------------------------------------------------

@@ -68,3 +68,35 @@ def test_random_subcommand_writes_a_model_folder(tmp_path, llogos):
     assert json.load(open(out / "config.json")) == tc.TINY_A
     assert cli.main(["random", "--config", str(tmp_path / "nope.json"), "--output-dir", str(out)]) == 1
     assert cli.main(["random", "--output-dir", str(out)]) == 1
+
+
+def test_a_library_built_from_other_sources_is_not_loaded(tmp_path, monkeypatch):
+    """A kernel library whose stamp does not match the sources is rebuilt before it is loaded,
+    and where that cannot be done loading raises; it is never loaded as it is."""
+    import importlib
+    library = importlib.import_module("daisi-llogos_amd.ops.library")
+    fake_dir = tmp_path / "_build"
+    fake_dir.mkdir()
+    (fake_dir / library.LIB_NAME).write_bytes(b"not a library")
+    (fake_dir / "sources.sha256").write_text("0" * 64)
+    monkeypatch.setattr(library, "build_dirs", lambda: [str(fake_dir)])
+    monkeypatch.setattr(library, "_PKG", str(tmp_path))
+    monkeypatch.setattr(library, "_lib", None)
+    monkeypatch.delenv("LLOGOS_KERNEL_LIBRARY", raising=False)
+    assert library.is_stale(str(fake_dir / library.LIB_NAME))
+    calls = []
+
+    def no_compiler():
+        calls.append(1)
+        raise library.KernelLibraryError("hipcc not found")
+    monkeypatch.setattr(library, "_hipcc", no_compiler)
+    import pytest
+    with pytest.raises(library.KernelLibraryError, match="stale and cannot be rebuilt"):
+        library.load()
+    assert calls == [1]
+    # a fresh stamp: found and taken as it is (loading these bytes then fails as a load error)
+    (fake_dir / "sources.sha256").write_text(library._source_hash())
+    assert not library.is_stale(str(fake_dir / library.LIB_NAME))
+    with pytest.raises(library.KernelLibraryError, match="cannot load"):
+        library.load()
+    assert calls == [1]

@@ -15,7 +15,7 @@ import tiny_configs as tc
 K = importlib.import_module("daisi-llogos_amd.ops.kernels")
 
 pytestmark = pytest.mark.gpu
-CONFIGS = ["tiny_a", "tiny_b", "tiny_c", "tiny_w", "tiny_d"]
+CONFIGS = ["tiny_a", "tiny_b", "tiny_c", "tiny_w", "tiny_d", "tiny_wd"]
 
 
 def _np(t):
@@ -124,7 +124,7 @@ def test_batch_composition_and_slot_do_not_change_float_results(dtype):
 
 
 @pytest.mark.parametrize("dtype", H.DTYPES)
-@pytest.mark.parametrize("name", ["tiny_c", "tiny_w", "tiny_d"])
+@pytest.mark.parametrize("name", ["tiny_c", "tiny_w", "tiny_d", "tiny_wd"])
 def test_long_decoding(name, dtype):
     """300 positions, most of them decoded one by one: crosses page borders, and in the
     windowed configuration pages leave the window and are given back meanwhile."""
@@ -136,7 +136,7 @@ def test_long_decoding(name, dtype):
     for t in toks[3:]:
         rows.append(_np(eng.step([(s, [t])], want="last")))
     H.close(np.concatenate(rows), want, dtype, f"{name} long decode", config=name)
-    if name == "tiny_w":
+    if name in ("tiny_w", "tiny_wd"):
         assert eng.cache.free_pages()[1] > eng.cache.free_pages()[0]           # the window group gave pages back
 
 
@@ -174,17 +174,105 @@ def test_first_tokens(name, dtype):
     H.close(got, want[[5, 2]], dtype, f"{name} wanted places", config=name)
 
 
-@pytest.mark.parametrize("name", ["tiny_a", "tiny_d"])
+@pytest.mark.parametrize("name", ["tiny_a", "tiny_d", "tiny_a_peaky", "tiny_d_peaky"])
 @pytest.mark.parametrize("dtype", H.DTYPES)
 def test_window_and_sinks_as_run_time_strategy(name, dtype):
+    """In the models with sharp attention a key too few or too many at the window's edge or among
+    the sinks moves the logits by far more than the bound, in bfloat16 too: the engine must lie
+    many times nearer to the windowed plain logits than those lie to windows that are off by one."""
+    H.folder(name)
     cfg, w = H.plain(name)
     toks = H.tokens(name, 100, 17)
     want = pm.forward(cfg, w, list(toks), window=24, sinks=3)
     eng = H.engine(name, dtype, attention_window=24, attention_sinks=3)
     s = eng.alloc_slot()
     rows = [_np(eng.step([(s, toks[:70])], want="all"))] + [_np(eng.step([(s, [t])])) for t in toks[70:]]
-    H.close(np.concatenate(rows), want, dtype, "window 24 sinks 3", config=name)
+    err = H.close(np.concatenate(rows), want, dtype, "window 24 sinks 3", config=name)
     assert np.abs(want - H.plain_logits(name, toks)).max() > 1e-3              # the window matters here
+    if name.endswith(H.PEAKY):
+        for other in (dict(window=23, sinks=3), dict(window=25, sinks=3), dict(window=24, sinks=2), dict(window=24, sinks=4),
+                      dict(window=0, sinks=0)):
+            off = np.abs(pm.forward(cfg, w, list(toks), **other) - want).max()
+            assert off > 4 * max(err, H.tol(dtype, name)), (other, off, err)
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+def test_matrix_core_attention_over_pages_that_were_given_back(dtype):
+    """Head size 64 with a configured window of 70 and no sinks: single tokens far beyond the
+    window and a prompt continued in a second and third portion after pages have left the
+    window.  Beside the logits, the host checks before every step that each page the step's
+    queries can see is still held (a page id of -1 there would be a read outside the pool)."""
+    name = "tiny_wd_peaky"
+    H.folder(name)
+    window = tc.ALL[name]["sliding_window"]
+    eng = H.engine(name, dtype, max_tokens=64 * 12, n_slots=2)
+    (g_win,) = [g for g in eng.cache.groups if g.spec.window]
+    assert g_win.spec.window == window and g_win.spec.sinks == 0 and g_win.spec.head_dim == 64
+
+    def step(entries, want):
+        for slot, new in entries:                    # every query of the step, every key it sees
+            start = eng.cache.length(slot)
+            pages = g_win.pages.seqs[slot].pages
+            for q in range(start, start + len(new)):
+                for page in range(max(0, q - window + 1) // 64, min(q, start - 1) // 64 + 1 if start else 0):
+                    assert pages[page] >= 0, f"position {q} sees page {page}, which was given back"
+        return _np(eng.step(entries, want=want))
+
+    a, b = H.tokens(name, 420, 61), H.tokens(name, 300, 62)
+    pa, pb = H.plain_logits(name, a), H.plain_logits(name, b)
+    sa, sb = eng.alloc_slot(), eng.alloc_slot()
+    got = step([(sa, a[:150]), (sb, b[:10])], want=[[149], [9]])
+    H.close(got, np.stack([pa[149], pb[9]]), dtype, "first portions", config=name)
+    assert g_win.pages.seqs[sa].pages[0] == -1                                  # a's first page has left the window
+    got = step([(sa, a[150:330]), (sb, [b[10]])], want=[[0, 50, 179], [0]])      # second portion over released pages
+    H.close(got, np.stack([pa[150], pa[200], pa[329], pb[10]]), dtype, "second portion", config=name)
+    assert g_win.pages.seqs[sa].pages[:3] == [-1, -1, -1]
+    rows_a, rows_b = [], []
+    for t in range(330, 330 + window + 8):                                       # single tokens past a whole window
+        got = step([(sa, [a[t]]), (sb, [b[t - 319]])], want="last")
+        rows_a.append(got[0]); rows_b.append(got[1])
+    H.close(np.stack(rows_a), pa[330:330 + window + 8], dtype, "single tokens, a", config=name)
+    H.close(np.stack(rows_b), pb[11:11 + window + 8], dtype, "single tokens, b", config=name)
+    got = step([(sb, b[11 + window + 8:300])], want=[[0, 300 - (11 + window + 8) - 1]])   # third portion, b alone
+    H.close(got, np.stack([pb[11 + window + 8], pb[299]]), dtype, "a long portion", config=name)
+    # in the sharp model an edge that is off by one would show
+    cfg, w = H.plain(name)
+    off = np.abs(pm.forward(cfg, w, list(a[:200]), window=window - 1)[199] - pa[199]).max()
+    assert off > 4 * H.tol(dtype, name), off
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+@pytest.mark.parametrize("name", ["tiny_c", "tiny_d_peaky"])
+def test_a_truncated_sequence_goes_on(name, dtype):
+    """A prompt of 150 positions, forgotten from position 70 on (the reference's SetLength,
+    Daisi.Llogos/Inference/IKvCache.cs:54; its use in tests/Daisi.Llogos.Tests/Inference/
+    ForwardPassTests.cs:90-103), then other tokens: the logits are those of the shortened
+    sequence followed by the new tokens, across the page border at 128, in a batch with a
+    sequence that was not cut; the pages beyond the cut went back to the pool."""
+    H.folder(name)
+    eng = H.engine(name, dtype, max_tokens=64 * 6, n_slots=2)
+    first, other = H.tokens(name, 150, 71), H.tokens(name, 100, 72)
+    new = H.tokens(name, 75, 73)
+    want = H.plain_logits(name, first[:70] + new)
+    po = H.plain_logits(name, other)
+    s, so = eng.alloc_slot(), eng.alloc_slot()
+    eng.step([(s, first), (so, other[:20])], want=None)
+    assert eng.cache.free_pages() == [2]
+    eng.cache.truncate(s, 70)
+    assert eng.cache.length(s) == 70 and eng.cache.free_pages() == [3]
+    got = _np(eng.step([(s, new[:6]), (so, other[20:22])], want="all"))          # a few tokens at once
+    H.close(got, np.concatenate([want[70:76], po[20:22]]), dtype, f"{name}: after the cut", config=name)
+    rows, rows_o = [], []
+    for i, t in enumerate(new[6:]):                                              # then one by one, past position 128
+        got = _np(eng.step([(s, [t]), (so, [other[22 + i]])], want="last"))
+        rows.append(got[0]); rows_o.append(got[1])
+    H.close(np.stack(rows), want[76:], dtype, f"{name}: tokens after the cut", config=name)
+    H.close(np.stack(rows_o), po[22:22 + len(rows_o)], dtype, f"{name}: the sequence beside it", config=name)
+    # the forgotten tokens matter: the uncut continuation gives other logits
+    assert np.abs(H.plain_logits(name, first + new)[150:156] - want[70:76]).max() > 3 * H.tol(dtype, name)
+    eng.cache.truncate(s, 0)                                                     # reset: the slot starts again
+    got = _np(eng.step([(s, other[:5])], want="all"))
+    H.close(got, po[:5], dtype, f"{name}: after a reset", config=name)
 
 
 @pytest.mark.parametrize("dtype", H.DTYPES)
@@ -249,11 +337,32 @@ def test_step_errors():
         eng.step([(s, [1, 2])], want=[[2]])
     with pytest.raises(H.llogos.CacheError):
         eng.step([(5, [1])])
-    with pytest.raises(H.llogos.CacheFull):
+    with pytest.raises(H.llogos.StepError, match="limit is 128"):          # max_position_embeddings of the configuration
         eng.step([(s, list(range(129)))])
+    s2 = eng.alloc_slot()
+    with pytest.raises(H.llogos.CacheFull):                                 # four pages wanted, the pool has two
+        eng.step([(s, list(range(100))), (s2, list(range(100)))])
+    eng.free_slot(s2)
     assert eng.cache.length(s) == 0 and eng.cache.free_pages() == [2]          # refused steps change nothing
     eng.step([(s, [1, 2, 3])])
     assert eng.cache.length(s) == 3
+
+
+def test_a_sequence_cannot_grow_beyond_the_limit():
+    """The engine's own limit (the command line's --max-context) within the model's positions:
+    the step that would cross it is refused as a whole and nothing changes."""
+    eng = H.engine("tiny_a", "float32", max_tokens=256, n_slots=2, max_seq=10)
+    assert eng.max_seq == 10
+    assert H.engine("tiny_a", "float32", max_tokens=256, n_slots=2, max_seq=1000).max_seq == 128
+    a, b = eng.alloc_slot(), eng.alloc_slot()
+    with pytest.raises(H.llogos.StepError, match="limit is 10"):
+        eng.step([(a, list(range(11)))])
+    eng.step([(a, list(range(10))), (b, [1, 2])])
+    with pytest.raises(H.llogos.StepError, match=r"sequence 0 \(slot %d\) would become 11" % a):
+        eng.step([(a, [5]), (b, [6])])
+    assert eng.cache.length(a) == 10 and eng.cache.length(b) == 2
+    eng.step([(b, [6])])
+    assert eng.cache.length(b) == 3
 
 
 @pytest.mark.parametrize("name", ["tiny_b", "tiny_w", "layer_14b"])
@@ -458,3 +567,56 @@ def test_greedy_generation_through_the_entry_point(name, dtype):
     cut = first.index(first[4])
     assert res2.tokens[0] == first[:cut] and res2.finish_reasons == ["stop"]
     assert llm.engine.cache.live_slots == []
+
+
+def test_the_library_rounds_a_batch_up_as_the_captured_steps_do():
+    """Where a kernel's shape depends on the batch (blocks along the context of the single-token
+    attention), the library takes the batch's class, the captured batch size that serves it, so
+    that a sequence's sums come in the same order alone and beside others of its class."""
+    graph = importlib.import_module("daisi-llogos_amd.engine.graph")
+    lib = importlib.import_module("daisi-llogos_amd.ops.library").load()
+    for b in range(1, 65):
+        assert lib.llogos_batch_class(b) == graph.bucket_batch(b)
+    assert lib.llogos_batch_class(65) == 128 and lib.llogos_page_tokens() == K.PAGE_TOKENS
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+def test_a_model_made_on_the_device_is_the_model_written_to_a_folder(dtype):
+    """Engine.from_config(config, seed) holds the weights that write_random_model(folder, config,
+    seed) writes: the same tensors, so the same logits bit for bit, and those of the plain
+    implementation reading the folder."""
+    name = "tiny_b"
+    a = H.engine(name, dtype)
+    b = H.llogos.Engine.from_config(tc.ALL[name], seed=11, dtype=dtype, max_tokens=2048, n_slots=4)
+    assert torch.equal(a.model.embed_table, b.model.embed_table)
+    for la, lb in zip(a.model.layers, b.model.layers):
+        assert torch.equal(la.mixer.qkv.weight, lb.mixer.qkv.weight) and torch.equal(la.ffn.down.weight, lb.ffn.down.weight)
+        assert torch.equal(la.mixer_norm.weight, lb.mixer_norm.weight) and torch.equal(la.mixer.q_norm_w, lb.mixer.q_norm_w)
+    toks = H.tokens(name, 50, 3)
+    outs = []
+    for eng in (a, b):
+        s = eng.alloc_slot()
+        outs.append(_np(eng.step([(s, toks)], want="all")))
+    assert np.array_equal(outs[0], outs[1])
+    H.close(outs[1], H.plain_logits(name, toks), dtype, "model made on the device", config=name)
+
+
+def test_benchmark_reports_bytes_and_flops_of_its_steps():
+    """Llogos.benchmark's roofline inputs for tiny_a, worked by hand: two layers of
+    qkv (128 x 64 + bias 128), o (64 x 64), gate/up (352 x 64), down (64 x 176), two norms (64 each), the
+    final norm and the head (256 x 64), float32."""
+    name = "tiny_a"
+    llm = H.llogos.Llogos(H.folder(name), dtype="float32", max_context=64, max_batch=2)
+    layer = (128 * 64 + 128) + 64 * 64 + 352 * 64 + 64 * 176 + 2 * 64
+    weights = (2 * layer + 64 + 256 * 64) * 4
+    assert llm.engine.model.step_weight_bytes() == weights
+    assert llm.engine.cache.bytes_per_position() == 2 * 2 * 2 * 16 * 4        # layers x (k, v) x kv heads x head size x bytes
+    prompts = [list(H.tokens(name, 10, 1)), list(H.tokens(name, 4, 2))]
+    r = llm.benchmark(prompts, 5)
+    assert (r.prompt_tokens, r.generated_tokens) == (14, 10)
+    # four decode steps of the batch of two: the weights four times, and positions 11..14 and 5..8 of the cache
+    assert r.decode_bytes == 4 * weights + 512 * (sum(range(11, 15)) + sum(range(5, 9)))
+    matrices = 2 * (128 * 64 + 64 * 64 + 352 * 64 + 64 * 176)
+    pairs = 10 * 11 / 2 + 4 * 5 / 2
+    assert r.prefill_flops == 2 * 14 * matrices + 2 * (4 * 4 * 16 * pairs) + 2 * 2 * 256 * 64
+    assert 0 < r.decode_fraction_of_peak < 1 and 0 < r.prefill_fraction_of_peak < 1 and r.dtype == "fp32"

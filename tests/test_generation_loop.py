@@ -207,3 +207,13 @@ def test_recent_tokens_are_the_tail_of_prompt_and_generated():
                                      ([1, 2, 3], [], 0), ([], [7], 3), ([1, 2, 3], [4, 5], 5), ([1, 2, 3], [4, 5], -1)):
         whole = prompt + generated
         assert gen.recent_tokens(prompt, generated, count) == (whole[-count:] if count > 0 else whole)
+
+
+def test_prevent_eos_refuses_more_stop_tokens_than_the_kernel_bans():
+    """Stop tokens beyond what one sampling call can ban are an error, not silently drawable."""
+    sampler_mod = importlib.import_module("daisi-llogos_amd.sampling.sampler")
+    params = GenerationParams(temperature=0.7, prevent_eos=True)
+    sampler_mod.Sampler(params, stop_tokens=range(64))
+    with pytest.raises(ValueError, match="at most 64"):
+        sampler_mod.Sampler(params, stop_tokens=range(65))
+    sampler_mod.Sampler(GenerationParams(temperature=0.7), stop_tokens=range(100))      # only stops, nothing to ban

@@ -584,3 +584,208 @@ def test_a_toy_feed_forward_with_routing_and_another_position_encoding(tmp_path)
         live = [i for i in range(3) if cut[i] + t < len(seqs[i])]
         out = _np(eng.step([(slots[i], [seqs[i][cut[i] + t]]) for i in live], want="last"))
         H.close(out, np.stack([want[i][cut[i] + t] for i in live]), "float32", f"routed token {t}")
+
+
+# ---------------------------------------------------------------------------
+# a toy block with two mixers side by side, a scaled embedding and capped logits, defined here
+# ---------------------------------------------------------------------------
+@P.register_block("toy_two_mixers")
+class TwoMixers(P.Block):
+    """x += pending; h = norm(x); x += mixer_0(h) + mixer_1(h); pending = ffn(ffn_norm(x)).
+    Each mixer has a cache of its own (keys and values for the one, fixed-size state for the other)."""
+
+    def __init__(self, norm, mixers, ffn_norm, ffn):
+        self.norm, self._mixers, self.ffn_norm, self.ffn = norm, list(mixers), ffn_norm, ffn
+
+    def mixers(self):
+        return self._mixers
+
+    def feed_forwards(self):
+        return [self.ffn]
+
+    def parts(self):
+        return [self.norm, *self._mixers, self.ffn_norm, self.ffn]
+
+    def forward(self, ctx, x, pending, caches):
+        h = self.norm.forward(x, pending)
+        a = self._mixers[0].forward(ctx, h, caches[0])
+        K.residual_add(x, K.sum_parts(a, None, torch.float32))
+        b = self._mixers[1].forward(ctx, h, caches[1])
+        return x, self.ffn.forward(ctx, self.ffn_norm.forward(x, b))
+
+
+@dataclasses.dataclass(frozen=True)
+class TwoMixerConfig:
+    vocab_size: int
+    hidden_size: int
+    n_layers: int
+    num_hidden_layers: int = 0
+    num_attention_heads: int = 2
+    num_key_value_heads: int = 1
+
+
+def _two_mixer_spec(cfg, **kw):
+    models = importlib.import_module("daisi-llogos_amd.models")
+    rot = P.Rotary(16, 16, 1e4)
+    norm = lambda name: ("norm", "rmsnorm", dict(name=name, width=cfg.hidden_size, eps=1e-6))
+    layers = []
+    for i in range(cfg.n_layers):
+        p = f"layers.{i}."
+        layers.append(models.LayerSpec(block="toy_two_mixers", more={
+            "norm": norm(p + "n1"),
+            "mixers": [("mixer", "attention", dict(prefix=p + "attn.", hidden=cfg.hidden_size, n_heads=2, n_kv_heads=1,
+                                                   head_dim=16, position=rot)),
+                       ("mixer", "toy_running_mean", dict(prefix=p, hidden=cfg.hidden_size))],
+            "ffn_norm": norm(p + "n2"),
+            "ffn": ("feed_forward", "swiglu", dict(prefix=p + "ffn.", hidden=cfg.hidden_size, intermediate=56))}))
+    return models.ModelSpec(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size, embed_name="embed.weight",
+                            layers=layers, final_norm=("rmsnorm", dict(name="norm", width=cfg.hidden_size, eps=1e-6)),
+                            head_name="head", tie_head=False, embed_scale=3.0, logit_scale=0.5, logit_softcap=2.0)
+
+
+L.register_architecture("ToyTwoMixersForCausalLM",
+                        lambda d: TwoMixerConfig(d["vocab_size"], d["hidden_size"], d["n_layers"]), _two_mixer_spec)
+
+
+def _plain_two_mixers(w, tokens, n_layers):
+    T = len(tokens)
+    x = 3.0 * pm.embedding(w["embed.weight"], tokens)
+    f = pm.rope_frequencies(16, 1e4)
+    for i in range(n_layers):
+        p = f"layers.{i}."
+        n = pm.rms_norm(x, w[p + "n1.weight"], 1e-6)
+        q = pm.rope_split_half(pm.linear(n, w[p + "attn.q_proj.weight"]), range(T), 2, 16, f)
+        k = pm.rope_split_half(pm.linear(n, w[p + "attn.k_proj.weight"]), range(T), 1, 16, f)
+        a = pm.linear(pm.attention(q, k, pm.linear(n, w[p + "attn.v_proj.weight"]), 2, 1, 16), w[p + "attn.o_proj.weight"])
+        b = pm.linear(np.cumsum(n, axis=0) / np.arange(1, T + 1)[:, None], w[p + "mix.weight"])
+        x = x + a + b
+        n = pm.rms_norm(x, w[p + "n2.weight"], 1e-6)
+        x = x + pm.swiglu_mlp(n, w[p + "ffn.gate_proj.weight"], w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
+    logits = 0.5 * pm.linear(pm.rms_norm(x, w["norm.weight"], 1e-6), w["head.weight"])
+    return 2.0 * np.tanh(logits / 2.0)
+
+
+def test_a_toy_block_with_two_mixers_and_scaled_embedding_and_logits(tmp_path):
+    """A block that holds two mixers (attention with keys and values, a running mean with
+    fixed-size state), an embedding scale and scaled, capped logits: registered here, built
+    from a model description and stepped whole, in an unequal batch and token by token."""
+    from safetensors.torch import load_file
+    cfg = {"architectures": ["ToyTwoMixersForCausalLM"], "vocab_size": 80, "hidden_size": 40, "n_layers": 2,
+           "torch_dtype": "float32"}
+    folder = L.write_random_model(str(tmp_path / "two"), cfg, seed=6)
+    w = {k: v.double().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    w["head.weight"] *= 40.0                                            # logits large enough for the cap to bend them
+    eng = L.Engine.from_folder(folder, dtype="float32", max_tokens=512, n_slots=3)
+    eng.model.head.weight.mul_(40.0)
+    needs = eng.model.cache_needs()
+    assert [(kv is not None, st is not None) for kv, st in needs] == [(True, False), (False, True)] * 2
+    assert eng.model.entry_units == [[0, 1], [2, 3]] and eng.graphs is None      # the running mean reads host lists
+    rng = np.random.default_rng(2)
+    seqs = [rng.integers(0, 80, size=n).tolist() for n in (70, 5, 33)]
+    want = [_plain_two_mixers(w, s, 2) for s in seqs]
+    assert np.abs(want[0]).max() > 1.5 and np.abs(want[0]).max() < 2.0          # the cap is at work
+    slot = eng.alloc_slot()
+    H.close(_np(eng.step([(slot, seqs[0])], want="all")), want[0], "float32", "two mixers whole")
+    eng.free_slot(slot)
+    slots = [eng.alloc_slot() for _ in seqs]
+    cut = [66, 2, 30]
+    out = _np(eng.step([(sl, s[:c]) for sl, s, c in zip(slots, seqs, cut)], want="all"))
+    H.close(out, np.concatenate([wnt[:c] for wnt, c in zip(want, cut)]), "float32", "two mixers, unequal batch")
+    for t in range(3):
+        out = _np(eng.step([(slots[i], [seqs[i][cut[i] + t]]) for i in range(3)], want="last"))
+        H.close(out, np.stack([want[i][cut[i] + t] for i in range(3)]), "float32", f"two mixers, token {t}")
+
+
+# ---------------------------------------------------------------------------
+# a toy mixer with state whose single-token steps are captured and replayed
+# ---------------------------------------------------------------------------
+@P.register_mixer("toy_running_mean_on_device")
+class RunningMeanOnDevice(P.Mixer):
+    """out_t = g * mean(h_0 .. h_t) with a weight vector g; single-token steps read and write
+    the state through the step's device tensors alone, so they may be captured."""
+    graph_safe = True
+
+    def __init__(self, prefix, hidden):
+        self.prefix, self.hidden = prefix, hidden
+
+    def tensor_specs(self):
+        return [P.TensorSpec(self.prefix + "gain.weight", (self.hidden,), "norm")]
+
+    def state_spec(self):
+        return P.StateSpec((self.hidden,), torch.float32)
+
+    def bind(self, get, rt):
+        self.rt = rt
+        self.g = get(self.prefix + "gain.weight").to(device=rt.device, dtype=torch.float32)
+
+    def forward(self, ctx, h, cache):
+        if ctx.is_decode:
+            slots = ctx.slots.long()
+            run = cache.state.index_select(0, slots) + h.float()
+            cache.state.index_copy_(0, slots, run)
+            return (run / (ctx.tok_pos + 1).float()[:, None] * self.g).to(h.dtype)
+        out = torch.empty_like(h)
+        for b in range(ctx.batch):
+            lo, hi = ctx.cu_seqlens[b], ctx.cu_seqlens[b + 1]
+            run = torch.cumsum(h[lo:hi].float(), 0) + cache.state[ctx.slot_ids[b]]
+            cache.state[ctx.slot_ids[b]] = run[-1]
+            count = torch.arange(ctx.starts[b] + 1, ctx.starts[b] + hi - lo + 1, device=h.device)[:, None]
+            out[lo:hi] = (run / count * self.g).to(h.dtype)
+        return out
+
+
+def _state_graph_spec(cfg, **kw):
+    models = importlib.import_module("daisi-llogos_amd.models")
+    layers = []
+    for i in range(cfg.n_layers):
+        p = f"layers.{i}."
+        layers.append(models.LayerSpec(
+            mixer=("toy_running_mean_on_device", dict(prefix=p, hidden=cfg.hidden_size)),
+            ffn=("swiglu", dict(prefix=p + "ffn.", hidden=cfg.hidden_size, intermediate=56)),
+            mixer_norm=("rmsnorm", dict(name=p + "n1", width=cfg.hidden_size, eps=1e-6)),
+            ffn_norm=("rmsnorm", dict(name=p + "n2", width=cfg.hidden_size, eps=1e-6))))
+    return models.ModelSpec(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size, embed_name="embed.weight",
+                            layers=layers, final_norm=("rmsnorm", dict(name="norm", width=cfg.hidden_size, eps=1e-6)),
+                            head_name="head", tie_head=False)
+
+
+L.register_architecture("ToyStateOnDeviceForCausalLM",
+                        lambda d: ToyConfig(d["vocab_size"], d["hidden_size"], d["n_layers"]), _state_graph_spec)
+
+
+def test_captured_steps_of_a_mixer_with_state_advance_the_state_once(tmp_path):
+    """A captured step is run once for real before its capture and then replayed: fixed-size
+    state must come out advanced once, not twice.  Replayed steps against the same steps launched
+    kernel by kernel, bit for bit, through several batch sizes (each a new capture), and against
+    the plain running mean."""
+    from safetensors.torch import load_file
+    cfg = {"architectures": ["ToyStateOnDeviceForCausalLM"], "vocab_size": 60, "hidden_size": 40, "n_layers": 2,
+           "torch_dtype": "float32"}
+    folder = L.write_random_model(str(tmp_path / "state"), cfg, seed=9)
+    w = {k: v.double().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+
+    def plain(tokens):
+        x = pm.embedding(w["embed.weight"], tokens)
+        for i in range(2):
+            p = f"layers.{i}."
+            n = pm.rms_norm(x, w[p + "n1.weight"], 1e-6)
+            x = x + np.cumsum(n, axis=0) / np.arange(1, len(tokens) + 1)[:, None] * w[p + "gain.weight"]
+            n = pm.rms_norm(x, w[p + "n2.weight"], 1e-6)
+            x = x + pm.swiglu_mlp(n, w[p + "ffn.gate_proj.weight"], w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
+        return pm.linear(pm.rms_norm(x, w["norm.weight"], 1e-6), w["head.weight"])
+
+    engines = [L.Engine.from_folder(folder, dtype="float32", max_tokens=512, n_slots=4, use_graphs=g) for g in (True, False)]
+    assert engines[0].graphs is not None and engines[1].graphs is None
+    rng = np.random.default_rng(4)
+    seqs = [rng.integers(0, 60, size=n).tolist() for n in (30, 12, 25)]
+    want = [plain(s) for s in seqs]
+    cut = [9, 2, 5]
+    slots = [[e.alloc_slot() for _ in seqs] for e in engines]
+    for e, sl in zip(engines, slots):
+        e.step([(s, q[:c]) for s, q, c in zip(sl, seqs, cut)], want=None)
+    for t in range(10):
+        live = [i for i in range(3) if cut[i] + t < len(seqs[i]) and (i != 1 or t < 4)]     # the batch shrinks: 3, then 2
+        outs = [_np(e.step([(sl[i], [seqs[i][cut[i] + t]]) for i in live], want="last")) for e, sl in zip(engines, slots)]
+        assert np.array_equal(outs[0], outs[1]), f"token {t}: replayed and launched steps differ by {np.abs(outs[0] - outs[1]).max()}"
+        H.close(outs[0], np.stack([want[i][cut[i] + t] for i in live]), "float32", f"state on device, token {t}")
+    assert len(engines[0].graphs.graphs) == 2

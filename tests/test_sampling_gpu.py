@@ -117,6 +117,31 @@ def test_prevent_eos_and_sampled_generation():
     assert len(b) == 8 and banned not in b
 
 
+def test_more_than_eight_banned_ids():
+    """Twelve stop tokens that may not be drawn: the twelve largest logits of every row are
+    theirs, the thirteenth must win (greedy) and no banned id is ever sampled."""
+    rng = np.random.default_rng(8)
+    V, R = 500, 5
+    logits = rng.standard_normal((R, V)).astype(np.float32)
+    banned = [int(t) for t in rng.choice(V, 12, replace=False)]
+    logits[:, banned] += 20.0
+    dev = torch.tensor(logits, device="cuda:0")
+    K = importlib.import_module("daisi-llogos_amd.ops.kernels")
+    work = K.sample_prepare(dev, None, None, 1.0, 0.0, 0.0, 1.0, False, banned).cpu().numpy()
+    assert np.isneginf(work[:, banned]).all()
+    keep = np.ones(V, bool); keep[banned] = False
+    assert np.array_equal(work[:, keep], logits[:, keep])
+    assert np.array_equal(K.argmax(torch.tensor(work, device="cuda:0")).cpu().numpy(),
+                          np.where(keep, logits, -np.inf).argmax(1))
+    with pytest.raises(K.KernelError, match="at most 64"):
+        K.sample_prepare(dev, None, None, 1.0, 0.0, 0.0, 1.0, False, list(range(65)))
+    params = S.GenerationParams(temperature=0.9, top_k=0, top_p=1.0, repetition_penalty=1.0, seed=3, prevent_eos=True)
+    sampler = S.Sampler(params, stop_tokens=banned)
+    for i in range(20):
+        drawn = sampler.sample(dev, list(range(R)), [i] * R).cpu().numpy()
+        assert not set(drawn.tolist()) & set(banned)
+
+
 def test_sampled_generation_draws_what_the_plain_sampler_draws():
     """Three prompts of 40 / 3 / 9 tokens, 24 new tokens each at temperature 0.8 with a fixed
     seed, in float32: along the engine's own token history, every token is the one the plain

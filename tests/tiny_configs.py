@@ -28,7 +28,7 @@ TINY_C = {   # Llama style: llama3 rotary scaling, head_dim 48, odd sizes, 5 hea
 TINY_W = {   # Qwen2 style with a sliding window in the upper layers
     "architectures": ["Qwen2ForCausalLM"], "vocab_size": 200, "hidden_size": 48, "intermediate_size": 80,
     "num_hidden_layers": 3, "num_attention_heads": 3, "num_key_value_heads": 1, "head_dim": 16,
-    "rms_norm_eps": 1e-6, "rope_theta": 10000.0, "max_position_embeddings": 512,
+    "rms_norm_eps": 1e-6, "rope_theta": 10000.0, "max_position_embeddings": 4096,
     "use_sliding_window": True, "sliding_window": 70, "max_window_layers": 1,
     "tie_word_embeddings": False, "torch_dtype": "bfloat16", "eos_token_id": 199,
 }
@@ -36,8 +36,17 @@ TINY_W = {   # Qwen2 style with a sliding window in the upper layers
 TINY_D = {   # Llama style with head size 64 and window: the matrix-core attention path
     "architectures": ["LlamaForCausalLM"], "vocab_size": 300, "hidden_size": 120, "intermediate_size": 200,
     "num_hidden_layers": 2, "num_attention_heads": 6, "num_key_value_heads": 2, "head_dim": 64,
-    "rms_norm_eps": 1e-5, "rope_theta": 10000.0, "max_position_embeddings": 512,
+    "rms_norm_eps": 1e-5, "rope_theta": 10000.0, "max_position_embeddings": 4096,
     "tie_word_embeddings": False, "torch_dtype": "bfloat16", "eos_token_id": 1,
+}
+
+TINY_WD = {  # Qwen2 style with head size 64 and a sliding window in the upper layer: the matrix-core attention
+             # over page tables with pages that were given back
+    "architectures": ["Qwen2ForCausalLM"], "vocab_size": 211, "hidden_size": 128, "intermediate_size": 152,
+    "num_hidden_layers": 2, "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 64,
+    "rms_norm_eps": 1e-6, "rope_theta": 10000.0, "max_position_embeddings": 4096,
+    "use_sliding_window": True, "sliding_window": 70, "max_window_layers": 1,
+    "tie_word_embeddings": False, "torch_dtype": "bfloat16", "eos_token_id": 210,
 }
 
 LAYER_8B = {   # two layers of the Llama-3.1-8B layer sizes with a small vocabulary: the kernels at real widths
@@ -56,4 +65,4 @@ LAYER_14B = {  # one layer of the Qwen3-14B layer sizes: widths that are no powe
     "tie_word_embeddings": False, "torch_dtype": "bfloat16", "eos_token_id": 2,
 }
 
-ALL = {"tiny_a": TINY_A, "tiny_b": TINY_B, "tiny_c": TINY_C, "tiny_w": TINY_W, "tiny_d": TINY_D, "layer_8b": LAYER_8B, "layer_14b": LAYER_14B}
+ALL = {"tiny_wd": TINY_WD, "tiny_a": TINY_A, "tiny_b": TINY_B, "tiny_c": TINY_C, "tiny_w": TINY_W, "tiny_d": TINY_D, "layer_8b": LAYER_8B, "layer_14b": LAYER_14B}
