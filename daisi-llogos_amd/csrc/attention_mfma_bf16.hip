@@ -20,6 +20,8 @@
 //  composite_ops.cu:275-512: tiles of keys with running maximum and sum, kv head = head /
 //  group, scale after the dot, query m of a prompt sees keys 0 .. start + m.)
 #include "common.h"
+#include "llogos_api.h"
+#include <mutex>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -888,6 +890,63 @@ LLOGOS_EXPORT int llogos_attn_decode_bf16(void* out, const void* q, int q_stride
     if ((q_stride % 8) || ((uintptr_t)q % 16)) return LLOGOS_UNSUPPORTED;
     return launch_decode(out, q, q_stride, nullptr, k_pool, v_pool, table, table_stride, table_width, tok_pos, batch,
                          n_heads, n_kv_heads, head_dim, scale, window, sinks, workspace, workspace_floats, stream);
+}
+
+// ---------------------------------------------------------------- decode without allocation
+// The decode attention for callers that cannot allocate (see llogos_api.h).  The partial
+// results of the blocks along the context, which llogos_attn_decode_bf16 takes in a workspace
+// from its caller, live in a file-scope device array here.  In host code the array's name is
+// only a stand-in for the symbol: its device address is asked for once per device, with that
+// device current, and that pointer is what the kernels, and anything else on the host, get.
+constexpr long long kStaticScratchFloats = 4ll << 20;                  // 16 MiB on each GPU the library runs on
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
+constexpr int kMaxDevices = 64;
+static float* scratch_ptr[kMaxDevices];                                // per device; null until asked for
+static std::mutex scratch_mutex;
+
+// The current device's copy of the array, through *ptr.
+static int static_scratch(float** ptr) {
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) return (int)e;
+    if (device < 0 || device >= kMaxDevices) return LLOGOS_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> hold(scratch_mutex);
+    if (scratch_ptr[device] == nullptr) {
+        float* p = nullptr;
+        e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (p == nullptr) return (int)hipErrorInvalidSymbol;
+        scratch_ptr[device] = p;
+    }
+    *ptr = scratch_ptr[device];
+    return 0;
+}
+
+LLOGOS_EXPORT long long llogos_attn_decode_static_capacity(void) { return kStaticScratchFloats; }
+
+LLOGOS_EXPORT int llogos_attn_decode_static_init(void) {
+    float* p = nullptr;
+    return static_scratch(&p);
+}
+
+LLOGOS_EXPORT int llogos_attn_decode_static_bf16(void* out, const void* q, int q_stride, const void* k_pool,
+                                                 const void* v_pool, const int* table, int table_stride,
+                                                 int table_width, const int* tok_pos, int batch, int n_heads,
+                                                 int n_kv_heads, int head_dim, float scale, int window, int sinks,
+                                                 hipStream_t stream) {
+    if ((q_stride % 8) || ((uintptr_t)q % 16)) return LLOGOS_UNSUPPORTED;
+    if (batch <= 0 || table_width <= 0) return LLOGOS_BAD_ARGUMENT;
+    if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim)) return LLOGOS_UNSUPPORTED;
+    // Nothing in the array has to start at zero: the merge kernel reads only the partial results
+    // that this call's blocks have written (blocks z < ceil(pages / pages per block) of each
+    // sequence), so what an earlier call left is never looked at.
+    const long long need = llogos_attn_decode_workspace(batch, n_heads, n_kv_heads, head_dim, table_width);
+    if (need > kStaticScratchFloats) return LLOGOS_TOO_LARGE;
+    float* ws = nullptr;
+    const int code = static_scratch(&ws);
+    if (code != 0) return code;
+    return launch_decode(out, q, q_stride, nullptr, k_pool, v_pool, table, table_stride, table_width, tok_pos, batch,
+                         n_heads, n_kv_heads, head_dim, scale, window, sinks, ws, kStaticScratchFloats, stream);
 }
 
 // The same from the fused projection (see QkvSource): head sizes 64 and 128; also writes the

@@ -10,7 +10,7 @@
 enum { DT_F32 = 0, DT_BF16 = 1 };
 
 // error codes returned by entry points (positive values are hipError_t)
-enum { LLOGOS_BAD_ARGUMENT = -1, LLOGOS_UNSUPPORTED = -2 };
+enum { LLOGOS_BAD_ARGUMENT = -1, LLOGOS_UNSUPPORTED = -2, LLOGOS_TOO_LARGE = -3 };
 
 constexpr int kWave = 64;        // CDNA wavefront
 constexpr int kPageTokens = 64;  // tokens per cache page

@@ -68,6 +68,8 @@ def _check(code: int, name: str) -> None:
             raise KernelError(f"{name}: bad argument")
         if code == -2:
             raise KernelError(f"{name}: size not supported")
+        if code == -3:
+            raise KernelError(f"{name}: larger than the library's fixed scratch array holds")
         raise KernelError(f"{name}: HIP error {code}")
 
 
