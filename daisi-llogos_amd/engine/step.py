@@ -47,6 +47,24 @@ def resolve_dtype(dtype: Union[str, torch.dtype]) -> torch.dtype:
         raise ValueError(f"dtype '{dtype}' is not supported (float32 or bfloat16)") from None
 
 
+def wants_packed_weights(model: Model, dtype: torch.dtype, max_tokens: int, device: torch.device) -> bool:
+    """Whether the bfloat16 matrices get their second, packed copy (the few-row products stream it
+    a quarter faster): when both copies and the cache fit the GPU with room to spare.  (The
+    Llama-3.1-70B sizes, 141 GB of matrices, do not: they run on the row-major copy alone.)"""
+    if dtype != torch.bfloat16:
+        return False
+    elements = 0
+    for spec in model.tensor_specs():
+        if spec.kind in ("matrix", "table"):
+            n = 1
+            for d in spec.shape:
+                n *= int(d)
+            elements += n
+    cache = max_tokens * sum(2 * kv.n_kv_heads * kv.head_dim * 2 for kv, _ in model.cache_needs() if kv is not None)
+    total = torch.cuda.get_device_properties(device).total_memory
+    return 2 * (2 * elements) + cache < 0.8 * total
+
+
 def require_gpu(device: Union[str, torch.device] = "cuda:0") -> torch.device:
     """The device the engine runs on.  There is no CPU path: without a GPU or without the
     kernel library this raises."""
@@ -81,9 +99,11 @@ class Engine:
     @classmethod
     def from_folder(cls, folder: str, dtype: Union[str, torch.dtype] = "bfloat16", max_tokens: int = 4096,
                     n_slots: int = 64, device: Union[str, torch.device] = "cuda:0",
-                    use_graphs: Optional[bool] = None, max_seq: Optional[int] = None, **spec_options) -> "Engine":
+                    use_graphs: Optional[bool] = None, max_seq: Optional[int] = None,
+                    pack_weights: Optional[bool] = None, **spec_options) -> "Engine":
         """config.json chooses the model class through the registry; model.safetensors is
-        checked against what the model needs before any tensor is read."""
+        checked against what the model needs before any tensor is read.  pack_weights: None
+        decides by the GPU's memory (wants_packed_weights)."""
         dev = require_gpu(device)
         data = read_config_json(folder)
         arch = architecture_of(data)
@@ -94,6 +114,7 @@ class Engine:
             tied = model.spec.head_name + ".weight" if model.spec.tie_head else None
             ckpt.check(model.tensor_specs(), tied_head=tied)
             rt = Runtime(dev, resolve_dtype(dtype))
+            rt.pack_weights = wants_packed_weights(model, rt.dtype, max_tokens, dev) if pack_weights is None else bool(pack_weights)
             with torch.cuda.device(dev):
                 model.bind(ckpt.get, rt)
                 torch.cuda.synchronize()
@@ -105,7 +126,7 @@ class Engine:
     def from_config(cls, config: dict, seed: int = 0, dtype: Union[str, torch.dtype] = "bfloat16",
                     max_tokens: int = 4096, n_slots: int = 64, device: Union[str, torch.device] = "cuda:0",
                     std: float = 0.02, use_graphs: Optional[bool] = None, max_seq: Optional[int] = None,
-                    **spec_options) -> "Engine":
+                    pack_weights: Optional[bool] = None, **spec_options) -> "Engine":
         """A model of the parsed config.json `config` with random weights made on the device,
         without a model folder: the weights that write_random_model(folder, config, seed) writes
         (matrices N(0, std), norm weights 1 + U(-0.1, 0.1)), stored in the configuration's
@@ -117,6 +138,7 @@ class Engine:
         model = Model(arch.model_spec(typed, **spec_options))
         specs = {s.name: s for s in model.tensor_specs()}
         rt = Runtime(dev, resolve_dtype(dtype))
+        rt.pack_weights = wants_packed_weights(model, rt.dtype, max_tokens, dev) if pack_weights is None else bool(pack_weights)
         store = storage_dtype(config)
 
         def get(name: str):

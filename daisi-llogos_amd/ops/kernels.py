@@ -549,8 +549,94 @@ def gemm_strips_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tens
     return out
 
 
+class PackedWeight:
+    """A bfloat16 matrix [N, K] in the order in which the matrix cores take it (pack_weights): blocks of
+    64 rows, steps of 32 values of k, one 16-byte fragment a lane, zero-padded.  The few-row
+    products stream it as one contiguous run per block."""
+    __slots__ = ("data", "N", "K")
+
+    def __init__(self, data: torch.Tensor, N: int, K: int):
+        self.data, self.N, self.K = data, N, K
+
+    def rows(self, n: int) -> Optional["PackedWeight"]:
+        """The first n rows as a packed matrix of their own (whole blocks of 64 rows only)."""
+        if n == self.N:
+            return self
+        if n <= 0 or n > self.N or n % 64:
+            return None
+        per_block = -(-self.K // 32) * 2048                  # bfloat16 elements of one block of rows
+        return PackedWeight(self.data[: (n // 64) * per_block], n, self.K)
+
+
+def pack_weights(w: torch.Tensor) -> PackedWeight:
+    """A packed copy of the bfloat16 matrix w [N, K]."""
+    _dev(w)
+    _need(w.dtype == torch.bfloat16 and w.dim() == 2, "pack_weights: w must be bfloat16 [N, K]")
+    N, K = w.shape
+    lib = _lib()
+    lib.llogos_packed_weight_bytes.restype = ctypes.c_longlong
+    data = torch.empty(lib.llogos_packed_weight_bytes(N, K) // 2, dtype=torch.bfloat16, device=w.device)
+    _check(lib.llogos_pack_weights(_p(data), _p(w), N, K, _stream()), "pack_weights")
+    return PackedWeight(data, N, K)
+
+
+def packed_plan(M: int, N: int, K: int) -> Tuple[int, int]:
+    """(blocks along k, values of k per LDS buffer) for the few-row product on packed weights: the
+    blocks along k as for the row-major form (the same trade of evenness, enough blocks and the
+    cost of partial sums, measured again on packed weights), and the shorter buffer for up to 16
+    rows, where it was 2 to 5 % faster.  One plan per class of row count (16, 32, 64)."""
+    return lds_splits(M, N, K), (128 if M <= 16 else 256)
+
+
+def gemm_packed_bf16(a: torch.Tensor, pw: PackedWeight, bias: Optional[torch.Tensor], out_dtype: torch.dtype,
+                     splits: int = 1, chunk: int = 256, swiglu: bool = False) -> Optional[torch.Tensor]:
+    """The few-row bfloat16 product on packed weights: [parts, M, N]; parts > 1 are float32 partial
+    sums over ranges of k that the consumer adds.  With `swiglu`, `a` is the fused gate/up product
+    ([M, 2 K] bfloat16 or float32 partial sums [parts, M, 2 K]) and silu(gate) * up is made on the
+    way.  None for shapes it does not take."""
+    if swiglu:
+        a_parts, a_stride = _parts(a)
+        M, K2 = a.shape[-2:]
+        K = K2 // 2
+        if a.dtype == torch.float32:
+            mode = 1
+        elif a.dtype == torch.bfloat16 and a_parts == 1:
+            mode = 2
+        else:
+            return None
+        lda = a.stride(-2)
+    else:
+        if a.dtype != torch.bfloat16 or a.dim() != 2:
+            return None
+        a_parts, a_stride, mode = 1, 0, 0
+        M, K = a.shape
+        lda = a.stride(0)
+    N = pw.N
+    if not (K == pw.K and 0 < M <= SKINNY_MAX_ROWS and K % 8 == 0 and a.stride(-1) == 1 and lda % 8 == 0
+            and a.data_ptr() % 16 == 0 and pw.data.data_ptr() % 16 == 0 and a_stride % 4 == 0):
+        return None
+    _dev(pw.data, bias)
+    _need(a.is_cuda and a.device == pw.data.device, "gemm: a and w must be on the same GPU")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.shape == (N,), "gemm: bias must be float32 [N]")
+    lib = _lib()
+    parts = lib.llogos_gemm_packed_parts(K, int(splits), int(chunk))
+    _need(parts >= 1, "gemm: the LDS buffer holds 128 or 256 values of k")
+    if parts > 1:
+        _need(bias is None, "gemm: a product in parts leaves the bias to its consumer")
+        out_dtype = torch.float32
+    out = torch.empty((parts, M, N), dtype=out_dtype, device=a.device)
+    code = lib.llogos_gemm_packed_bf16(
+        _p(out), _DT[out_dtype], _p(a), mode, lda, a_parts, ctypes.c_longlong(a_stride), _p(pw.data), _p(bias),
+        M, N, K, N, ctypes.c_longlong(M * N), int(splits), int(chunk), _stream())
+    if code == -2:
+        return None
+    _check(code, "gemm_packed_bf16")
+    return out
+
+
 def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swiglu_input: bool = False,
-                 f32_ok: bool = False) -> torch.Tensor:
+                 f32_ok: bool = False, packed: Optional[PackedWeight] = None) -> torch.Tensor:
     """a [M, K] . w [N, K]^T without bias, as [M, N] of `out_dtype` or as float32 partial sums
     [parts, M, N] for a consumer that adds them (rmsnorm, qk_rope_cache, swiglu, sum_parts).
     With `swiglu_input`, `a` is a fused gate/up product ([M, 2 K] or parts of it) and the
@@ -558,10 +644,23 @@ def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swigl
     [M, N], which spares the result a rounding to bfloat16.
 
     float32 operands: plain FMAs in 32-bit throughout.  bfloat16 operands: up to 64 rows the
-    hand-written weight-streaming kernels, up to 128 rows too where w is much longer than it
-    has rows (see long_inner); otherwise the library product (as the reference uses a library
-    for its prompt products, Daisi.Llogos.Cuda/CudaBackend.cs:158-316)."""
+    hand-written weight-streaming kernels (on the packed copy of w when there is one: `packed`),
+    up to 128 rows too where w is much longer than it has rows (see long_inner); otherwise the
+    library product (as the reference uses a library for its prompt products,
+    Daisi.Llogos.Cuda/CudaBackend.cs:158-316)."""
     M = a.shape[-2]
+    if packed is not None and w.dtype == torch.bfloat16 and M <= SKINNY_MAX_ROWS and out_dtype == torch.bfloat16:
+        splits, chunk = packed_plan(M, packed.N, packed.K)
+        src, fused = a, swiglu_input
+        # silu(gate) * up inside the product costs every block of rows of w a second read of the
+        # gate/up row: worth it for few rows in bfloat16, not for partial sums or many rows
+        if fused and not (M <= 16 and a.dtype == torch.bfloat16 and (a.dim() == 2 or a.shape[0] == 1)):
+            src, fused = swiglu(a, out_dtype), False
+        if not fused and src.dim() == 3 and src.shape[0] == 1:
+            src = src[0]
+        out = gemm_packed_bf16(src, packed, None, torch.float32 if f32_ok else out_dtype, splits, chunk, fused)
+        if out is not None:
+            return out
     if w.dtype == torch.bfloat16 and M <= SKINNY_MAX_ROWS and out_dtype == torch.bfloat16:
         few_dtype = torch.float32 if f32_ok else out_dtype              # what a product in one part is written as
         kernel, splits, row_blocks = skinny_plan(M, w.shape[0], w.shape[1])
@@ -607,10 +706,15 @@ def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swigl
     return gemm_generic(a, w, None, out_dtype)
 
 
-def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype) -> torch.Tensor:
+def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype,
+         packed: Optional[PackedWeight] = None) -> torch.Tensor:
     """a [M, K] . w [N, K]^T (+ bias [N]) -> one plain [M, N] tensor of `out_dtype`."""
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
         M = a.shape[0]
+        if packed is not None and M <= SKINNY_MAX_ROWS:
+            out = gemm_packed_bf16(a, packed, bias, out_dtype, 1, packed_plan(M, packed.N, packed.K)[1])
+            if out is not None:
+                return out[0]
         if M <= SKINNY_MAX_ROWS:
             kernel, _, row_blocks = skinny_plan(M, w.shape[0], w.shape[1])
             if kernel == "stationary":

@@ -29,6 +29,7 @@ class Runtime:
     """Where and in which element type a model computes."""
     device: torch.device
     dtype: torch.dtype                  # torch.float32 or torch.bfloat16: matrices, activations, cache
+    pack_weights: bool = True           # bfloat16 matrices get a second copy in the matrix cores' order (few-row products)
 
     @property
     def is_f32(self) -> bool:

@@ -23,6 +23,7 @@ class Linear(Part):
         self.has_bias = bias
         self.weight: Optional[torch.Tensor] = None
         self.bias: Optional[torch.Tensor] = None
+        self.packed: Optional[K.PackedWeight] = None     # the copy that steps of up to 64 rows stream
 
     @property
     def total_out(self) -> int:
@@ -40,6 +41,7 @@ class Linear(Part):
         super().bind(get, rt)
         mats = [get(n + ".weight") for n in self.names]
         self.weight = _to_device(mats, rt.dtype, rt.device)
+        self._pack(rt)
         if self.has_bias:
             self.bias = _to_device([get(n + ".bias") for n in self.names], torch.float32, rt.device)
 
@@ -50,6 +52,20 @@ class Linear(Part):
         """Use a matrix that another part already holds on the device (tied embeddings)."""
         self.rt = rt
         self.weight = weight
+        self._pack(rt)
+
+    def _pack(self, rt: Runtime) -> None:
+        self.packed = K.pack_weights(self.weight) if (rt.pack_weights and self.weight.dtype == torch.bfloat16) else None
+
+    def _packed_rows(self, rows_out: Optional[int]) -> Optional[K.PackedWeight]:
+        if self.packed is None or rows_out is None:
+            return self.packed
+        return self.packed.rows(rows_out)
+
+    def weight_bytes(self) -> int:
+        """What a step reads of this product: the matrix once (whichever copy) and the bias."""
+        total = self.weight.numel() * self.weight.element_size() if self.weight is not None else 0
+        return total + (self.bias.numel() * self.bias.element_size() if self.bias is not None else 0)
 
     def product(self, a: torch.Tensor, rows_out: Optional[int] = None, swiglu_input: bool = False,
                 f32_ok: bool = False) -> torch.Tensor:
@@ -58,7 +74,8 @@ class Linear(Part):
         fused gate/up product (maybe in parts) and W is applied to silu(gate) * up; with `f32_ok`
         the consumer also takes a float32 result."""
         w = self.weight if rows_out is None else self.weight[:rows_out]
-        return K.gemm_product(a, w, self.rt.dtype, swiglu_input=swiglu_input, f32_ok=f32_ok)
+        return K.gemm_product(a, w, self.rt.dtype, swiglu_input=swiglu_input, f32_ok=f32_ok,
+                              packed=self._packed_rows(rows_out))
 
     def bias_rows(self, rows_out: Optional[int] = None) -> Optional[torch.Tensor]:
         return self.bias if (self.bias is None or rows_out is None) else self.bias[:rows_out]
@@ -68,7 +85,7 @@ class Linear(Part):
         """a [M, in] -> [M, out]; `rows_out` uses only the first rows of the stacked matrix."""
         w = self.weight if rows_out is None else self.weight[:rows_out]
         b = self.bias if (self.bias is None or rows_out is None) else self.bias[:rows_out]
-        return K.gemm(a, w, b, out_dtype or self.rt.dtype)
+        return K.gemm(a, w, b, out_dtype or self.rt.dtype, packed=self._packed_rows(rows_out))
 
 
 def _to_device(parts: List[torch.Tensor], dtype: torch.dtype, device: torch.device) -> torch.Tensor:

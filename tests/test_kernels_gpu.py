@@ -530,3 +530,58 @@ def test_kernels_refuse_what_they_cannot_do():
         K.qk_rope_cache(torch.zeros(1, 3 * 1024, device=DEV), None, torch.float32, 1, 1, 1024, 2, 0, None, None, 1e-6,
                         torch.zeros(1, 1, 2, device=DEV), None, None, None,
                         torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV))
+
+
+@pytest.mark.parametrize("M,N,K_", [(1, 4096, 4096), (8, 331, 1000), (16, 100, 72), (17, 4096, 14336), (33, 257, 2048),
+                                    (64, 1000, 520), (48, 6144, 4096), (5, 64, 32), (64, 65, 8)])
+def test_gemm_on_packed_weights(M, N, K_):
+    """The few-row product on the packed copy of the weights (blocks of 64 rows, steps of 32 k,
+    zero-padded): every row count class, heights and lengths that fill no block or step, one part
+    and several, bias, float32 and bfloat16 results."""
+    rng = np.random.default_rng(M * 1000 + N)
+    a, w = _t(rng.standard_normal((M, K_)), torch.bfloat16), _t(rng.standard_normal((N, K_)) * 0.05, torch.bfloat16)
+    bias = _t(rng.standard_normal(N))
+    want = _np(a) @ _np(w).T
+    pw = K.pack_weights(w)
+    assert pw.N == N and pw.K == K_ and pw.data.numel() == -(-N // 64) * 64 * -(-K_ // 32) * 32
+    for chunk in (128, 256):
+        for splits in (1, 2, 5):
+            out = K.gemm_packed_bf16(a, pw, None, torch.float32, splits, chunk)
+            assert out is not None and out.dtype == torch.float32
+            _close(out.sum(0), want, "float32", scale=np.abs(want).max() * 10)        # bfloat16 operands, float32 sums
+        out = K.gemm_packed_bf16(a, pw, bias, torch.bfloat16, 1, chunk)
+        _close(out[0], want + _np(bias), "bfloat16")
+    # through the dispatch, as a part calls it
+    out = K.gemm_product(a, w, torch.bfloat16, f32_ok=True, packed=pw)
+    _close(K.sum_parts(out, None, torch.float32), want, "float32", scale=np.abs(want).max() * 10)
+    _close(K.gemm(a, w, bias, torch.float32, packed=pw), want + _np(bias), "float32", scale=np.abs(want).max() * 10)
+    # a row's result does not depend on the other rows of its class
+    if M > 1:
+        alone = K.gemm_packed_bf16(a[:1].contiguous(), pw, None, torch.float32, 1, 256)
+        if (M + 15) // 16 in (1,):
+            assert torch.equal(alone[0], K.gemm_packed_bf16(a, pw, None, torch.float32, 1, 256)[0][:1])
+
+
+def test_first_rows_of_packed_weights_and_the_fused_swiglu():
+    rng = np.random.default_rng(3)
+    I, H = 200, 136
+    w = _t(rng.standard_normal((192, H)) * 0.1, torch.bfloat16)
+    pw = K.pack_weights(w)
+    a = _t(rng.standard_normal((9, H)), torch.bfloat16)
+    first = pw.rows(128)
+    assert first is not None and first.N == 128 and pw.rows(100) is None and pw.rows(192) is pw
+    _close(K.gemm_packed_bf16(a, first, None, torch.float32, 1, 128)[0], (_np(a) @ _np(w).T)[:, :128], "float32", scale=50.0)
+    # down product of silu(gate) * up made on the way, from a bfloat16 row [gate | up] and from float32 partial sums
+    wd = _t(rng.standard_normal((H, I)) * 0.1, torch.bfloat16)
+    pd = K.pack_weights(wd)
+    gu = _t(rng.standard_normal((9, 2 * I)), torch.bfloat16)
+    g, u = _np(gu)[:, :I], _np(gu)[:, I:]
+    act = _np(_t(pm.silu(g) * u, torch.bfloat16))                     # the kernel rounds the product to bfloat16
+    want = act @ _np(wd).T
+    out = K.gemm_packed_bf16(gu, pd, None, torch.float32, 1, 128, swiglu=True)
+    _close(out[0], want, "bfloat16")
+    parts = _t(rng.standard_normal((3, 9, 2 * I)))
+    tot = _np(parts).sum(0)
+    want = _np(_t(pm.silu(tot[:, :I]) * tot[:, I:], torch.bfloat16)) @ _np(wd).T
+    out = K.gemm_packed_bf16(parts, pd, None, torch.float32, 2, 128, swiglu=True)
+    _close(out.sum(0), want, "bfloat16")
