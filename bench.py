@@ -107,7 +107,7 @@ def main(argv=None) -> int:
             bw = K.measure_read_bandwidth(n)
             print(f"[ceilings] read {label}: {bw / 1e12:.2f} TB/s ({bw / HBM_PEAK:.3f} of {HBM_PEAK / 1e12:g})", flush=True)
         rate = K.measure_mfma_rate()
-        print(f"[ceilings] mfma 16x16x32 bf16: {rate / 1e15:.3f} PFLOP/s ({rate / MFMA_PEAK['bf16']:.3f} of "
+        print(f"[ceilings] mfma bf16 (better of 16x16x32 and 32x32x16): {rate / 1e15:.3f} PFLOP/s ({rate / MFMA_PEAK['bf16']:.3f} of "
               f"{MFMA_PEAK['bf16'] / 1e15:g})", flush=True)
         return 0
 

@@ -47,12 +47,13 @@ def resolve_dtype(dtype: Union[str, torch.dtype]) -> torch.dtype:
         raise ValueError(f"dtype '{dtype}' is not supported (float32 or bfloat16)") from None
 
 
-def wants_packed_weights(model: Model, dtype: torch.dtype, max_tokens: int, device: torch.device) -> bool:
-    """Whether the bfloat16 matrices get their second, packed copy (the few-row products stream it
-    a quarter faster): when both copies and the cache fit the GPU with room to spare.  (The
-    Llama-3.1-70B sizes, 141 GB of matrices, do not: they run on the row-major copy alone.)"""
+def packed_weight_budget(model: Model, dtype: torch.dtype, max_tokens: int, device: torch.device) -> int:
+    """Bytes that the packed copies of the bfloat16 matrices may take (the few-row products stream
+    a packed copy a quarter faster; prompts need the row-major one): what is left of 85 % of the
+    GPU's memory beside the matrices themselves and the cache.  At the Llama-3.1-70B sizes, 141 GB
+    of matrices, about two thirds of the layers get their packed copy; smaller models all."""
     if dtype != torch.bfloat16:
-        return False
+        return 0
     elements = 0
     for spec in model.tensor_specs():
         if spec.kind in ("matrix", "table"):
@@ -62,7 +63,13 @@ def wants_packed_weights(model: Model, dtype: torch.dtype, max_tokens: int, devi
             elements += n
     cache = max_tokens * sum(2 * kv.n_kv_heads * kv.head_dim * 2 for kv, _ in model.cache_needs() if kv is not None)
     total = torch.cuda.get_device_properties(device).total_memory
-    return 2 * (2 * elements) + cache < 0.8 * total
+    return max(0, int(0.85 * total) - 2 * elements - cache)
+
+
+def _packing(rt: Runtime, model: Model, max_tokens: int, pack_weights: Optional[bool]) -> None:
+    """pack_weights None: packed copies as far as the GPU's memory allows; True: all; False: none."""
+    rt.pack_weights = pack_weights is not False and rt.dtype == torch.bfloat16
+    rt.pack_budget = packed_weight_budget(model, rt.dtype, max_tokens, rt.device) if pack_weights is None else None
 
 
 def require_gpu(device: Union[str, torch.device] = "cuda:0") -> torch.device:
@@ -103,7 +110,7 @@ class Engine:
                     pack_weights: Optional[bool] = None, **spec_options) -> "Engine":
         """config.json chooses the model class through the registry; model.safetensors is
         checked against what the model needs before any tensor is read.  pack_weights: None
-        decides by the GPU's memory (wants_packed_weights)."""
+        gives as many matrices a packed copy as the GPU's memory allows (packed_weight_budget)."""
         dev = require_gpu(device)
         data = read_config_json(folder)
         arch = architecture_of(data)
@@ -114,7 +121,7 @@ class Engine:
             tied = model.spec.head_name + ".weight" if model.spec.tie_head else None
             ckpt.check(model.tensor_specs(), tied_head=tied)
             rt = Runtime(dev, resolve_dtype(dtype))
-            rt.pack_weights = wants_packed_weights(model, rt.dtype, max_tokens, dev) if pack_weights is None else bool(pack_weights)
+            _packing(rt, model, max_tokens, pack_weights)
             with torch.cuda.device(dev):
                 model.bind(ckpt.get, rt)
                 torch.cuda.synchronize()
@@ -138,7 +145,7 @@ class Engine:
         model = Model(arch.model_spec(typed, **spec_options))
         specs = {s.name: s for s in model.tensor_specs()}
         rt = Runtime(dev, resolve_dtype(dtype))
-        rt.pack_weights = wants_packed_weights(model, rt.dtype, max_tokens, dev) if pack_weights is None else bool(pack_weights)
+        _packing(rt, model, max_tokens, pack_weights)
         store = storage_dtype(config)
 
         def get(name: str):

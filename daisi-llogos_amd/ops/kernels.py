@@ -568,15 +568,17 @@ class PackedWeight:
         return PackedWeight(self.data[: (n // 64) * per_block], n, self.K)
 
 
+def packed_weight_bytes(N: int, K: int) -> int:
+    return -(-N // 64) * -(-K // 32) * 4096
+
+
 def pack_weights(w: torch.Tensor) -> PackedWeight:
     """A packed copy of the bfloat16 matrix w [N, K]."""
     _dev(w)
     _need(w.dtype == torch.bfloat16 and w.dim() == 2, "pack_weights: w must be bfloat16 [N, K]")
     N, K = w.shape
-    lib = _lib()
-    lib.llogos_packed_weight_bytes.restype = ctypes.c_longlong
-    data = torch.empty(lib.llogos_packed_weight_bytes(N, K) // 2, dtype=torch.bfloat16, device=w.device)
-    _check(lib.llogos_pack_weights(_p(data), _p(w), N, K, _stream()), "pack_weights")
+    data = torch.empty(packed_weight_bytes(N, K) // 2, dtype=torch.bfloat16, device=w.device)
+    _check(_lib().llogos_pack_weights(_p(data), _p(w), N, K, _stream()), "pack_weights")
     return PackedWeight(data, N, K)
 
 
@@ -942,8 +944,8 @@ def sample_pipeline(work: torch.Tensor, uniforms: torch.Tensor, top_k: int, top_
 # ----------------------------------------------------------------------------
 def measure_read_bandwidth(n_bytes: int, repeats: int = 20, blocks_per_unit: int = 8, device="cuda:0") -> float:
     """Bytes a second at which a kernel that only reads streams `n_bytes` of device memory
-    (16-byte loads, four in flight per thread), best of `repeats` runs over a buffer that was
-    not the last thing read."""
+    (16-byte loads that do not stay in the caches, 32 KB of consecutive memory a block and round),
+    best of `repeats` runs over a buffer that was not the last thing read."""
     dev = torch.device(device)
     n_bytes = max(1 << 20, n_bytes // 16 * 16)
     with torch.cuda.device(dev):
@@ -964,18 +966,18 @@ def measure_read_bandwidth(n_bytes: int, repeats: int = 20, blocks_per_unit: int
 
 
 def measure_mfma_rate(iters: int = 20000, blocks_per_unit: int = 2, device="cuda:0") -> float:
-    """bfloat16 flops a second of v_mfma_f32_16x16x32_bf16 issued back to back by eight waves
-    on every compute unit (eight independent accumulators a wave)."""
+    """bfloat16 flops a second of MFMAs issued back to back by eight waves on every compute unit
+    (independent accumulators): the better of v_mfma_f32_16x16x32_bf16 and v_mfma_f32_32x32x16_bf16."""
     dev = torch.device(device)
     with torch.cuda.device(dev):
         blocks = compute_units(dev) * blocks_per_unit
         out = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
         lib, best = _lib(), 0.0
-        for _ in range(4):
+        for shape, per_iter in ((16, 8 * 16384.0), (32, 4 * 32768.0), (16, 8 * 16384.0), (32, 4 * 32768.0)):
             start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             start.record()
-            _check(lib.llogos_measure_mfma(_p(out), blocks, iters, _stream()), "measure_mfma")
+            _check(lib.llogos_measure_mfma(_p(out), blocks, iters, shape, _stream()), "measure_mfma")
             end.record()
             end.synchronize()
-            best = max(best, blocks * 4 * iters * 8 * 16384.0 / (start.elapsed_time(end) * 1e-3))
+            best = max(best, blocks * 4 * iters * per_iter / (start.elapsed_time(end) * 1e-3))
     return best

@@ -30,6 +30,7 @@ class Runtime:
     device: torch.device
     dtype: torch.dtype                  # torch.float32 or torch.bfloat16: matrices, activations, cache
     pack_weights: bool = True           # bfloat16 matrices get a second copy in the matrix cores' order (few-row products)
+    pack_budget: Optional[int] = None   # bytes that the packed copies may take together (None: no limit); bind() counts it down
 
     @property
     def is_f32(self) -> bool:

@@ -55,7 +55,16 @@ class Linear(Part):
         self._pack(rt)
 
     def _pack(self, rt: Runtime) -> None:
-        self.packed = K.pack_weights(self.weight) if (rt.pack_weights and self.weight.dtype == torch.bfloat16) else None
+        """The packed copy, if the runtime wants packed weights and its budget still holds this one."""
+        self.packed = None
+        if not (rt.pack_weights and self.weight.dtype == torch.bfloat16):
+            return
+        need = K.packed_weight_bytes(self.weight.shape[0], self.weight.shape[1])
+        if rt.pack_budget is not None:
+            if need > rt.pack_budget:
+                return
+            rt.pack_budget -= need
+        self.packed = K.pack_weights(self.weight)
 
     def _packed_rows(self, rows_out: Optional[int]) -> Optional[K.PackedWeight]:
         if self.packed is None or rows_out is None:
