@@ -93,7 +93,7 @@ __device__ __forceinline__ uint4 produce8(const ActSource& src, int m, int k, in
 
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
-template <int RB, int MB, int MODE, typename TO, int CHUNK, int WAVES = kLdsWaves, bool PACKED = false>
+template <int RB, int MB, int MODE, typename TO, int CHUNK, int WAVES = kLdsWaves, bool PACKED = false, bool GATED = false>
 __global__ __launch_bounds__(WAVES * kWave) void gemm_skinny_lds_kernel(
         TO* __restrict__ out, ActSource src, const bf16_t* __restrict__ w, const float* __restrict__ bias,
         int M, int N, int K, int ldo, size_t part_stride, int k_per_block, int parts) {
@@ -120,7 +120,9 @@ __global__ __launch_bounds__(WAVES * kWave) void gemm_skinny_lds_kernel(
         wrow[rb] = w + (size_t)min(n0 + rb * 16 + r, N - 1) * K + g * 8;
 
     // PACKED: w is [blocks of 16 * WAVES rows][steps of 32 k][wave][lane] 16-byte fragments, zero-padded
-    const u32x4* wpk = reinterpret_cast<const u32x4*>(w) + ((size_t)n_block * ((K + 31) / 32) * WAVES + wave) * kWave + lane;
+    // (packed blocks are 64 rows: a block of 8 waves takes two of them)
+    const u32x4* wpk = reinterpret_cast<const u32x4*>(w) +
+                       ((size_t)(n_block * (WAVES / 4) + wave / 4) * ((K + 31) / 32) * 4 + (wave & 3)) * kWave + lane;
 
     f32x4 acc[RB][MB];
 #pragma unroll
@@ -152,7 +154,7 @@ __global__ __launch_bounds__(WAVES * kWave) void gemm_skinny_lds_kernel(
         for (int s = 0; s < (CHUNK / 32); ++s) {
             if (PACKED) {
                 u32x4 v = {0, 0, 0, 0};
-                if (k0 + s * 32 < k_end) v = __builtin_nontemporal_load(wpk + (size_t)((k0 >> 5) + s) * (WAVES * kWave));
+                if (k0 + s * 32 < k_end) v = __builtin_nontemporal_load(wpk + (size_t)((k0 >> 5) + s) * (4 * kWave));
                 wf[s][0] = __builtin_bit_cast(bf16x8, v);
                 continue;
             }
@@ -200,6 +202,36 @@ __global__ __launch_bounds__(WAVES * kWave) void gemm_skinny_lds_kernel(
         __syncthreads();
     }
 
+    if (GATED) {
+        // The packed strips alternate between 16 gate rows and the 16 up rows of the same columns
+        // (llogos_pack_weights with gate_rows): waves 0 and 2 hold gate values, waves 1 and 3 the up
+        // values of the same (column, token) in the same lane and register.  The up waves hand
+        // theirs over through LDS, and out [M][N / 2] gets silu(gate) * up: the gate/up product
+        // never goes to memory.  One part only.
+        float* xch = reinterpret_cast<float*>(&lds[0][0][0]);
+        __syncthreads();                                             // the last chunk has been read
+        if (wave & 1) {
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) xch[(((wave >> 1) * MB + mb) * 4 + i) * kWave + lane] = acc[0][mb][i];
+        }
+        __syncthreads();
+        if (wave & 1) return;
+        const int col0 = (n_block * 2 + (wave >> 1)) * 16 + 4 * g;   // column of silu(gate) * up
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            const int m = mb * 16 + r;
+            if (m >= M) continue;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float gate = acc[0][mb][i], up = xch[(((wave >> 1) * MB + mb) * 4 + i) * kWave + lane];
+                const float y = gate * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * gate)) * up;
+                if (col0 + i < N / 2) store_f32(out + (size_t)m * ldo + col0 + i, y);
+            }
+        }
+        return;
+    }
     // acc[rb][mb][i] = sum for row n0 + rb * 16 + 4 g + i of w and activation row mb * 16 + r
     TO* dst = out + (size_t)split * part_stride;
 #pragma unroll
@@ -226,15 +258,15 @@ LLOGOS_EXPORT int llogos_gemm_skinny_lds_parts(int K, int splits) {
     return (K + kpb - 1) / kpb;
 }
 
-template <int RB, int MB, int MODE, int CHUNK = kChunkK, int WAVES = kLdsWaves, bool PACKED = false>
+template <int RB, int MB, int MODE, int CHUNK = kChunkK, int WAVES = kLdsWaves, bool PACKED = false, bool GATED = false>
 static int launch_lds(void* out, int out_dtype, const ActSource& src, const bf16_t* w, const float* bias,
                       int M, int N, int K, int ldo, size_t part_stride, int kpb, int parts, hipStream_t stream) {
     const int n_blocks = (N + 16 * RB * WAVES - 1) / (16 * RB * WAVES);
     if (out_dtype == DT_BF16)
-        gemm_skinny_lds_kernel<RB, MB, MODE, bf16_t, CHUNK, WAVES, PACKED><<<n_blocks * parts, WAVES * kWave, 0, stream>>>(
+        gemm_skinny_lds_kernel<RB, MB, MODE, bf16_t, CHUNK, WAVES, PACKED, GATED><<<n_blocks * parts, WAVES * kWave, 0, stream>>>(
             (bf16_t*)out, src, w, bias, M, N, K, ldo, part_stride, kpb, parts);
     else
-        gemm_skinny_lds_kernel<RB, MB, MODE, float, CHUNK, WAVES, PACKED><<<n_blocks * parts, WAVES * kWave, 0, stream>>>(
+        gemm_skinny_lds_kernel<RB, MB, MODE, float, CHUNK, WAVES, PACKED, GATED><<<n_blocks * parts, WAVES * kWave, 0, stream>>>(
             (float*)out, src, w, bias, M, N, K, ldo, part_stride, kpb, parts);
     return LLOGOS_LAUNCH_CHECK();
 }
@@ -283,14 +315,23 @@ LLOGOS_EXPORT int llogos_gemm_skinny_lds_bf16(void* out, int out_dtype, const vo
 
 // w [N][K] bf16 row-major -> packed [ceil(N / 64)][ceil(K / 32)][4][64] fragments of 8 bf16, zero-padded:
 // fragment (block, step, wave, lane) holds row 64 block + 16 wave + (lane & 15), k = 32 step + 8 (lane >> 4) .. + 7
-__global__ void pack_weights_kernel(uint4* __restrict__ dst, const bf16_t* __restrict__ src, int N, int K, long long pieces) {
+// gate_rows > 0: w is [gate (gate_rows rows); up (gate_rows rows)], gate_rows a multiple of 16, and the packed
+// strips alternate: strip 2 j holds gate rows 16 j .., strip 2 j + 1 the up rows 16 j .. (for the products
+// that make silu(gate) * up in their epilogue).
+__global__ void pack_weights_kernel(uint4* __restrict__ dst, const bf16_t* __restrict__ src, int N, int K, long long pieces,
+                                    int gate_rows) {
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= pieces) return;
     const int lane = (int)(i & 63), wave = (int)((i >> 6) & 3);
     const long long bs = i >> 8;
     const int steps = (K + 31) / 32;
     const int step = (int)(bs % steps), block = (int)(bs / steps);
-    const int n = block * 64 + wave * 16 + (lane & 15), k = step * 32 + (lane >> 4) * 8;
+    int n = block * 64 + wave * 16 + (lane & 15);
+    const int k = step * 32 + (lane >> 4) * 8;
+    if (gate_rows > 0) {
+        const int strip = n >> 4;
+        n = ((strip & 1) ? gate_rows : 0) + (strip >> 1) * 16 + (n & 15);
+    }
     bf16_t v[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] = (n < N && k + e < K) ? src[(size_t)n * K + k + e] : (bf16_t)0;
@@ -301,10 +342,11 @@ LLOGOS_EXPORT long long llogos_packed_weight_bytes(int N, int K) {
     return (long long)((N + 63) / 64) * ((K + 31) / 32) * 4096;
 }
 
-LLOGOS_EXPORT int llogos_pack_weights(void* dst, const void* src, int N, int K, hipStream_t stream) {
+LLOGOS_EXPORT int llogos_pack_weights(void* dst, const void* src, int N, int K, int gate_rows, hipStream_t stream) {
     if (N <= 0 || K <= 0 || dst == nullptr || src == nullptr) return LLOGOS_BAD_ARGUMENT;
+    if (gate_rows < 0 || (gate_rows > 0 && (gate_rows % 16 || N != 2 * gate_rows))) return LLOGOS_BAD_ARGUMENT;
     const long long pieces = llogos_packed_weight_bytes(N, K) / 16;
-    pack_weights_kernel<<<(unsigned)((pieces + 255) / 256), 256, 0, stream>>>((uint4*)dst, (const bf16_t*)src, N, K, pieces);
+    pack_weights_kernel<<<(unsigned)((pieces + 255) / 256), 256, 0, stream>>>((uint4*)dst, (const bf16_t*)src, N, K, pieces, gate_rows);
     return LLOGOS_LAUNCH_CHECK();
 }
 
@@ -353,5 +395,27 @@ LLOGOS_EXPORT int llogos_gemm_packed_bf16(void* out, int out_dtype, const void* 
     BY_ROWS(256);
 #undef BY_ROWS
 #undef BY_MODE
+#undef GO
+}
+
+// The same on a matrix packed with gate_rows (strips of gate and up rows in turn): out [M][ldo]
+// (ldo >= N / 2) = silu(a . gate^T) * (a . up^T) in bfloat16 or float32; plain activations, one
+// part, no bias.
+LLOGOS_EXPORT int llogos_gemm_packed_gated_bf16(void* out, int out_dtype, const void* act, int lda, const void* packed_w,
+                                                int M, int N, int K, int ldo, int chunk, hipStream_t stream) {
+    if (M <= 0 || N <= 0 || K <= 0 || (N % 32) || ldo < N / 2) return LLOGOS_BAD_ARGUMENT;
+    if (out_dtype != DT_BF16 && out_dtype != DT_F32) return LLOGOS_BAD_ARGUMENT;
+    if (chunk != 128 && chunk != 256) return LLOGOS_BAD_ARGUMENT;
+    if (M > 64 || (K % 8) || (lda % 8) || lda < K || ((uintptr_t)act % 16) || ((uintptr_t)packed_w % 16)) return LLOGOS_UNSUPPORTED;
+    const int kpb = packed_k_per_block(K, 1, chunk);
+    ActSource src{act, lda, 1, 0};
+    const bf16_t* W = (const bf16_t*)packed_w;
+    const int mb = (M + 15) / 16;
+#define GO(MB, CH) return launch_lds<1, MB, PRODUCE_PLAIN, CH, kLdsWaves, true, true>(out, out_dtype, src, W, nullptr, M, N, K, ldo, \
+                                                                                     0, kpb, 1, stream)
+#define BY_ROWS(CH) do { if (mb == 1) GO(1, CH); if (mb == 2) GO(2, CH); GO(4, CH); } while (0)
+    if (chunk == 128) BY_ROWS(128);
+    BY_ROWS(256);
+#undef BY_ROWS
 #undef GO
 }

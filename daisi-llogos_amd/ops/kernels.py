@@ -553,16 +553,18 @@ class PackedWeight:
     """A bfloat16 matrix [N, K] in the order in which the matrix cores take it (pack_weights): blocks of
     64 rows, steps of 32 values of k, one 16-byte fragment a lane, zero-padded.  The few-row
     products stream it as one contiguous run per block."""
-    __slots__ = ("data", "N", "K")
+    __slots__ = ("data", "N", "K", "gate_rows")
 
-    def __init__(self, data: torch.Tensor, N: int, K: int):
-        self.data, self.N, self.K = data, N, K
+    def __init__(self, data: torch.Tensor, N: int, K: int, gate_rows: int = 0):
+        # gate_rows > 0: w is [gate; up] of gate_rows rows each and the packed strips of 16 rows alternate
+        # between the two, for the product that makes silu(gate) * up in its epilogue (and for no other)
+        self.data, self.N, self.K, self.gate_rows = data, N, K, gate_rows
 
     def rows(self, n: int) -> Optional["PackedWeight"]:
         """The first n rows as a packed matrix of their own (whole blocks of 64 rows only)."""
         if n == self.N:
             return self
-        if n <= 0 or n > self.N or n % 64:
+        if n <= 0 or n > self.N or n % 64 or self.gate_rows:
             return None
         per_block = -(-self.K // 32) * 2048                  # bfloat16 elements of one block of rows
         return PackedWeight(self.data[: (n // 64) * per_block], n, self.K)
@@ -572,14 +574,37 @@ def packed_weight_bytes(N: int, K: int) -> int:
     return -(-N // 64) * -(-K // 32) * 4096
 
 
-def pack_weights(w: torch.Tensor) -> PackedWeight:
-    """A packed copy of the bfloat16 matrix w [N, K]."""
+def pack_weights(w: torch.Tensor, gate_rows: int = 0) -> PackedWeight:
+    """A packed copy of the bfloat16 matrix w [N, K].  gate_rows: w is a gate matrix on top of an up
+    matrix of gate_rows rows each (a multiple of 16), and strips of 16 gate rows and of the 16 up
+    rows of the same columns follow one another in the copy (see gemm_packed_gated_bf16)."""
     _dev(w)
     _need(w.dtype == torch.bfloat16 and w.dim() == 2, "pack_weights: w must be bfloat16 [N, K]")
     N, K = w.shape
+    _need(gate_rows == 0 or (gate_rows % 16 == 0 and N == 2 * gate_rows), "pack_weights: gate and up of a multiple of 16 rows each")
     data = torch.empty(packed_weight_bytes(N, K) // 2, dtype=torch.bfloat16, device=w.device)
-    _check(_lib().llogos_pack_weights(_p(data), _p(w), N, K, _stream()), "pack_weights")
-    return PackedWeight(data, N, K)
+    _check(_lib().llogos_pack_weights(_p(data), _p(w), N, K, int(gate_rows), _stream()), "pack_weights")
+    return PackedWeight(data, N, K, int(gate_rows))
+
+
+def gemm_packed_gated_bf16(a: torch.Tensor, pw: PackedWeight, out_dtype: torch.dtype, chunk: int = 256) -> Optional[torch.Tensor]:
+    """silu(a . gate^T) * (a . up^T) as [M, gate_rows] for up to 64 rows of bfloat16 activations, on a matrix
+    packed with gate_rows: the gate/up product stays in registers.  None for shapes it does not take."""
+    if pw.gate_rows <= 0 or a.dtype != torch.bfloat16 or a.dim() != 2:
+        return None
+    M, K = a.shape
+    if not (K == pw.K and 0 < M <= SKINNY_MAX_ROWS and K % 8 == 0 and a.stride(1) == 1 and a.stride(0) % 8 == 0
+            and a.data_ptr() % 16 == 0 and pw.data.data_ptr() % 16 == 0):
+        return None
+    _dev(pw.data)
+    _need(a.is_cuda and a.device == pw.data.device, "gemm: a and w must be on the same GPU")
+    out = torch.empty((M, pw.gate_rows), dtype=out_dtype, device=a.device)
+    code = _lib().llogos_gemm_packed_gated_bf16(_p(out), _DT[out_dtype], _p(a), a.stride(0), _p(pw.data), M, pw.N, K,
+                                                pw.gate_rows, int(chunk), _stream())
+    if code == -2:
+        return None
+    _check(code, "gemm_packed_gated_bf16")
+    return out
 
 
 def packed_plan(M: int, N: int, K: int) -> Tuple[int, int]:
@@ -651,6 +676,8 @@ def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swigl
     library product (as the reference uses a library for its prompt products,
     Daisi.Llogos.Cuda/CudaBackend.cs:158-316)."""
     M = a.shape[-2]
+    if packed is not None and packed.gate_rows:
+        packed = None                                       # its rows are in another order: only the gated product reads it
     if packed is not None and w.dtype == torch.bfloat16 and M <= SKINNY_MAX_ROWS and out_dtype == torch.bfloat16:
         splits, chunk = packed_plan(M, packed.N, packed.K)
         src, fused = a, swiglu_input
@@ -713,7 +740,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dty
     """a [M, K] . w [N, K]^T (+ bias [N]) -> one plain [M, N] tensor of `out_dtype`."""
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
         M = a.shape[0]
-        if packed is not None and M <= SKINNY_MAX_ROWS:
+        if packed is not None and not packed.gate_rows and M <= SKINNY_MAX_ROWS:
             out = gemm_packed_bf16(a, packed, bias, out_dtype, 1, packed_plan(M, packed.N, packed.K)[1])
             if out is not None:
                 return out[0]

@@ -16,7 +16,12 @@ class Linear(Part):
     the output row is the concatenation of their outputs."""
 
     def __init__(self, names: Sequence[str], in_features: int, out_features: Sequence[int],
-                 bias: bool = False, suffix: str = ".weight"):
+                 bias: bool = False, suffix: str = ".weight", gated: bool = False):
+        # gated: the two stacked matrices are a gate and an up projection whose product is only ever
+        # wanted as silu(gate) * up; their packed copy then serves the product that makes that in its
+        # epilogue (gated_product)
+        self.gated = bool(gated) and len(out_features) == 2 and out_features[0] == out_features[1] \
+            and out_features[0] % 16 == 0 and not bias
         self.names = list(names)
         self.in_features = in_features
         self.out_features = list(out_features)
@@ -64,7 +69,7 @@ class Linear(Part):
             if need > rt.pack_budget:
                 return
             rt.pack_budget -= need
-        self.packed = K.pack_weights(self.weight)
+        self.packed = K.pack_weights(self.weight, self.out_features[0] if self.gated else 0)
 
     def _packed_rows(self, rows_out: Optional[int]) -> Optional[K.PackedWeight]:
         if self.packed is None or rows_out is None:
@@ -85,6 +90,13 @@ class Linear(Part):
         w = self.weight if rows_out is None else self.weight[:rows_out]
         return K.gemm_product(a, w, self.rt.dtype, swiglu_input=swiglu_input, f32_ok=f32_ok,
                               packed=self._packed_rows(rows_out))
+
+    def gated_product(self, a: torch.Tensor) -> Optional[torch.Tensor]:
+        """silu(a . gate^T) * (a . up^T) as [M, out] in the runtime's type, made in one kernel from the
+        packed copy; None where that does not apply (no packed copy, more than 64 rows, float32)."""
+        if self.packed is None or not self.packed.gate_rows or a.dim() != 2 or a.shape[0] > K.SKINNY_MAX_ROWS:
+            return None
+        return K.gemm_packed_gated_bf16(a, self.packed, self.rt.dtype, K.packed_plan(a.shape[0], self.packed.N, self.packed.K)[1])
 
     def bias_rows(self, rows_out: Optional[int] = None) -> Optional[torch.Tensor]:
         return self.bias if (self.bias is None or rows_out is None) else self.bias[:rows_out]

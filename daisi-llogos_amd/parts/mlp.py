@@ -18,7 +18,7 @@ class SwiGLU(FeedForward):
     def __init__(self, prefix: str, hidden: int, intermediate: int):
         self.prefix = prefix
         self.hidden, self.intermediate = hidden, intermediate
-        self.gate_up = Linear([prefix + "gate_proj", prefix + "up_proj"], hidden, [intermediate, intermediate])
+        self.gate_up = Linear([prefix + "gate_proj", prefix + "up_proj"], hidden, [intermediate, intermediate], gated=True)
         self.down = Linear([prefix + "down_proj"], intermediate, [hidden])
 
     def tensor_specs(self) -> List[TensorSpec]:
@@ -30,7 +30,12 @@ class SwiGLU(FeedForward):
         self.down.bind(get, rt)
 
     def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
+        act = self.gate_up.gated_product(h)
+        if act is not None:
+            # up to 64 rows on packed weights: silu(gate) * up is the epilogue of the gate/up product
+            # (the reference's MatMulSwiGLU, Daisi.Llogos/IComputeBackend.cs:448-456)
+            return self.down.product(act, f32_ok=True)
         gu = self.gate_up.product(h)
-        # silu(gate) * up is made inside the down product where its kernel can (few rows), by a
-        # kernel of its own otherwise; the residual sum that follows adds the product's parts
+        # otherwise silu(gate) * up is made inside the down product where its kernel can (few rows), by a
+        # kernel of its own for many; the residual sum that follows adds the product's parts
         return self.down.product(gu, swiglu_input=True, f32_ok=True)

@@ -585,3 +585,27 @@ def test_first_rows_of_packed_weights_and_the_fused_swiglu():
     want = _np(_t(pm.silu(tot[:, :I]) * tot[:, I:], torch.bfloat16)) @ _np(wd).T
     out = K.gemm_packed_bf16(parts, pd, None, torch.float32, 2, 128, swiglu=True)
     _close(out.sum(0), want, "bfloat16")
+
+
+@pytest.mark.parametrize("M,I,H", [(1, 208, 136), (9, 14336, 4096), (16, 64, 72), (33, 1008, 264), (64, 2048, 520), (47, 16, 40)])
+def test_gate_up_product_with_the_swiglu_epilogue(M, I, H):
+    """The few-row product on a matrix packed as strips of gate rows and up rows in turn gives
+    silu(a gate^T) * (a up^T) directly; against the plain functions, every class of row count,
+    widths that fill no block."""
+    rng = np.random.default_rng(M + I)
+    wg, wu = (_t(rng.standard_normal((I, H)) * 0.08, torch.bfloat16) for _ in range(2))
+    a = _t(rng.standard_normal((M, H)), torch.bfloat16)
+    w = torch.cat([wg, wu]).contiguous()
+    pw = K.pack_weights(w, gate_rows=I)
+    assert pw.gate_rows == I and pw.rows(64) is None
+    want = pm.silu(_np(a) @ _np(wg).T) * (_np(a) @ _np(wu).T)
+    for chunk in (128, 256):
+        got = K.gemm_packed_gated_bf16(a, pw, torch.float32, chunk)
+        assert got is not None and got.shape == (M, I)
+        _close(got, want, "float32", scale=np.abs(want).max() * 50)           # hardware exp2 and reciprocal: about 1e-6 relative
+    _close(K.gemm_packed_gated_bf16(a, pw, torch.bfloat16, 256), want, "bfloat16")
+    # a packed copy in this order serves no other product: the dispatch leaves it aside
+    out = K.gemm_product(a, w, torch.bfloat16, packed=pw)
+    _close(K.sum_parts(out, None, torch.float32), _np(a) @ _np(w).T, "bfloat16")
+    with pytest.raises(K.KernelError):
+        K.pack_weights(w, gate_rows=I + 16)
