@@ -106,9 +106,12 @@ def main(argv=None) -> int:
                          ("o 34 MB", 4096 * 4096 * 2), ("1 GiB", 1 << 30), ("4 GiB", 1 << 32)):
             bw = K.measure_read_bandwidth(n)
             print(f"[ceilings] read {label}: {bw / 1e12:.2f} TB/s ({bw / HBM_PEAK:.3f} of {HBM_PEAK / 1e12:g})", flush=True)
-        rate = K.measure_mfma_rate()
-        print(f"[ceilings] mfma bf16 (better of 16x16x32 and 32x32x16): {rate / 1e15:.3f} PFLOP/s ({rate / MFMA_PEAK['bf16']:.3f} of "
-              f"{MFMA_PEAK['bf16'] / 1e15:g})", flush=True)
+        for shape in (16, 32):
+            for noisy in (False, True):
+                rate = K.measure_mfma_rate(shapes=(shape,), noisy=noisy)
+                print(f"[ceilings] mfma bf16 {'16x16x32' if shape == 16 else '32x32x16'}, "
+                      f"{'random operands' if noisy else 'constant operands'}: {rate / 1e15:.3f} PFLOP/s "
+                      f"({rate / MFMA_PEAK['bf16']:.3f} of {MFMA_PEAK['bf16'] / 1e15:g})", flush=True)
         return 0
 
     model_name, cfg = MODELS[args.model]

@@ -40,10 +40,22 @@ LLOGOS_EXPORT int llogos_measure_read(const void* src, long long bytes, int bloc
 
 // Each wave keeps eight independent accumulators and issues `iters` rounds of eight MFMAs
 // (2 * 16 * 16 * 32 flops each) on operands that never change.
-__global__ __launch_bounds__(256) void mfma_peak_kernel(float* __restrict__ out, int iters) {
+// noisy: operands of pseudo-random values in (-1, 1) (every bit of the mantissas toggles from lane to
+// lane, as in real data) instead of a few small constants: the matrix cores' rate depends on it,
+// the chip lowers its clock under the power of real data.
+__device__ __forceinline__ float measure_value(unsigned seed, int noisy) {
+    unsigned x = seed * 2654435761u + 12345u;
+    x ^= x >> 15; x *= 2246822519u; x ^= x >> 13;
+    return noisy ? ((float)(x & 0xffff) / 32768.0f - 1.0f) : 0.001f * (float)(seed % 7);
+}
+
+__global__ __launch_bounds__(256) void mfma_peak_kernel(float* __restrict__ out, int iters, int noisy) {
     bf16x8_m a, b;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) { a[i] = (__bf16)(0.001f * (float)(threadIdx.x % 7)); b[i] = (__bf16)(0.002f * (float)(threadIdx.x % 5)); }
+    for (int i = 0; i < 8; ++i) {
+        a[i] = (__bf16)measure_value(threadIdx.x * 16 + i, noisy);
+        b[i] = (__bf16)measure_value(threadIdx.x * 16 + 8 + i + blockIdx.x * 4096, noisy);
+    }
     f32x4_m acc[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = f32x4_m{0.f, 0.f, 0.f, 0.f};
@@ -60,10 +72,13 @@ __global__ __launch_bounds__(256) void mfma_peak_kernel(float* __restrict__ out,
 // The same with v_mfma_f32_32x32x16_bf16 (2 * 32 * 32 * 16 flops each, four accumulators of 16 floats).
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_m;
 
-__global__ __launch_bounds__(256) void mfma32_peak_kernel(float* __restrict__ out, int iters) {
+__global__ __launch_bounds__(256) void mfma32_peak_kernel(float* __restrict__ out, int iters, int noisy) {
     bf16x8_m a, b;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) { a[i] = (__bf16)(0.001f * (float)(threadIdx.x % 7)); b[i] = (__bf16)(0.002f * (float)(threadIdx.x % 5)); }
+    for (int i = 0; i < 8; ++i) {
+        a[i] = (__bf16)measure_value(threadIdx.x * 16 + i, noisy);
+        b[i] = (__bf16)measure_value(threadIdx.x * 16 + 8 + i + blockIdx.x * 4096, noisy);
+    }
     f32x16_m acc[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
@@ -81,9 +96,9 @@ __global__ __launch_bounds__(256) void mfma32_peak_kernel(float* __restrict__ ou
 
 // out: blocks * 256 floats.  shape 16: v_mfma_f32_16x16x32_bf16, flops = blocks * 4 waves * iters * 8 * 16384;
 // shape 32: v_mfma_f32_32x32x16_bf16, flops = blocks * 4 waves * iters * 4 * 32768.
-LLOGOS_EXPORT int llogos_measure_mfma(float* out, int blocks, int iters, int shape, hipStream_t stream) {
+LLOGOS_EXPORT int llogos_measure_mfma(float* out, int blocks, int iters, int shape, int noisy, hipStream_t stream) {
     if (out == nullptr || blocks <= 0 || iters <= 0 || (shape != 16 && shape != 32)) return LLOGOS_BAD_ARGUMENT;
-    if (shape == 16) mfma_peak_kernel<<<blocks, 256, 0, stream>>>(out, iters);
-    else mfma32_peak_kernel<<<blocks, 256, 0, stream>>>(out, iters);
+    if (shape == 16) mfma_peak_kernel<<<blocks, 256, 0, stream>>>(out, iters, noisy);
+    else mfma32_peak_kernel<<<blocks, 256, 0, stream>>>(out, iters, noisy);
     return LLOGOS_LAUNCH_CHECK();
 }

@@ -7,6 +7,7 @@ tensors used as device memory; launches go to torch's current stream.
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Optional, Sequence, Tuple
 
 import torch
@@ -662,6 +663,37 @@ def gemm_packed_bf16(a: torch.Tensor, pw: PackedWeight, bias: Optional[torch.Ten
     return out
 
 
+# Which product serves more than 64 rows of bfloat16 (prompts): "library" (the default: the library's
+# product on the row-major matrix, as the reference uses a library there) or "tiles" (gemm_tiles_bf16
+# on the packed copy: hand-written, with the SwiGLU epilogue, measured at two thirds of the library's
+# speed at the 8B sizes).  LLOGOS_PROMPT_PRODUCT in the environment sets the default.
+PROMPT_PRODUCT = os.environ.get("LLOGOS_PROMPT_PRODUCT", "library")
+
+
+def gemm_tiles_bf16(a: torch.Tensor, pw: PackedWeight, bias: Optional[torch.Tensor], out_dtype: torch.dtype) -> Optional[torch.Tensor]:
+    """a [M, K] . w^T on the packed copy of w for any number of rows (tiles of 128 tokens x 256 rows,
+    v_mfma_f32_32x32x16_bf16): [M, N] with the bias added, or, for a matrix packed with gate_rows,
+    [M, gate_rows] = silu(gate) * up.  None for shapes it does not take (K no multiple of 64)."""
+    if a.dtype != torch.bfloat16 or a.dim() != 2:
+        return None
+    M, K = a.shape
+    if not (K == pw.K and M > 0 and K % 64 == 0 and a.stride(1) == 1 and a.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0):
+        return None
+    gated = pw.gate_rows > 0
+    _dev(pw.data, bias)
+    _need(a.is_cuda and a.device == pw.data.device, "gemm: a and w must be on the same GPU")
+    _need(not (gated and bias is not None), "gemm: the gated product takes no bias")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.shape == (pw.N,), "gemm: bias must be float32 [N]")
+    out = torch.empty((M, pw.gate_rows if gated else pw.N), dtype=out_dtype, device=a.device)
+    code = _lib().llogos_gemm_tiles_bf16(_p(out), _DT[out_dtype], _p(a), a.stride(0), _p(pw.data), _p(bias), M, pw.N, K,
+                                         out.stride(0), int(gated), 4, _stream())
+    if code == -2:
+        return None
+    _check(code, "gemm_tiles_bf16")
+    return out
+
+
 def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swiglu_input: bool = False,
                  f32_ok: bool = False, packed: Optional[PackedWeight] = None) -> torch.Tensor:
     """a [M, K] . w [N, K]^T without bias, as [M, N] of `out_dtype` or as float32 partial sums
@@ -725,6 +757,10 @@ def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swigl
     if SKINNY_MAX_ROWS < M <= LDS_MAX_ROWS and long_inner(w) and a.dtype == torch.bfloat16 and out_dtype == torch.bfloat16:
         out = gemm_skinny_lds_bf16(a, w, None, torch.float32 if f32_ok else out_dtype,
                                    lds_splits(M, w.shape[0], w.shape[1]), 1)
+        if out is not None:
+            return out
+    if packed is not None and PROMPT_PRODUCT == "tiles" and M > SKINNY_MAX_ROWS and out_dtype == torch.bfloat16:
+        out = gemm_tiles_bf16(a, packed, None, torch.float32 if f32_ok else out_dtype)
         if out is not None:
             return out
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out_dtype == torch.bfloat16 and a.is_contiguous() \
@@ -992,18 +1028,22 @@ def measure_read_bandwidth(n_bytes: int, repeats: int = 20, blocks_per_unit: int
     return best
 
 
-def measure_mfma_rate(iters: int = 20000, blocks_per_unit: int = 2, device="cuda:0") -> float:
+def measure_mfma_rate(iters: int = 20000, blocks_per_unit: int = 2, device="cuda:0", noisy: bool = True,
+                      shapes=(16, 32)) -> float:
     """bfloat16 flops a second of MFMAs issued back to back by eight waves on every compute unit
-    (independent accumulators): the better of v_mfma_f32_16x16x32_bf16 and v_mfma_f32_32x32x16_bf16."""
+    (independent accumulators): the better of v_mfma_f32_16x16x32_bf16 and v_mfma_f32_32x32x16_bf16.
+    noisy: operands of random values, as real data is (the chip clocks lower under their power than
+    with the few small constants of noisy=False)."""
     dev = torch.device(device)
     with torch.cuda.device(dev):
         blocks = compute_units(dev) * blocks_per_unit
         out = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
         lib, best = _lib(), 0.0
-        for shape, per_iter in ((16, 8 * 16384.0), (32, 4 * 32768.0), (16, 8 * 16384.0), (32, 4 * 32768.0)):
+        for shape in tuple(shapes) * 2:
+            per_iter = 8 * 16384.0 if shape == 16 else 4 * 32768.0
             start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             start.record()
-            _check(lib.llogos_measure_mfma(_p(out), blocks, iters, shape, _stream()), "measure_mfma")
+            _check(lib.llogos_measure_mfma(_p(out), blocks, iters, shape, int(noisy), _stream()), "measure_mfma")
             end.record()
             end.synchronize()
             best = max(best, blocks * 4 * iters * per_iter / (start.elapsed_time(end) * 1e-3))

@@ -609,3 +609,43 @@ def test_gate_up_product_with_the_swiglu_epilogue(M, I, H):
     _close(K.sum_parts(out, None, torch.float32), _np(a) @ _np(w).T, "bfloat16")
     with pytest.raises(K.KernelError):
         K.pack_weights(w, gate_rows=I + 16)
+
+
+@pytest.mark.parametrize("M,N,K_", [(65, 256, 64), (300, 1000, 512), (2048, 4096, 4096), (129, 6144, 1024), (700, 130, 192)])
+def test_tiled_product_for_many_rows_on_packed_weights(M, N, K_):
+    """The hand-written prompt-size product (tiles of 128 tokens x 256 rows, 32x32x16 MFMAs on the
+    packed copy): token counts and heights that fill no tile, float32 and bfloat16 results, bias."""
+    rng = np.random.default_rng(M + N)
+    a, w = _t(rng.standard_normal((M, K_)), torch.bfloat16), _t(rng.standard_normal((N, K_)) * 0.05, torch.bfloat16)
+    bias = _t(rng.standard_normal(N))
+    want = _np(a) @ _np(w).T
+    pw = K.pack_weights(w)
+    _close(K.gemm_tiles_bf16(a, pw, None, torch.float32), want, "float32", scale=np.abs(want).max() * 10)
+    _close(K.gemm_tiles_bf16(a, pw, bias, torch.bfloat16), want + _np(bias), "bfloat16")
+    assert K.gemm_tiles_bf16(a[:, :K_ - 8].contiguous(), K.pack_weights(w[:, :K_ - 8].contiguous()), None, torch.float32) is None
+
+
+@pytest.mark.parametrize("M,I,H", [(200, 1008, 256), (2048, 14336, 4096), (65, 16, 64)])
+def test_tiled_product_with_the_swiglu_epilogue(M, I, H):
+    rng = np.random.default_rng(M + I)
+    wg, wu = (_t(rng.standard_normal((I, H)) * 0.08, torch.bfloat16) for _ in range(2))
+    a = _t(rng.standard_normal((M, H)) * (0.25 if H > 1000 else 1.0), torch.bfloat16)
+    pw = K.pack_weights(torch.cat([wg, wu]).contiguous(), gate_rows=I)
+    want = pm.silu(_np(a) @ _np(wg).T) * (_np(a) @ _np(wu).T)
+    got = K.gemm_tiles_bf16(a, pw, None, torch.float32)
+    assert got.shape == (M, I)
+    _close(got, want, "float32", scale=np.abs(want).max() * 50)
+    _close(K.gemm_tiles_bf16(a, pw, None, torch.bfloat16), want, "bfloat16")
+
+
+def test_prompts_through_the_tiled_product(monkeypatch):
+    """An engine whose prompt products are the hand-written ones gives the plain logits like the default."""
+    import gpu_helpers as H
+    monkeypatch.setattr(K, "PROMPT_PRODUCT", "tiles")
+    name = "layer_8b"
+    eng = H.engine(name, "bfloat16", max_tokens=64 * 8, n_slots=2)
+    assert eng.model.layers[0].ffn.gate_up.packed.gate_rows == 14336
+    toks = H.tokens(name, 150, 1)
+    s = eng.alloc_slot()
+    got = eng.step([(s, toks)], want="all").cpu().double().numpy()
+    H.close(got, H.plain_logits(name, toks), "bfloat16", "prompt through the tiled product", config=name)
