@@ -4,9 +4,10 @@
 //
 // One wave works on 16 "columns" and one page of 64 keys at a time:
 //   decode  (one token per sequence): the columns are the query heads of one kv head;
-//           a block of 4 waves takes 4 consecutive pages of one (sequence, kv head), the
-//           waves' running (max, sum, output) are merged through LDS, blocks along the
-//           context write partial results that a second small kernel merges;
+//           a block of 4 waves takes a run of pages of one (sequence, kv head), each wave
+//           every fourth of them in turn; the waves' running (max, sum, output) are merged
+//           through LDS, blocks along the context write partial results that a second small
+//           kernel merges;
 //   prefill (many tokens per sequence): the columns are 16 consecutive tokens of one
 //           sequence for one query head; each wave walks the pages up to its last row.
 // Scores are computed transposed, S^T[key][column] = K . Q^T, so that the lane that holds
@@ -21,6 +22,7 @@
 //  group, scale after the dot, query m of a prompt sees keys 0 .. start + m.)
 #include "common.h"
 #include "llogos_api.h"
+#include <algorithm>
 #include <mutex>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -151,34 +153,35 @@ __device__ __forceinline__ bool page_fully_visible(int first_pos, int last_pos, 
     return key0 + kPageTokens - 1 < sinks || key0 > last_pos - window;
 }
 
-// One page of 64 keys.  qf: the columns' queries as second operands (lane (c, g) holds
-// Q[c][32 s + 8 g ..]); kpage [64][HD], vpage [HD][64]; q_pos: position of this lane's column
-// (-1: the column is not in use); key0: position of the page's first key; valid_keys: how
-// many of the page's keys have been written (the rest of the page holds whatever was there
-// before: such scores are masked, and such values are zeroed because 0 * NaN is NaN).
+// The parts of a page's work, apart so that a kernel can ask for the next page's keys and values
+// while it works on this one's.  kpage [64][HD], vpage [HD][64] of one kv head.
 template <int HD>
-__device__ __forceinline__ void attend_page(WaveState<HD>& st, const bf16x8 (&qf)[HD / 32],
-                                            const bf16_t* __restrict__ kpage, const bf16_t* __restrict__ vpage,
-                                            int q_pos, int key0, int valid_keys, bool all_visible,
-                                            float scale_log2, int window, int sinks) {
+__device__ __forceinline__ void load_keys(bf16x8 (&kf)[4][HD / 32], const bf16_t* __restrict__ kpage) {
     const int lane = threadIdx.x & (kWave - 1);
     const int i = lane & 15, g = lane >> 4;
-    // all of the page's loads are issued before the first product
-    bf16x8 kf[4][HD / 32], vf[HD / 16][2];
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb) {
         const bf16_t* krow = kpage + (size_t)(16 * (i >> 2) + 4 * rb + (i & 3)) * HD + 8 * g;
 #pragma unroll
         for (int sk = 0; sk < HD / 32; ++sk) kf[rb][sk] = ld_frag(krow + 32 * sk);
     }
+}
+
+template <int HD>
+__device__ __forceinline__ void load_values(bf16x8 (&vf)[HD / 16][2], const bf16_t* __restrict__ vpage) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int i = lane & 15, g = lane >> 4;
 #pragma unroll
     for (int db = 0; db < HD / 16; ++db) {
         const bf16_t* vrow = vpage + (size_t)(16 * db + i) * kPageTokens + 16 * g;
         vf[db][0] = ld_frag(vrow);
         vf[db][1] = ld_frag(vrow + 8);
     }
-    // S^T = K . Q^T, four blocks of 16 keys; this lane: column i, keys key0 + 16 g + 4 rb + r
-    f32x4 s[4];
+}
+
+// S^T = K . Q^T, four blocks of 16 keys; this lane: column lane & 15, keys 16 g + 4 rb + r in s[rb][r]
+template <int HD>
+__device__ __forceinline__ void page_scores(f32x4 (&s)[4], const bf16x8 (&kf)[4][HD / 32], const bf16x8 (&qf)[HD / 32]) {
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb) {
         s[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -186,11 +189,14 @@ __device__ __forceinline__ void attend_page(WaveState<HD>& st, const bf16x8 (&qf
         for (int sk = 0; sk < HD / 32; ++sk)
             s[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[rb][sk], qf[sk], s[rb], 0, 0, 0);
     }
-    bf16x8 pf[2];
-    float corr;
-    if (all_visible) softmax_page<false, 16, 4, HD>(s, st, scale_log2, q_pos, key0, window, sinks, pf, corr);
-    else             softmax_page<true, 16, 4, HD>(s, st, scale_log2, q_pos, key0, window, sinks, pf, corr);
-    // O^T = O^T * corr + V^T . P^T; slot (g, e) of step t is key 16 g + 8 t + e
+}
+
+// O^T = O^T * corr + V^T . P^T; slot (g, e) of step t is key 16 g + 8 t + e.  Values of keys
+// that have not been written (valid_keys and on) are zeroed: 0 * NaN is NaN.
+template <int HD>
+__device__ __forceinline__ void weigh_values(WaveState<HD>& st, const bf16x8 (&vf)[HD / 16][2], const bf16x8 (&pf)[2],
+                                             float corr, int valid_keys) {
+    const int g = (threadIdx.x & (kWave - 1)) >> 4;
     const bool rescale = __ballot(corr != 1.0f) != 0;
 #pragma unroll
     for (int db = 0; db < HD / 16; ++db) {
@@ -210,6 +216,29 @@ __device__ __forceinline__ void attend_page(WaveState<HD>& st, const bf16x8 (&qf
     }
 }
 
+// One page of 64 keys.  qf: the columns' queries as second operands (lane (c, g) holds
+// Q[c][32 s + 8 g ..]); kpage [64][HD], vpage [HD][64]; q_pos: position of this lane's column
+// (-1: the column is not in use); key0: position of the page's first key; valid_keys: how
+// many of the page's keys have been written (the rest of the page holds whatever was there
+// before: such scores are masked, and such values are zeroed because 0 * NaN is NaN).
+template <int HD>
+__device__ __forceinline__ void attend_page(WaveState<HD>& st, const bf16x8 (&qf)[HD / 32],
+                                            const bf16_t* __restrict__ kpage, const bf16_t* __restrict__ vpage,
+                                            int q_pos, int key0, int valid_keys, bool all_visible,
+                                            float scale_log2, int window, int sinks) {
+    // all of the page's loads are issued before the first product
+    bf16x8 kf[4][HD / 32], vf[HD / 16][2];
+    load_keys<HD>(kf, kpage);
+    load_values<HD>(vf, vpage);
+    f32x4 s[4];
+    page_scores<HD>(s, kf, qf);
+    bf16x8 pf[2];
+    float corr;
+    if (all_visible) softmax_page<false, 16, 4, HD>(s, st, scale_log2, q_pos, key0, window, sinks, pf, corr);
+    else             softmax_page<true, 16, 4, HD>(s, st, scale_log2, q_pos, key0, window, sinks, pf, corr);
+    weigh_values<HD>(st, vf, pf, corr, valid_keys);
+}
+
 // Whether any key of the page [key0, key0 + 63] can be visible to a query at q_pos.
 __device__ __forceinline__ bool page_may_be_visible(int q_pos, int key0, int window, int sinks) {
     if (key0 > q_pos) return false;
@@ -227,10 +256,13 @@ __device__ __forceinline__ bool page_may_be_visible_to_range(int first_pos, int 
 }
 
 // ---------------------------------------------------------------- decode
-// grid (batch, kv heads, ceil(table width / WAVES)); block of WAVES waves, wave w takes page
-// WAVES z + w.  With one block along the context (gridDim.z == 1) the block writes the
-// attention output itself; otherwise partial: [batch][heads][grid.z][HD + 2] floats (max, sum,
-// unnormalised output) for the merge kernel.  Dynamic LDS: decode_lds_bytes(WAVES, group, HD).
+// grid (batch, kv heads, blocks along the context); a block of WAVES waves covers WAVES * ppw
+// consecutive pages, wave w taking pages w, w + WAVES, ... of them one after the other.  (Asking
+// for the next page's keys and values while a wave works on this one takes twice the registers
+// and was slower: what hides the latency is the other waves.)  With one block
+// along the context (gridDim.z == 1) the block writes the attention output itself; otherwise
+// partial: [batch][heads][grid.z][HD + 2] floats (max, sum, unnormalised output) for the merge
+// kernel.  Dynamic LDS: decode_lds_bytes(WAVES, group, HD).
 __host__ __device__ constexpr size_t decode_lds_bytes(int waves, int group, int hd) {
     return (size_t)waves * (group * (hd + 1) + 32) * sizeof(float);
 }
@@ -259,7 +291,7 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_decode_kernel(
         bf16_t* __restrict__ out, float* __restrict__ partial, const bf16_t* __restrict__ q, int q_stride,
         QkvSource src, const bf16_t* k_pool, const bf16_t* v_pool,
         const int* __restrict__ table, int table_stride, const int* __restrict__ tok_pos,
-        int n_heads, int n_kv_heads, int group, float scale, int window, int sinks) {
+        int n_heads, int n_kv_heads, int group, float scale, int window, int sinks, int ppw) {
     extern __shared__ float lds[];
     float* lds_m = lds;                                   // [WAVES][16]
     float* lds_l = lds + WAVES * 16;                      // [WAVES][16]
@@ -270,8 +302,19 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_decode_kernel(
     const int c = lane & 15, g = lane >> 4;
     const int pos = tok_pos[b];
     const int n_pages = pos / kPageTokens + 1;
-    if (z * WAVES >= n_pages) return;                            // nothing of this sequence here
-    const int page_idx = z * WAVES + wave;
+    const int first_page = z * WAVES * ppw;
+    if (first_page >= n_pages) return;                           // nothing of this sequence here
+    const int* row = table + (size_t)b * table_stride;
+
+    // this wave's pages: first_page + wave + WAVES j, j < ppw, as far as the sequence goes and a
+    // query at pos can see any of their keys (a page outside the window may have been given back)
+    auto page_at = [&](int j) { return first_page + wave + WAVES * j; };
+    auto next_from = [&](int j) {
+        while (j < ppw && page_at(j) < n_pages && !page_may_be_visible(pos, page_at(j) * kPageTokens, window, sinks)) ++j;
+        return (j < ppw && page_at(j) < n_pages) ? j : -1;
+    };
+    auto page_base = [&](int j) { return ((size_t)row[page_at(j)] * n_kv_heads + kvh) * kPageTokens * HD; };
+    int j = next_from(0);
 
     if (FUSED) {
         // items 0 .. group - 1: the kv head's query heads; then, in the block that holds the
@@ -280,11 +323,10 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_decode_kernel(
         // rotation partner, HD / 2 dimensions away, is lane l ^ 32.
         constexpr int PER = HD / kWave;
         static_assert(PER == 1 || PER == 2, "head sizes 64 and 128");
-        const bool writer = (n_pages - 1) / WAVES == z;
+        const bool writer = (n_pages - 1) / (WAVES * ppw) == z;
         const int items = group + (writer ? 2 : 0);
         const int d = PER * lane;
-        const size_t page_base = writer
-            ? ((size_t)table[(size_t)b * table_stride + n_pages - 1] * n_kv_heads + kvh) * kPageTokens * HD : 0;
+        const size_t wbase = writer ? ((size_t)row[n_pages - 1] * n_kv_heads + kvh) * kPageTokens * HD : 0;
         for (int item = wave; item < items; item += WAVES) {
             const bool is_q = item < group, is_k = item == group;
             const int head = is_q ? kvh * group + item : (is_k ? n_heads + kvh : n_heads + n_kv_heads + kvh);
@@ -296,15 +338,15 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_decode_kernel(
             for (int part0 = 1; part0 < src.parts; part0 += 8) {     // eight loads in flight, added in ascending order
                 float y[8][PER];
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
+                for (int jj = 0; jj < 8; ++jj)
 #pragma unroll
                     for (int e = 0; e < PER; ++e)
-                        y[j][e] = part0 + j < src.parts ? p[(part0 + j) * src.part_stride + e] : 0.f;
+                        y[jj][e] = part0 + jj < src.parts ? p[(part0 + jj) * src.part_stride + e] : 0.f;
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    if (part0 + j < src.parts) {
+                for (int jj = 0; jj < 8; ++jj)
+                    if (part0 + jj < src.parts) {
 #pragma unroll
-                        for (int e = 0; e < PER; ++e) x[e] += y[j][e];
+                        for (int e = 0; e < PER; ++e) x[e] += y[jj][e];
                     }
             }
             if (src.bias) {
@@ -312,7 +354,7 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_decode_kernel(
                 for (int e = 0; e < PER; ++e) x[e] += src.bias[col + e];
             }
             if (!is_q && !is_k) {
-                bf16_t* vdst = src.v_pool + page_base + (pos % kPageTokens);
+                bf16_t* vdst = src.v_pool + wbase + (pos % kPageTokens);
 #pragma unroll
                 for (int e = 0; e < PER; ++e) vdst[(size_t)(d + e) * kPageTokens] = f32_to_bf16(x[e]);
                 continue;
@@ -330,10 +372,10 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_decode_kernel(
 #pragma unroll
             for (int e = 0; e < PER; ++e) {
                 const float partner = __shfl_xor(x[e], 32, kWave);
-                const float2 c = src.cs[(size_t)b * (HD / 2) + ((d + e) & (HD / 2 - 1))];
-                y[e] = f32_to_bf16(lane < 32 ? x[e] * c.x - partner * c.y : partner * c.y + x[e] * c.x);
+                const float2 cs = src.cs[(size_t)b * (HD / 2) + ((d + e) & (HD / 2 - 1))];
+                y[e] = f32_to_bf16(lane < 32 ? x[e] * cs.x - partner * cs.y : partner * cs.y + x[e] * cs.x);
             }
-            bf16_t* dst = is_q ? &q_lds[item][d] : src.k_pool + page_base + (size_t)(pos % kPageTokens) * HD + d;
+            bf16_t* dst = is_q ? &q_lds[item][d] : src.k_pool + wbase + (size_t)(pos % kPageTokens) * HD + d;
 #pragma unroll
             for (int e = 0; e < PER; ++e) dst[e] = y[e];
         }
@@ -342,20 +384,21 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_decode_kernel(
 
     WaveState<HD> st;
     st.init();
-    if (page_idx < n_pages && page_may_be_visible(pos, page_idx * kPageTokens, window, sinks)) {
+    if (j >= 0) {
         bf16x8 qf[HD / 32];
         const bool col_ok = c < group;
         const bf16_t* qrow = FUSED ? &q_lds[col_ok ? c : 0][8 * g]
                                    : q + (size_t)b * q_stride + (size_t)(kvh * group + (col_ok ? c : 0)) * HD + 8 * g;
 #pragma unroll
         for (int sk = 0; sk < HD / 32; ++sk) qf[sk] = col_ok ? ld_frag(qrow + 32 * sk) : zero_frag();
-        const int page = table[(size_t)b * table_stride + page_idx];
-        const size_t base = ((size_t)page * n_kv_heads + kvh) * kPageTokens * HD;
-        const int key0 = page_idx * kPageTokens;
         // unused columns (c >= group) have zero queries and are never stored: they may run unmasked
-        attend_page<HD>(st, qf, k_pool + base, v_pool + base, col_ok ? pos : -1, key0,
-                        min(kPageTokens, pos - key0 + 1), page_fully_visible(pos, pos, key0, window, sinks),
-                        scale * kLog2e, window, sinks);
+        for (; j >= 0; j = next_from(j + 1)) {
+            const int key0 = page_at(j) * kPageTokens;
+            const size_t base = page_base(j);
+            attend_page<HD>(st, qf, k_pool + base, v_pool + base, col_ok ? pos : -1, key0,
+                            min(kPageTokens, pos - key0 + 1), page_fully_visible(pos, pos, key0, window, sinks),
+                            scale * kLog2e, window, sinks);
+        }
     }
     // merge the waves
     if (g == 0) { lds_m[wave * 16 + c] = st.m; lds_l[wave * 16 + c] = st.l; }
@@ -804,10 +847,10 @@ static bool mfma_shape_ok(int n_heads, int n_kv_heads, int head_dim) {
     return (head_dim == 64 || head_dim == 128) && n_heads / n_kv_heads <= 16;
 }
 
-// Waves (= pages) per block of the decode kernel.  A block's pages all come through one CU's
-// vector memory path, so few large blocks are slower than many small ones: blocks grow only
-// while there are enough of them for every CU (then the merge kernel falls away for contexts
-// of up to 1,024 positions), within the LDS that the waves' outputs need.
+// How the decode kernel shares out a sequence's pages: waves per block and pages per wave
+// (a block covers waves * ppw pages; more than one block along the context needs the merge
+// kernel).  A block's pages all come through one CU's vector memory path, so few large blocks
+// are slower than many small ones: blocks grow only while two of them are left for every CU.
 // The choice must not depend on how many other sequences happen to be in the step beyond the
 // step's class of batch sizes (the sizes at which single-token steps are captured: a batch in
 // between runs padded to the next of them), or a sequence's sums would come in another order
@@ -831,21 +874,47 @@ static int compute_units() {
     return cached[device];
 }
 
-static int decode_waves(int group, int table_width, int batch, int n_kv_heads) {
+constexpr int kDecodeWaves = 4;
+constexpr int kMaxPagesPerWave = 16;
+
+// Pages per wave.  A wave's pages come one after the other, a "step" each; a CU works on one
+// block's waves at a time as far as timings show, so a launch takes about as many steps as the
+// blocks that fall to the busiest CU have together: blocks of ppw steps go round by round over
+// the CUs, the shorter last block of each sequence after them.  Every round of blocks costs a
+// quarter of a step more (queries, merge through LDS), the merge kernel three quarters.  The
+// count of steps is what 26 shapes measured at the 8B head shape (32 query heads, 8 kv heads of
+// 128; batch 1 to 64, 640 to 131,000 positions) order by.  Against one page a wave in blocks of
+// up to 16 waves: batch 64 at 640 positions 42.5 us from 46.2, at 8,192 361 from 417; batch 8
+// at 32,768 192 from 211; batch 1 at 131,000 102 from 117; batch 32 at 640 25.1 from 23.6.
+static int decode_pages_per_wave(int table_width, int batch, int n_kv_heads) {
     const long long pairs = (long long)llogos_batch_class(batch) * n_kv_heads;
-    const int units = compute_units();
-    int waves = group <= 4 ? 16 : (group <= 8 ? 8 : 4);
-    while (waves > 4 && (waves / 2 >= table_width || pairs * ((table_width + waves - 1) / waves) < units))
-        waves /= 2;
-    return waves;
+    const long long units = compute_units();
+    int best = 1;
+    double best_cost = 0;
+    for (int ppw = 1; ppw <= kMaxPagesPerWave; ++ppw) {
+        const int chunk = kDecodeWaves * ppw;
+        const long long full = table_width / chunk;                       // whole blocks of a sequence
+        const int rest = table_width % chunk;                             // pages of its last, shorter block
+        const long long full_rounds = (pairs * full + units - 1) / units;
+        double steps = (double)full_rounds * ppw, rounds = (double)full_rounds;
+        if (rest > 0) {
+            const long long room = full_rounds * units - pairs * full;    // places the last round of whole blocks leaves
+            const long long more = pairs > room ? (pairs - room + units - 1) / units : 0;
+            steps += (double)more * ((rest + kDecodeWaves - 1) / kDecodeWaves);
+            rounds += (double)more;
+        }
+        const double cost = steps + 0.25 * rounds + (full + (rest > 0) > 1 ? 0.75 : 0.0);
+        if (ppw == 1 || cost < best_cost - 1e-9) { best = ppw; best_cost = cost; }
+    }
+    return best;
 }
 
 // floats the decode workspace needs
 LLOGOS_EXPORT long long llogos_attn_decode_workspace(int batch, int n_heads, int n_kv_heads, int head_dim,
                                                      int table_width) {
     if (n_kv_heads <= 0 || n_heads % n_kv_heads) return 0;
-    const int waves = decode_waves(n_heads / n_kv_heads, table_width, batch, n_kv_heads);
-    const int n_z = (table_width + waves - 1) / waves;
+    const int ppw = decode_pages_per_wave(table_width, batch, n_kv_heads);
+    const int n_z = (table_width + kDecodeWaves * ppw - 1) / (kDecodeWaves * ppw);
     return n_z == 1 ? 0 : (long long)batch * n_heads * n_z * (head_dim + 2);
 }
 
@@ -859,25 +928,22 @@ static int launch_decode(void* out, const void* q, int q_stride, const QkvSource
     if (workspace_floats < llogos_attn_decode_workspace(batch, n_heads, n_kv_heads, head_dim, table_width))
         return LLOGOS_BAD_ARGUMENT;
     const int group = n_heads / n_kv_heads;
-    const int waves = decode_waves(group, table_width, batch, n_kv_heads);
-    const int n_z = (table_width + waves - 1) / waves;
+    const int waves = kDecodeWaves, ppw = decode_pages_per_wave(table_width, batch, n_kv_heads);
+    const int n_z = (table_width + waves * ppw - 1) / (waves * ppw);
     if (n_z > 1 && workspace == nullptr) return LLOGOS_BAD_ARGUMENT;
     dim3 grid(batch, n_kv_heads, n_z), mgrid(batch, n_heads);
     const size_t smem = decode_lds_bytes(waves, group, head_dim);
     const QkvSource none{};
-#define GO(HD, W, FUSED) do { \
-    attn_decode_kernel<HD, W, FUSED><<<grid, W * kWave, smem, stream>>>( \
+#define GO(HD, FUSED) do { \
+    attn_decode_kernel<HD, kDecodeWaves, FUSED><<<grid, kDecodeWaves * kWave, smem, stream>>>( \
         (bf16_t*)out, workspace, (const bf16_t*)q, q_stride, FUSED ? *src : none, (const bf16_t*)k_pool, \
-        (const bf16_t*)v_pool, table, table_stride, tok_pos, n_heads, n_kv_heads, group, scale, window, sinks); \
+        (const bf16_t*)v_pool, table, table_stride, tok_pos, n_heads, n_kv_heads, group, scale, window, sinks, ppw); \
     if (n_z > 1) attn_decode_merge_kernel<HD><<<mgrid, kMergeLanes * HD, 0, stream>>>((bf16_t*)out, workspace, tok_pos, n_heads, \
-                                                                        n_z, W); } while (0)
-#define BY_WAVES(HD, FUSED) do { if (waves == 16) GO(HD, 16, FUSED); else if (waves == 8) GO(HD, 8, FUSED); \
-                                 else GO(HD, 4, FUSED); } while (0)
-    if (src != nullptr && head_dim == 64) BY_WAVES(64, true);
-    else if (src != nullptr) BY_WAVES(128, true);
-    else if (head_dim == 64) BY_WAVES(64, false);
-    else BY_WAVES(128, false);
-#undef BY_WAVES
+                                                                        n_z, kDecodeWaves * ppw); } while (0)
+    if (src != nullptr && head_dim == 64) GO(64, true);
+    else if (src != nullptr) GO(128, true);
+    else if (head_dim == 64) GO(64, false);
+    else GO(128, false);
 #undef GO
     return LLOGOS_LAUNCH_CHECK();
 }
