@@ -26,11 +26,12 @@ class KVGroup:
         self.pages = GroupPages(n_pages, spec.window, spec.sinks)
         self.k = self.v = None
         if rt is not None:
-            # keys [.., token in page, head size]; values transposed [.., head size, token in page];
-            # one page more than the pool hands out: the page of padding rows (Cache.pad_page)
-            shape = (len(entries), n_pages + 1, spec.n_kv_heads, PAGE_TOKENS, spec.head_dim)
+            # a kv head's part of a page is PAGE_TOKENS * head size elements in the matrix cores'
+            # operand order (pages.key_offset, pages.value_offset); one page more than the pool
+            # hands out: the page of padding rows (Cache.pad_page)
+            shape = (len(entries), n_pages + 1, spec.n_kv_heads, PAGE_TOKENS * spec.head_dim)
             self.k = torch.zeros(shape, dtype=rt.dtype, device=rt.device)
-            self.v = torch.zeros(shape[:3] + (spec.head_dim, PAGE_TOKENS), dtype=rt.dtype, device=rt.device)
+            self.v = torch.zeros(shape, dtype=rt.dtype, device=rt.device)
 
     def bytes(self) -> int:
         return 0 if self.k is None else 2 * self.k.numel() * self.k.element_size()

@@ -17,6 +17,32 @@ class CacheFull(CacheError):
     """Not enough free pages (or slots) for what a step asks."""
 
 
+def key_offset(token: int, d: int, head_dim: int) -> int:
+    """Where dimension d of the key at position `token` of a page lies within one kv head's
+    part of the page (PAGE_TOKENS * head_dim elements).  Pages are stored in the order in
+    which the matrix cores take them as operands: blocks of 4 tokens, then 8 dimensions, then
+    16 rows of 8 values, so that a wave's load of a fragment is 1 KB of consecutive memory.
+    The kernel library has the same rule compiled in (page_key_offset) and loading it fails
+    if the two differ."""
+    return ((((token >> 2) & 3) * (head_dim >> 3) + (d >> 3)) * 16 + (((token >> 4) << 2) | (token & 3))) * 8 + (d & 7)
+
+
+def value_offset(token: int, d: int) -> int:
+    """The same for values: 16 dimensions, then halves of 8 tokens, then 16 tokens' groups,
+    then 16 rows (dimensions) of 8 consecutive tokens."""
+    return ((((d >> 4) * 2 + ((token >> 3) & 1)) * 4 + (token >> 4)) * 16 + (d & 15)) * 8 + (token & 7)
+
+
+def page_offsets(head_dim: int):
+    """(keys, values): two lists [PAGE_TOKENS][head_dim] of element offsets within one kv
+    head's part of a page, for code that fills or reads pages on the host (tests, tools)."""
+    if head_dim <= 0 or head_dim % 16:
+        raise ValueError(f"head size {head_dim} is not a multiple of 16")
+    keys = [[key_offset(t, d, head_dim) for d in range(head_dim)] for t in range(PAGE_TOKENS)]
+    values = [[value_offset(t, d) for d in range(head_dim)] for t in range(PAGE_TOKENS)]
+    return keys, values
+
+
 def pages_for(n_tokens: int) -> int:
     return (n_tokens + PAGE_TOKENS - 1) // PAGE_TOKENS
 

@@ -40,9 +40,10 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
         const bool vis = key_visible(pos, j, window, sinks);
         float s = -INFINITY;
         if (vis) {
-            const T* krow = k_pool + paged_offset(cache, seq, kvh, j);
+            const T* kpage = k_pool + paged_base(cache, seq, kvh, j);
             float dot = 0.f;
-            for (int d = 0; d < head_dim; ++d) dot = fmaf(qf[d], load_f32(krow + d), dot);
+            for (int d = 0; d < head_dim; ++d)
+                dot = fmaf(qf[d], load_f32(kpage + page_key_offset(j % kPageTokens, d, head_dim)), dot);
             s = dot * scale;
         }
         const float tile_max = block_max(s, red);
@@ -62,8 +63,8 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
                 for (int jj = 0; jj < n_keys; ++jj) {
                     const float pj = p_lds[jj];
                     if (pj != 0.f)
-                        a = fmaf(pj, load_f32(v_pool + paged_v_offset(cache, seq, kvh, j0 + jj)
-                                              + (size_t)d * kPageTokens), a);
+                        a = fmaf(pj, load_f32(v_pool + paged_base(cache, seq, kvh, j0 + jj)
+                                              + page_value_offset((j0 + jj) % kPageTokens, d)), a);
                 }
                 acc[r] = a;
             }

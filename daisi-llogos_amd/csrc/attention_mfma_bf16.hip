@@ -13,10 +13,11 @@
 // Scores are computed transposed, S^T[key][column] = K . Q^T, so that the lane that holds
 // the scores of a column for 16 keys is the lane that must supply them as the second
 // operand of O^T[d][column] = V^T[d][key] . P^T[key][column]; no shuffle or LDS pass sits
-// between the two products.  Value pages are stored transposed ([head_dim][64 tokens]), so
-// a lane reads eight consecutive tokens of one dimension with one 16-byte load.  The rows
-// of a key page are visited in the order key = 16 * (i / 4) + 4 * rb + i % 4 (i = operand
-// row, rb = block of 16), which makes lane group g own keys 16 g .. 16 g + 15.
+// between the two products.  Pages are stored in the order of these operands (common.h): a
+// fragment is 1 KB of consecutive memory, a lane's eight values 16 bytes of it; a value
+// fragment holds eight consecutive tokens of one dimension per lane, and the rows of a key
+// fragment are the keys 16 * (i / 4) + 4 * rb + i % 4 (i = operand row, rb = block of 16),
+// which makes lane group g own keys 16 g .. 16 g + 15.
 // (reference: gated_attention / batched_gated_attention, Daisi.Llogos.Cuda/kernels/
 //  composite_ops.cu:275-512: tiles of keys with running maximum and sum, kv head = head /
 //  group, scale after the dot, query m of a prompt sees keys 0 .. start + m.)
@@ -32,6 +33,13 @@ constexpr int kAttnWaves = 4;
 
 __device__ __forceinline__ bf16x8 ld_frag(const bf16_t* p) {
     return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
+}
+
+// A fragment of a page, read once: 64 lanes x 16 bytes of consecutive memory, past the caches'
+// keeping (a step reads every page once and the next step comes after all other layers).
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ bf16x8 ld_frag_once(const bf16_t* p) {
+    return __builtin_bit_cast(bf16x8, __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)));
 }
 
 __device__ __forceinline__ bf16x8 zero_frag() {
@@ -111,9 +119,7 @@ __device__ __forceinline__ void softmax_page(f32x4 (&s)[4], WaveState<HD>& st, f
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             if (MASKED) {
-                // GS < 0: eight consecutive keys per lane group and half page (the layout of the
-                // kernel whose pages go straight to LDS)
-                const int key = GS < 0 ? key0 + 32 * (rb >> 1) + 8 * g + 4 * (rb & 1) + r : key0 + g * GS + rb * RS + r;
+                const int key = key0 + g * GS + rb * RS + r;
                 if (!(q_pos >= 0 && key_visible(q_pos, key, window, sinks))) s[rb][r] = -INFINITY;
             }
             tile_max = fmaxf(tile_max, s[rb][r]);
@@ -153,29 +159,24 @@ __device__ __forceinline__ bool page_fully_visible(int first_pos, int last_pos, 
     return key0 + kPageTokens - 1 < sinks || key0 > last_pos - window;
 }
 
-// The parts of a page's work, apart so that a kernel can ask for the next page's keys and values
-// while it works on this one's.  kpage [64][HD], vpage [HD][64] of one kv head.
+// The parts of a page's work.  kpage, vpage: one kv head's part of a page, in fragment order
+// (common.h): fragment f of either is the 512 elements from 512 f on, lane l's eight at 8 l.
 template <int HD>
 __device__ __forceinline__ void load_keys(bf16x8 (&kf)[4][HD / 32], const bf16_t* __restrict__ kpage) {
-    const int lane = threadIdx.x & (kWave - 1);
-    const int i = lane & 15, g = lane >> 4;
+    const bf16_t* mine = kpage + 8 * (threadIdx.x & (kWave - 1));
 #pragma unroll
-    for (int rb = 0; rb < 4; ++rb) {
-        const bf16_t* krow = kpage + (size_t)(16 * (i >> 2) + 4 * rb + (i & 3)) * HD + 8 * g;
+    for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
-        for (int sk = 0; sk < HD / 32; ++sk) kf[rb][sk] = ld_frag(krow + 32 * sk);
-    }
+        for (int sk = 0; sk < HD / 32; ++sk) kf[rb][sk] = ld_frag_once(mine + 512 * (rb * (HD / 32) + sk));
 }
 
 template <int HD>
 __device__ __forceinline__ void load_values(bf16x8 (&vf)[HD / 16][2], const bf16_t* __restrict__ vpage) {
-    const int lane = threadIdx.x & (kWave - 1);
-    const int i = lane & 15, g = lane >> 4;
+    const bf16_t* mine = vpage + 8 * (threadIdx.x & (kWave - 1));
 #pragma unroll
     for (int db = 0; db < HD / 16; ++db) {
-        const bf16_t* vrow = vpage + (size_t)(16 * db + i) * kPageTokens + 16 * g;
-        vf[db][0] = ld_frag(vrow);
-        vf[db][1] = ld_frag(vrow + 8);
+        vf[db][0] = ld_frag_once(mine + 512 * (2 * db));
+        vf[db][1] = ld_frag_once(mine + 512 * (2 * db + 1));
     }
 }
 
@@ -217,7 +218,7 @@ __device__ __forceinline__ void weigh_values(WaveState<HD>& st, const bf16x8 (&v
 }
 
 // One page of 64 keys.  qf: the columns' queries as second operands (lane (c, g) holds
-// Q[c][32 s + 8 g ..]); kpage [64][HD], vpage [HD][64]; q_pos: position of this lane's column
+// Q[c][32 s + 8 g ..]); kpage, vpage: one kv head's part of a page; q_pos: position of this lane's column
 // (-1: the column is not in use); key0: position of the page's first key; valid_keys: how
 // many of the page's keys have been written (the rest of the page holds whatever was there
 // before: such scores are masked, and such values are zeroed because 0 * NaN is NaN).
@@ -354,9 +355,9 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_decode_kernel(
                 for (int e = 0; e < PER; ++e) x[e] += src.bias[col + e];
             }
             if (!is_q && !is_k) {
-                bf16_t* vdst = src.v_pool + wbase + (pos % kPageTokens);
+                bf16_t* vdst = src.v_pool + wbase;
 #pragma unroll
-                for (int e = 0; e < PER; ++e) vdst[(size_t)(d + e) * kPageTokens] = f32_to_bf16(x[e]);
+                for (int e = 0; e < PER; ++e) vdst[page_value_offset(pos % kPageTokens, d + e)] = f32_to_bf16(x[e]);
                 continue;
             }
             const float* norm_w = is_q ? src.q_norm_w : src.k_norm_w;
@@ -375,7 +376,8 @@ __global__ __launch_bounds__(WAVES * kWave) void attn_decode_kernel(
                 const float2 cs = src.cs[(size_t)b * (HD / 2) + ((d + e) & (HD / 2 - 1))];
                 y[e] = f32_to_bf16(lane < 32 ? x[e] * cs.x - partner * cs.y : partner * cs.y + x[e] * cs.x);
             }
-            bf16_t* dst = is_q ? &q_lds[item][d] : src.k_pool + wbase + (size_t)(pos % kPageTokens) * HD + d;
+            // (a lane's one or two dimensions are neighbours in a key page too)
+            bf16_t* dst = is_q ? &q_lds[item][d] : src.k_pool + wbase + page_key_offset(pos % kPageTokens, d, HD);
 #pragma unroll
             for (int e = 0; e < PER; ++e) dst[e] = y[e];
         }
@@ -548,36 +550,16 @@ constexpr int kTileRows = 128;
 // kernel; the 4 waves of a block take 32 rows each (two blocks of 16 columns) and walk the same
 // pages: a page is copied to LDS once per block (two buffers, the copy of the next page is in
 // flight while the current one is used), and every key and value fragment a wave reads serves
-// both of its column blocks.  A page's keys and transposed
-// values go from global memory into LDS without passing through registers (16 bytes a lane, a
-// wave's 64 lanes to 1 KB of consecutive LDS), which frees the 32 registers of the copy and the
-// time of the stores.  Such a copy cannot pad rows, so the 16-byte pieces of a row are swizzled
-// instead: piece p of row r lies at p ^ f(r).  LDS serves a wave's 16-byte reads in four groups
-// of lanes {c, c + 16 : c = 8 h .. 8 h + 7} (+32), and a group is free of bank conflicts when its
-// 16 pieces cover the 64 banks once; with f(r) = 2 j(r), where j counts the rows that such a group
-// reads one after the other, that holds for rows of 256 bytes (the keys at head size 128); rows
-// of 128 bytes (the values, and the keys at head size 64) lie two to a bank line, and j counts
-// the rows of equal parity.
-// Operand row i = 4 g' + r of key block rb is key 32 (rb >> 1) + 8 g' + 4 (rb & 1) + r, so the
-// lane of group g holds, after both blocks of a half page, the scores of the 8 consecutive keys
-// 32 t + 8 g .. + 7, and its value operand for that half page is one 16-byte read.
+// both of its column blocks.  A page's keys and values go from global memory into LDS without
+// passing through registers (16 bytes a lane, a wave's 64 lanes to 1 KB of consecutive LDS),
+// which frees the 32 registers of the copy and the time of the stores.  Pages are in fragment
+// order in memory, and so they are in LDS: a wave's read of a fragment is 64 x 16 consecutive
+// bytes, which LDS serves without a bank conflict; no padding and no swizzle.
 template <int HD>
 struct DirectPageLds {
-    bf16_t k[kPageTokens][HD];
-    bf16_t v[HD][kPageTokens];
+    bf16_t k[HD / 8][512];               // fragment (rb, sk) at rb * (HD / 32) + sk
+    bf16_t v[HD / 8][512];               // fragment (db, half) at 2 db + half
 };
-
-__device__ __forceinline__ int direct_key_row(int rb, int i) {
-    return 32 * (rb >> 1) + 8 * (i >> 2) + 4 * (rb & 1) + (i & 3);
-}
-template <int HD>
-__device__ __forceinline__ int direct_k_swizzle(int row) {                // rows read together: i = 0..7 of one block
-    return HD == 128 ? 2 * ((row & 3) | (((row >> 3) & 1) << 2))
-                     : 2 * (((row >> 1) & 1) | (((row >> 3) & 1) << 1));
-}
-__device__ __forceinline__ int direct_v_swizzle(int row) {                // rows of equal parity among 8 consecutive
-    return 2 * ((row >> 1) & 3);
-}
 
 // HALVES = 2: a block of 8 waves, two sets of 4 with page buffers of their own, takes the same
 // 128 rows; the sets take the tile's pages in turn and add their results through LDS at the end.
@@ -658,25 +640,22 @@ void attn_prefill_direct_kernel(
     };
     auto page_id = [&](int pi) { return table[(size_t)b * table_stride + pi]; };
     auto page_base = [&](int id) { return ((size_t)id * n_kv_heads + kvh) * kPageTokens * HD; };
-    // This wave's share of a page's copy, in instructions of 1 KB (64 lanes x 16 bytes): a row of
-    // keys has HD / 8 pieces, a row of values 8; the block's instructions go to its waves in turn.
+    // This wave's share of a page's copy, in instructions of 1 KB (64 lanes x 16 bytes, a fragment):
+    // the block's instructions go to its waves in turn.
     auto copy_page = [&](int id, DirectPageLds<HD>& pg) {
         const bf16_t* kpage = k_pool + page_base(id);
         const bf16_t* vpage = v_pool + page_base(id);
-        constexpr int kKeyPieces = HD / 8, kKeyRows = kWave / kKeyPieces;    // pieces a row, rows an instruction
 #pragma unroll
-        for (int j = 0; j < kPageTokens / kKeyRows / kAttnWaves; ++j) {
-            const int krow0 = kKeyRows * (kAttnWaves * j + wave), krow = krow0 + lane / kKeyPieces;
-            const bf16_t* ksrc = kpage + (size_t)krow * HD + 8 * ((lane % kKeyPieces) ^ direct_k_swizzle<HD>(krow));
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ksrc,
-                                             (__attribute__((address_space(3))) void*)&pg.k[krow0][0], 16, 0, 0);
+        for (int j = 0; j < HD / 8 / kAttnWaves; ++j) {
+            const int f = kAttnWaves * j + wave;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kpage + 512 * f + 8 * lane),
+                                             (__attribute__((address_space(3))) void*)&pg.k[f][0], 16, 0, 0);
         }
 #pragma unroll
         for (int j = 0; j < HD / 8 / kAttnWaves; ++j) {
-            const int vrow0 = 8 * (kAttnWaves * j + wave), vrow = vrow0 + (lane >> 3);
-            const bf16_t* vsrc = vpage + (size_t)vrow * kPageTokens + 8 * ((lane & 7) ^ direct_v_swizzle(vrow));
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vsrc,
-                                             (__attribute__((address_space(3))) void*)&pg.v[vrow0][0], 16, 0, 0);
+            const int f = kAttnWaves * j + wave;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vpage + 512 * f + 8 * lane),
+                                             (__attribute__((address_space(3))) void*)&pg.v[f][0], 16, 0, 0);
         }
     };
     // The values of tokens that have not been written may be anything, also NaN, and 0 * NaN is
@@ -687,10 +666,10 @@ void attn_prefill_direct_kernel(
     auto zero_unwritten = [&](DirectPageLds<HD>& pg, int valid_keys) {
 #pragma unroll
         for (int j = 0; j < HD / 8 / kAttnWaves; ++j) {
-            const int vrow = 8 * (kAttnWaves * j + wave) + (lane >> 3);
-            const int keep = valid_keys - 8 * ((lane & 7) ^ direct_v_swizzle(vrow));   // of the tokens this piece holds
+            const int f = kAttnWaves * j + wave;
+            const int keep = valid_keys - 16 * (lane >> 4) - 8 * (f & 1);          // of the tokens this piece holds
             if (keep >= 8) continue;
-            uint4* at = reinterpret_cast<uint4*>(&pg.v[vrow][8 * (lane & 7)]);
+            uint4* at = reinterpret_cast<uint4*>(&pg.v[f][8 * lane]);
             *at = __builtin_bit_cast(uint4, keep_first(__builtin_bit_cast(bf16x8, *at), keep));
         }
     };
@@ -734,17 +713,14 @@ void attn_prefill_direct_kernel(
         for (int sk = 0; sk < HD / 32; ++sk) {
 #pragma unroll
             for (int rb = 0; rb < 4; ++rb) {
-                const int row = direct_key_row(rb, c);
                 const bf16x8 kf = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(
-                    &pg.k[row][8 * ((4 * sk + g) ^ direct_k_swizzle<HD>(row))]));
+                    &pg.k[rb * (HD / 32) + sk][8 * lane]));
                 s0[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf0[sk], s0[rb], 0, 0, 0);
                 s1[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf1[sk], s1[rb], 0, 0, 0);
             }
         }
         auto read_v = [&](int db, int t) {
-            const int row = 16 * db + c;
-            return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(
-                &pg.v[row][8 * ((4 * t + g) ^ direct_v_swizzle(row))]));
+            return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(&pg.v[2 * db + t][8 * lane]));
         };
         constexpr int kEarly = 2;
         bf16x8 vf[HD / 16][2];
@@ -755,11 +731,11 @@ void attn_prefill_direct_kernel(
         const bool all_visible = wave_rows == 32 &&
                                  page_fully_visible(wave_first_pos, wave_last_pos, key0, window, sinks);
         if (all_visible) {
-            softmax_page<false, -1, 0, HD>(s0, st0, scale_log2, q_pos0, key0, window, sinks, pf0, corr0);
-            softmax_page<false, -1, 0, HD>(s1, st1, scale_log2, q_pos1, key0, window, sinks, pf1, corr1);
+            softmax_page<false, 16, 4, HD>(s0, st0, scale_log2, q_pos0, key0, window, sinks, pf0, corr0);
+            softmax_page<false, 16, 4, HD>(s1, st1, scale_log2, q_pos1, key0, window, sinks, pf1, corr1);
         } else {
-            softmax_page<true, -1, 0, HD>(s0, st0, scale_log2, q_pos0, key0, window, sinks, pf0, corr0);
-            softmax_page<true, -1, 0, HD>(s1, st1, scale_log2, q_pos1, key0, window, sinks, pf1, corr1);
+            softmax_page<true, 16, 4, HD>(s0, st0, scale_log2, q_pos0, key0, window, sinks, pf0, corr0);
+            softmax_page<true, 16, 4, HD>(s1, st1, scale_log2, q_pos1, key0, window, sinks, pf1, corr1);
         }
         const bool rescale = __ballot(corr0 != 1.0f || corr1 != 1.0f) != 0;
         __builtin_amdgcn_sched_barrier(0);
@@ -847,14 +823,10 @@ static bool mfma_shape_ok(int n_heads, int n_kv_heads, int head_dim) {
     return (head_dim == 64 || head_dim == 128) && n_heads / n_kv_heads <= 16;
 }
 
-// How the decode kernel shares out a sequence's pages: waves per block and pages per wave
-// (a block covers waves * ppw pages; more than one block along the context needs the merge
-// kernel).  A block's pages all come through one CU's vector memory path, so few large blocks
-// are slower than many small ones: blocks grow only while two of them are left for every CU.
-// The choice must not depend on how many other sequences happen to be in the step beyond the
-// step's class of batch sizes (the sizes at which single-token steps are captured: a batch in
-// between runs padded to the next of them), or a sequence's sums would come in another order
-// alone than beside others of its class: `batch` is rounded up to its class first.
+// The classes of batch sizes: the sizes at which single-token steps are captured (a batch in
+// between runs padded to the next of them).  Whatever a kernel's shape takes from the batch it
+// takes from the class, or a sequence's sums would come in another order alone than beside
+// others of its class.
 LLOGOS_EXPORT int llogos_batch_class(int batch) {
     static const int classes[] = {1, 2, 3, 4, 5, 6, 7, 8, 12, 16, 24, 32, 48, 64};
     for (int c : classes) if (batch <= c) return c;

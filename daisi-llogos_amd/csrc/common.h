@@ -77,10 +77,27 @@ __device__ __forceinline__ float block_max(float v, float* red) {
 }
 
 // A layer's keys and values live in pages of kPageTokens tokens.  A sequence's pages are
-// listed in its row of the step's page table.
-//   keys:   pool[page][kv_head][token in page][head_dim]
-//   values: pool[page][kv_head][head_dim][token in page]   (transposed, so that the
-//           matrix cores can take eight consecutive tokens of one dimension in one load)
+// listed in its row of the step's page table.  pool[page][kv_head] is one kv head's part of a
+// page: kPageTokens * head_dim elements, keys in one pool and values in another, laid out in
+// the order in which the matrix cores take them as operands, so that a wave's load of a
+// fragment (64 lanes x 8 elements) is one run of consecutive memory and every cache line that
+// is fetched is used whole:
+//   keys:   [block of 4 tokens rb = (t >> 2) & 3][8 dimensions d >> 3][row i = 4 (t >> 4) + (t & 3)][d & 7]
+//           fragment (rb, d >> 5) holds, for lane (i, g), dimensions 32 (d >> 5) + 8 g .. + 7 of
+//           token 16 (i >> 2) + 4 rb + (i & 3): after the four blocks' products S^T = K . Q^T, lane
+//           group g holds the scores of tokens 16 g .. 16 g + 15.
+//   values: [16 dimensions d >> 4][half (t >> 3) & 1][tokens t >> 4][d & 15][t & 7]
+//           fragment (d >> 4, half) holds, for lane (i, g), tokens 16 g + 8 half .. + 7 of
+//           dimension 16 (d >> 4) + i: the first operand of O^T += V^T . P^T.
+// head_dim is a multiple of 16.
+__host__ __device__ __forceinline__ int page_key_offset(int token, int d, int head_dim) {
+    return ((((token >> 2) & 3) * (head_dim >> 3) + (d >> 3)) * 16 + (((token >> 4) << 2) | (token & 3))) * 8 + (d & 7);
+}
+
+__host__ __device__ __forceinline__ int page_value_offset(int token, int d) {
+    return ((((d >> 4) * 2 + ((token >> 3) & 1)) * 4 + (token >> 4)) * 16 + (d & 15)) * 8 + (token & 7);
+}
+
 struct PagedKV {
     const int* table;      // [batch, table_stride] page ids of this step's sequences
     int table_stride;
@@ -88,15 +105,10 @@ struct PagedKV {
     int head_dim;
 };
 
-__device__ __forceinline__ size_t paged_offset(const PagedKV& c, int seq, int kv_head, int pos) {
+// offset of the kv head's part of the page that holds position pos of sequence seq
+__device__ __forceinline__ size_t paged_base(const PagedKV& c, int seq, int kv_head, int pos) {
     const int page = c.table[(size_t)seq * c.table_stride + pos / kPageTokens];
-    return (((size_t)page * c.n_kv_heads + kv_head) * kPageTokens + (pos % kPageTokens)) * c.head_dim;
-}
-
-// offset of dimension 0 of a value vector; dimension d lies d * kPageTokens further
-__device__ __forceinline__ size_t paged_v_offset(const PagedKV& c, int seq, int kv_head, int pos) {
-    const int page = c.table[(size_t)seq * c.table_stride + pos / kPageTokens];
-    return ((size_t)page * c.n_kv_heads + kv_head) * kPageTokens * c.head_dim + (pos % kPageTokens);
+    return ((size_t)page * c.n_kv_heads + kv_head) * kPageTokens * c.head_dim;
 }
 
 // A query at q_pos sees key k_pos when it is not in the future and, with a window,

@@ -6,6 +6,9 @@
 
 // what the host side checks its own page size against when it loads the library
 LLOGOS_EXPORT int llogos_page_tokens(void) { return kPageTokens; }
+// where element (token, d) of a kv head's part of a page lies (for checks of the host's copy of the rule)
+LLOGOS_EXPORT int llogos_page_key_offset(int token, int d, int head_dim) { return page_key_offset(token, d, head_dim); }
+LLOGOS_EXPORT int llogos_page_value_offset(int token, int d) { return page_value_offset(token, d); }
 LLOGOS_EXPORT int llogos_wave_size(void) { return kWave; }
 
 // ---------------------------------------------------------------- embedding
@@ -315,15 +318,15 @@ __global__ void qk_rope_cache_kernel(const TI* __restrict__ qkv, int parts, size
     __syncthreads();
     if (!active) return;
 
+    const int in_page = tok_pos[t] % kPageTokens;
     T* dst;
     if (is_q) {
         dst = q_out + ((size_t)t * n_heads + head) * head_dim;
     } else if (is_k) {
-        dst = k_pool + paged_offset(cache, tok_seq[t], head - n_heads, tok_pos[t]);
+        dst = k_pool + paged_base(cache, tok_seq[t], head - n_heads, tok_pos[t]);
     } else {
-        // values are stored transposed: dimension d of this token lies d * kPageTokens further
-        T* vdst = v_pool + paged_v_offset(cache, tok_seq[t], head - n_heads - n_kv_heads, tok_pos[t]);
-        for (int d = lane; d < head_dim; d += kWave) store_f32(vdst + (size_t)d * kPageTokens, buf[d]);
+        T* vdst = v_pool + paged_base(cache, tok_seq[t], head - n_heads - n_kv_heads, tok_pos[t]);
+        for (int d = lane; d < head_dim; d += kWave) store_f32(vdst + page_value_offset(in_page, d), buf[d]);
         return;
     }
     const float2* c = cs + (size_t)t * half;
@@ -339,7 +342,7 @@ __global__ void qk_rope_cache_kernel(const TI* __restrict__ qkv, int parts, size
                 else              v = buf[d - 1] * c[i].y + buf[d] * c[i].x;
             }
         }
-        store_f32(dst + d, v);
+        store_f32(dst + (is_q ? d : page_key_offset(in_page, d, head_dim)), v);
     }
 }
 
@@ -367,9 +370,9 @@ __global__ void qk_rope_cache_hd128_kernel(const TI* __restrict__ qkv, int parts
     const bool is_q = head < n_heads;
     const bool is_k = !is_q && head < n_heads + n_kv_heads;
     if (!is_q && !is_k) {
-        T* vdst = v_pool + paged_v_offset(cache, tok_seq[t], head - n_heads - n_kv_heads, tok_pos[t]);
-        store_f32(vdst + (size_t)d * kPageTokens, x0);
-        store_f32(vdst + (size_t)(d + 1) * kPageTokens, x1);
+        T* vdst = v_pool + paged_base(cache, tok_seq[t], head - n_heads - n_kv_heads, tok_pos[t]);
+        store_f32(vdst + page_value_offset(tok_pos[t] % kPageTokens, d), x0);
+        store_f32(vdst + page_value_offset(tok_pos[t] % kPageTokens, d + 1), x1);
         return;
     }
     const float* norm_w = is_q ? q_norm_w : k_norm_w;
@@ -384,10 +387,12 @@ __global__ void qk_rope_cache_hd128_kernel(const TI* __restrict__ qkv, int parts
     float y0, y1;
     if (lane < 32) { y0 = x0 * c0.x - p0 * c0.y; y1 = x1 * c1.x - p1 * c1.y; }
     else           { y0 = p0 * c0.y + x0 * c0.x; y1 = p1 * c1.y + x1 * c1.x; }
-    T* dst = is_q ? q_out + ((size_t)t * n_heads + head) * HD
-                  : k_pool + paged_offset(cache, tok_seq[t], head - n_heads, tok_pos[t]);
-    store_f32(dst + d, y0);
-    store_f32(dst + d + 1, y1);
+    // (dimensions 2 l and 2 l + 1 are neighbours in a key page too)
+    T* dst = is_q ? q_out + ((size_t)t * n_heads + head) * HD + d
+                  : k_pool + paged_base(cache, tok_seq[t], head - n_heads, tok_pos[t])
+                           + page_key_offset(tok_pos[t] % kPageTokens, d, HD);
+    store_f32(dst, y0);
+    store_f32(dst + 1, y1);
 }
 
 // qkv: the fused projection [parts][T][row_stride] in float32 or in the cache's type (parts are

@@ -89,10 +89,12 @@ def _parts(t: Optional[torch.Tensor]) -> Tuple[int, int]:
 
 
 def _check_pools(k_pool: torch.Tensor, v_pool: torch.Tensor, n_kv_heads: int, head_dim: int, who: str) -> None:
-    _need(tuple(k_pool.shape[1:]) == (n_kv_heads, PAGE_TOKENS, head_dim),
-          f"{who}: key pool must be [pages, kv_heads, {PAGE_TOKENS}, head_dim]")
-    _need(tuple(v_pool.shape) == (k_pool.shape[0], n_kv_heads, head_dim, PAGE_TOKENS),
-          f"{who}: value pool must be [pages, kv_heads, head_dim, {PAGE_TOKENS}] (transposed pages)")
+    _need(head_dim % 16 == 0, f"{who}: head size {head_dim} is not a multiple of 16")
+    _need(tuple(k_pool.shape[1:]) == (n_kv_heads, PAGE_TOKENS * head_dim),
+          f"{who}: key pool must be [pages, kv_heads, {PAGE_TOKENS} * head_dim]")
+    _need(tuple(v_pool.shape) == tuple(k_pool.shape),
+          f"{who}: value pool must be [pages, kv_heads, {PAGE_TOKENS} * head_dim] like the key pool")
+    _need(k_pool.is_contiguous() and v_pool.is_contiguous(), f"{who}: the pools must be contiguous")
 
 
 # ----------------------------------------------------------------------------

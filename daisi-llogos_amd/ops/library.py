@@ -205,10 +205,14 @@ def load() -> ctypes.CDLL:
     except OSError as e:
         raise KernelLibraryError(f"cannot load {path}: {e}") from e
     lib.llogos_attn_decode_workspace.restype = ctypes.c_longlong       # every other entry returns an int code
-    from ..cache.pages import PAGE_TOKENS
+    from ..cache.pages import PAGE_TOKENS, key_offset, value_offset
     if lib.llogos_page_tokens() != PAGE_TOKENS:
         raise KernelLibraryError(f"{path} was built for pages of {lib.llogos_page_tokens()} positions, "
                                  f"the cache uses {PAGE_TOKENS}")
+    for token, d, hd in ((0, 0, 16), (5, 9, 16), (63, 127, 128), (37, 70, 96), (18, 33, 64), (44, 255, 256)):
+        if (lib.llogos_page_key_offset(token, d, hd) != key_offset(token, d, hd)
+                or lib.llogos_page_value_offset(token, d) != value_offset(token, d)):
+            raise KernelLibraryError(f"{path} lays pages out otherwise than cache/pages.py does")
     with _lock:
         _lib = lib
     return lib

@@ -65,8 +65,8 @@ class GroupView:
 @dataclass
 class LayerCache:
     """What one scheduled layer sees of the cache in a step."""
-    k_pool: Optional[torch.Tensor] = None     # [pages, kv_heads, 64, head_dim]
-    v_pool: Optional[torch.Tensor] = None     # [pages, kv_heads, head_dim, 64] (transposed pages)
+    k_pool: Optional[torch.Tensor] = None     # [pages, kv_heads, 64 * head_dim], a page in the matrix cores'
+    v_pool: Optional[torch.Tensor] = None     # operand order (cache/pages.py: key_offset, value_offset)
     table: Optional[torch.Tensor] = None      # int32 [batch, pages]
     writes: bool = True                       # False: reads the pages another layer wrote
     state: Optional[torch.Tensor] = None      # [slots, *StateSpec.shape]

@@ -151,3 +151,35 @@ def test_random_traffic_never_loses_or_doubles_a_page():
         for s, n in live.items():
             assert c.length(s) == n
             assert len(c.groups[0].pages.seqs[s].pages) == pages.pages_for(n)
+
+
+@pytest.mark.parametrize("hd", [16, 48, 64, 128, 256])
+def test_a_page_holds_every_element_once_and_a_fragment_is_one_run_of_memory(hd):
+    """The page layout is a rule of its own (the kernels have a copy of it): every (token,
+    dimension) has a place of its own inside the kv head's part of the page, and the eight
+    values a lane of the matrix cores takes lie together, the 64 lanes of a fragment one after
+    the other: keys, lane (i, g) of fragment (rb, sk) = dimensions 32 sk + 8 g .. + 7 of token
+    16 (i / 4) + 4 rb + i % 4; values, lane (i, g) of fragment (db, half) = tokens
+    16 g + 8 half .. + 7 of dimension 16 db + i."""
+    keys, values = pages.page_offsets(hd)
+    for table in (keys, values):
+        flat = sorted(x for row in table for x in row)
+        assert flat == list(range(pages.PAGE_TOKENS * hd))
+    for rb in range(4):
+        for piece in range(hd // 8):                                    # eight dimensions of 16 rows: 256 bytes in bfloat16
+            for i in range(16):
+                token = 16 * (i // 4) + 4 * rb + i % 4
+                want = ((rb * (hd // 8) + piece) * 16 + i) * 8
+                assert [keys[token][8 * piece + e] for e in range(8)] == list(range(want, want + 8))
+        for sk in range(hd // 32 if hd % 32 == 0 else 0):               # four pieces are a fragment of the matrix cores
+            for lane in range(64):
+                i, g = lane & 15, lane >> 4
+                assert keys[16 * (i // 4) + 4 * rb + i % 4][32 * sk + 8 * g] == ((rb * (hd // 32) + sk) * 64 + lane) * 8
+    for db in range(hd // 16):
+        for half in range(2):
+            for lane in range(64):
+                i, g = lane & 15, lane >> 4
+                want = ((2 * db + half) * 64 + lane) * 8
+                assert [values[16 * g + 8 * half + e][16 * db + i] for e in range(8)] == list(range(want, want + 8))
+    with pytest.raises(ValueError):
+        pages.page_offsets(40)

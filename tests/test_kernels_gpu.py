@@ -234,6 +234,14 @@ def test_rope_table_is_double_precision():
     assert np.abs(cs[..., 0] - np.cos(ang)).max() < 1e-7 and np.abs(cs[..., 1] - np.sin(ang)).max() < 1e-7
 
 
+def _page_index(hd):
+    """(keys, values): index tensors [64, hd] of where (token, dimension) lies in one kv head's part
+    of a page, by the cache's own rule (cache/pages.py)."""
+    pages = importlib.import_module("daisi-llogos_amd.cache.pages")
+    ki, vi = pages.page_offsets(hd)
+    return torch.tensor(ki, device=DEV), torch.tensor(vi, device=DEV)
+
+
 def _pages(n_seqs, max_len, rng):
     """A shuffled page table: sequences' pages lie anywhere in the pool."""
     per = (max_len + 63) // 64
@@ -262,8 +270,8 @@ def test_qk_rope_cache(dtype, nh, nkv, hd, rot, pairing, norm, lens, new):
     kw = 1 + 0.1 * rng.standard_normal(hd)
     f = pm.rope_frequencies(rot, 1e4)
     cs = K.rope_table(_t(tok_pos, torch.int32), _t(f, torch.float64))
-    kp = torch.zeros((n_pages, nkv, 64, hd), dtype=DT[dtype], device=DEV)
-    vp = torch.zeros((n_pages, nkv, hd, 64), dtype=DT[dtype], device=DEV)     # value pages are transposed
+    kp = torch.zeros((n_pages, nkv, 64 * hd), dtype=DT[dtype], device=DEV)
+    vp = torch.zeros((n_pages, nkv, 64 * hd), dtype=DT[dtype], device=DEV)
     args = (nh, nkv, hd, rot, pairing, _t(qw) if norm else None, _t(kw) if norm else None, 1e-5,
             cs, kp, vp, _t(table, torch.int32), _t(tok_seq, torch.int32), _t(tok_pos, torch.int32))
     q_out = K.qk_rope_cache(qkv, bias, DT[dtype], *args)
@@ -279,10 +287,11 @@ def test_qk_rope_cache(dtype, nh, nkv, hd, rot, pairing, norm, lens, new):
     q, k = rope(q, tok_pos, nh, hd, f), rope(k, tok_pos, nkv, hd, f)
     _close(q_out, q, dtype)
     kc, vc = _np(kp), _np(vp)
+    ki, vi = (_np(i).astype(np.int64) for i in _page_index(hd))
     for t in range(T):
         page = table[tok_seq[t], tok_pos[t] // 64]
-        got_k = kc[page, :, tok_pos[t] % 64, :].reshape(-1)
-        got_v = vc[page, :, :, tok_pos[t] % 64].reshape(-1)
+        got_k = kc[page][:, ki[tok_pos[t] % 64]].reshape(-1)
+        got_v = vc[page][:, vi[tok_pos[t] % 64]].reshape(-1)
         assert np.abs(got_k - k[t]).max() <= RT[dtype] * max(1, np.abs(k).max())
         assert np.abs(got_v - v[t]).max() <= RT[dtype] * max(1, np.abs(v).max())
     assert np.count_nonzero(kc) == T * nkv * hd and np.count_nonzero(vc) == T * nkv * hd   # nothing else was written
@@ -294,8 +303,9 @@ def _attention_case(dtype, nh, nkv, hd, lens, new, window=0, sinks=0, seed=4, sc
     rng = np.random.default_rng(seed)
     B, T = len(lens), sum(new)
     table, n_pages = _pages(B, max(lens), rng)
-    kp = torch.zeros((n_pages, nkv, 64, hd), dtype=DT[dtype], device=DEV)
-    vp = torch.zeros((n_pages, nkv, hd, 64), dtype=DT[dtype], device=DEV)
+    kp = torch.zeros((n_pages, nkv, 64 * hd), dtype=DT[dtype], device=DEV)
+    vp = torch.zeros((n_pages, nkv, 64 * hd), dtype=DT[dtype], device=DEV)
+    ki, vi = _page_index(hd)
     ks = [rng.standard_normal((l, nkv * hd)) for l in lens]
     vs = [rng.standard_normal((l, nkv * hd)) for l in lens]
     for b in range(B):
@@ -303,13 +313,13 @@ def _attention_case(dtype, nh, nkv, hd, lens, new, window=0, sinks=0, seed=4, sc
         ks[b], vs[b] = _np(kb), _np(vb)
         for p0 in range(0, lens[b], 64):                                # page by page
             n = min(64, lens[b] - p0)
-            kp[table[b, p0 // 64], :, :n, :] = kb[p0:p0 + n].view(n, nkv, hd).permute(1, 0, 2)
-            vp[table[b, p0 // 64], :, :, :n] = vb[p0:p0 + n].view(n, nkv, hd).permute(1, 2, 0)
+            kp[table[b, p0 // 64]][:, ki[:n]] = kb[p0:p0 + n].view(n, nkv, hd).permute(1, 0, 2)
+            vp[table[b, p0 // 64]][:, vi[:n]] = vb[p0:p0 + n].view(n, nkv, hd).permute(1, 0, 2)
     stride = nh * hd + 24                                               # queries sit in a wider row
     qbuf = _t(rng.standard_normal((T, stride)) * scale_q, DT[dtype])
     tok_seq = np.repeat(np.arange(B), new).astype(np.int32)
     tok_pos = np.concatenate([np.arange(l - n, l) for l, n in zip(lens, new)]).astype(np.int32)
-    return dict(q=qbuf, stride=stride, kp=kp, vp=vp, table=_t(table, torch.int32), ks=ks, vs=vs,
+    return dict(q=qbuf, stride=stride, kp=kp, vp=vp, ki=ki, vi=vi, table=_t(table, torch.int32), ks=ks, vs=vs,
                 tok_seq=tok_seq, tok_pos=tok_pos, new=new, lens=lens)
 
 
@@ -362,8 +372,8 @@ def test_single_token_attention_with_blocks_of_every_size(nh, nkv, hd, batch, lo
     for b, l in enumerate(lens):                                        # unwritten page tails must not matter
         if l % 64:
             page = int(c["table"][b, l // 64])
-            c["kp"][page, :, l % 64:, :] = float("nan")
-            c["vp"][page, :, :, l % 64:] = float("nan")
+            c["kp"][page][:, c["ki"][l % 64:]] = float("nan")
+            c["vp"][page][:, c["vi"][l % 64:]] = float("nan")
     ctx = type("Ctx", (), dict(tok_seq=_t(c["tok_seq"], torch.int32), tok_pos=_t(c["tok_pos"], torch.int32),
                                is_decode=True, max_context=max(lens), batch=batch, n_tokens=batch,
                                cu_seqlens=list(range(batch + 1)), cu_dev=None, starts=[l - 1 for l in lens],
@@ -392,8 +402,8 @@ def test_attention_of_random_shapes(dtype):
         for b, l in enumerate(lens):                                        # unwritten page tails must not matter
             if l % 64:
                 page = int(c["table"][b, l // 64])
-                c["kp"][page, :, l % 64:, :] = float("nan")
-                c["vp"][page, :, :, l % 64:] = float("nan")
+                c["kp"][page][:, c["ki"][l % 64:]] = float("nan")
+                c["vp"][page][:, c["vi"][l % 64:]] = float("nan")
         ctx = type("Ctx", (), dict(tok_seq=_t(c["tok_seq"], torch.int32), tok_pos=_t(c["tok_pos"], torch.int32),
                                    is_decode=max(new) == 1, max_context=max(lens), batch=B, n_tokens=sum(new),
                                    cu_seqlens=np.concatenate([[0], np.cumsum(new)]).tolist(),
@@ -426,8 +436,8 @@ def test_prompt_attention_on_the_matrix_cores(tile_rows, halves, nh, nkv, hd, wi
             for b, l in enumerate(lens):
                 if l % 64:
                     page = int(c["table"][b, l // 64])
-                    c["kp"][page, :, l % 64:, :] = float("nan")
-                    c["vp"][page, :, :, l % 64:] = float("nan")
+                    c["kp"][page][:, c["ki"][l % 64:]] = float("nan")
+                    c["vp"][page][:, c["vi"][l % 64:]] = float("nan")
             out = K.attention_mfma_bf16(ctx, c["q"], c["stride"], c["kp"], c["vp"], c["table"], nh, nkv, hd,
                                         1 / math.sqrt(hd), window, sinks)
             assert out is not None
@@ -445,7 +455,7 @@ def test_attention_finds_a_far_key_among_hundreds(dtype):
     far = 5
     page, off = int(c["table"][0, far // 64]), far % 64
     key = torch.zeros(hd, device=DEV); key[3] = 40.0
-    c["kp"][page, :, off, :] = key.to(c["kp"].dtype)
+    c["kp"][page][:, c["ki"][off]] = key.to(c["kp"].dtype)
     q[0, :nh * hd] = (key.repeat(nh) * 2).to(q.dtype)                   # score 40 * 80 / 8 = 400 for that key
     ctx = type("Ctx", (), dict(tok_seq=_t(c["tok_seq"], torch.int32), tok_pos=_t(c["tok_pos"], torch.int32),
                                is_decode=True, max_context=L, batch=1, n_tokens=1, cu_seqlens=[0, 1], cu_dev=None,
@@ -467,8 +477,8 @@ def test_attention_window_edges(dtype, window, sinks, hd):
             for p in (l - 1 - window, l - window):
                 if p >= max(sinks, 0) and p >= 0:
                     page, off = int(c["table"][b, p // 64]), p % 64
-                    c["kp"][page, :, off, :] *= 6.0
-                    c["ks"][b][p] = _np(c["kp"][page, :, off, :]).reshape(-1)    # as stored
+                    c["kp"][page][:, c["ki"][off]] *= 6.0
+                    c["ks"][b][p] = _np(c["kp"][page][:, c["ki"][off]]).reshape(-1)    # as stored
         ctx = type("Ctx", (), dict(tok_seq=_t(c["tok_seq"], torch.int32), tok_pos=_t(c["tok_pos"], torch.int32),
                                    is_decode=max(new) == 1, max_context=max(lens), batch=len(lens),
                                    n_tokens=sum(new), cu_seqlens=np.concatenate([[0], np.cumsum(new)]).tolist(),

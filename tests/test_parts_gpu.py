@@ -135,8 +135,8 @@ def test_attention_part_alone(dtype, nh, nkv, hd, bias, qk_norm, window):
     q, k = pm.rope_split_half(q, range(T), nh, hd, f), pm.rope_split_half(k, range(T), nkv, hd, f)
     want = pm.linear(pm.attention(q, k, v, nh, nkv, hd, window=window), plain["a.o_proj.weight"])
     # engine part, with a cache of its own
-    pool = lambda *shape: torch.zeros((3, nkv) + shape, dtype=DT[dtype], device=DEV)
-    cache = P.LayerCache(k_pool=pool(64, hd), v_pool=pool(hd, 64), table=torch.tensor([[2, 0]], dtype=torch.int32, device=DEV))
+    pool = lambda: torch.zeros((3, nkv, 64 * hd), dtype=DT[dtype], device=DEV)
+    cache = P.LayerCache(k_pool=pool(), v_pool=pool(), table=torch.tensor([[2, 0]], dtype=torch.int32, device=DEV))
     plain_out = lambda o: K.sum_parts(o, None, DT[dtype])            # a mixer may hand on partial sums
     outs = [plain_out(att.forward(_ctx(rt, [68], [68]), x[:68].to(DEV), cache))]
     for t in (68, 69):
@@ -174,8 +174,8 @@ def test_single_token_steps_from_the_projection_in_one_kernel(nh, nkv, bias, qk_
     results = []
     for fused in (False, True):
         att.fuse_decode = fused
-        pool = lambda *shape: torch.full((12, nkv) + shape, float("nan"), dtype=DT[dtype], device=DEV)
-        cache = P.LayerCache(k_pool=pool(64, hd), v_pool=pool(hd, 64), table=table)
+        pool = lambda: torch.full((12, nkv, 64 * hd), float("nan"), dtype=DT[dtype], device=DEV)
+        cache = P.LayerCache(k_pool=pool(), v_pool=pool(), table=table)
         x0 = torch.cat([x[:l] for (x, _), l in zip(xs, lens)]).to(DEV)
         outs = [K.sum_parts(att.forward(_ctx(rt, lens, lens), x0, cache), None, DT[dtype])]
         for t in range(steps):
@@ -240,8 +240,8 @@ def test_block_arrangement_alone(dtype):
     f = cfg.frequencies()
     want = pm.decoder_layer(cfg, w, 1, x0 + pend, list(range(T + 1)), f)
     kv = block.mixer.kv_spec()
-    pool = lambda *shape: torch.zeros((2, kv.n_kv_heads) + shape, dtype=DT[dtype], device=DEV)
-    cache = P.LayerCache(k_pool=pool(64, kv.head_dim), v_pool=pool(kv.head_dim, 64),
+    pool = lambda: torch.zeros((2, kv.n_kv_heads, 64 * kv.head_dim), dtype=DT[dtype], device=DEV)
+    cache = P.LayerCache(k_pool=pool(), v_pool=pool(),
                          table=torch.tensor([[1]], dtype=torch.int32, device=DEV))
     got = []
     for lo, hi in ((0, T), (T, T + 1)):

@@ -40,8 +40,8 @@ def _case(seed, lens, nh, nkv, hd):
     for b, l in enumerate(lens):
         used = (l + 63) // 64
         table[b, :used] = perm[b, :used]
-    kp = torch.randn((n_pages, nkv, 64, hd), generator=g).to(torch.bfloat16)
-    vp = torch.randn((n_pages, nkv, hd, 64), generator=g).to(torch.bfloat16)
+    kp = torch.randn((n_pages, nkv, 64 * hd), generator=g).to(torch.bfloat16)
+    vp = torch.randn((n_pages, nkv, 64 * hd), generator=g).to(torch.bfloat16)
     q = torch.randn((B, nh * hd), generator=g).to(torch.bfloat16)
     pos = torch.tensor([l - 1 for l in lens], dtype=torch.int32)
     return [t.to(DEV) for t in (q, kp, vp, table, pos)]
