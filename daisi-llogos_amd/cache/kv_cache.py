@@ -148,6 +148,13 @@ class Cache:
             for s, n in zip(slot_ids, new_lens):
                 g.pages.extend(s, n)
 
+    def unreserve(self, slot_ids: Sequence[int]) -> None:
+        """The step did not run: the pages that reserve added beyond each sequence's length go
+        back to their pools."""
+        for g in self.groups:
+            for s in slot_ids:
+                g.pages.trim(s, self.lengths[s])
+
     def commit(self, slot_ids: Sequence[int], new_lens: Sequence[int]) -> None:
         """The step has run: the sequences are new_len long; windowed groups give back the
         pages that no later query can see."""
@@ -174,7 +181,7 @@ class Cache:
         index, -1 where a sequence has no page."""
         out = []
         for g in self.groups:
-            rows = [g.pages.seqs[s].pages for s in slot_ids]
+            rows = [g.pages.seqs[s].row() for s in slot_ids]
             width = max(1, max(len(r) for r in rows))
             t = np.full((len(rows), width), -1, dtype=np.int32)
             for i, r in enumerate(rows):

@@ -124,9 +124,22 @@ class SequencePages:
 
     def __init__(self):
         self.pages: List[int] = []
+        self._row = None                    # the list as an int32 array, made when asked for
 
     def held(self) -> List[int]:
         return [p for p in self.pages if p >= 0]
+
+    def touched(self) -> None:
+        """The list has changed (GroupPages says so after every change it makes)."""
+        self._row = None
+
+    def row(self):
+        """The list as a numpy int32 array, kept until the list changes: a step's page table is
+        put together from these rows, and a sequence's list changes once in PAGE_TOKENS steps."""
+        if self._row is None or len(self._row) != len(self.pages):
+            import numpy as np
+            self._row = np.asarray(self.pages, dtype=np.int32)
+        return self._row
 
 
 class GroupPages:
@@ -155,6 +168,7 @@ class GroupPages:
         n = self.pages_needed(slot, new_len)
         if n:
             self.seqs[slot].pages += self.pool.take(n)
+            self.seqs[slot].touched()
 
     def release_behind_window(self, slot: int, length: int) -> int:
         """After the sequence has `length` tokens: a later query at position >= length sees
@@ -172,6 +186,8 @@ class GroupPages:
                 dead.append(p)
                 pages[i] = -1
         self.pool.give(dead)
+        if dead:
+            self.seqs[slot].touched()
         return len(dead)
 
     def truncate(self, slot: int, length: int) -> None:
@@ -180,5 +196,13 @@ class GroupPages:
         keep = pages_for(length)
         if self.window > 0 and any(p < 0 for p in pages[:keep]) and length > 0:
             raise CacheError("a windowed group cannot be truncated into pages it has given back")
+        self.trim(slot, length)
+
+    def trim(self, slot: int, length: int) -> None:
+        """Give back the pages beyond those that `length` positions need (what a step reserved
+        and did not come to use)."""
+        pages = self.seqs[slot].pages
+        keep = pages_for(length)
         self.pool.give([p for p in pages[keep:] if p >= 0])
         del pages[keep:]
+        self.seqs[slot].touched()

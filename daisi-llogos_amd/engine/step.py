@@ -219,7 +219,17 @@ class Engine:
         rows = self._want_rows(want, counts, cu)
 
         self.cache.reserve(slot_ids, new_lens)
-        T, B = int(cu[-1]), len(entries)
+        try:
+            logits = self._run(ids, counts, cu, rows, slot_ids, starts, new_lens, device_ids)
+        except BaseException:
+            self.cache.unreserve(slot_ids)             # the sequences are as long as before, and hold no page more
+            raise
+        self.cache.commit(slot_ids, new_lens)
+        self.steps_run += 1
+        return logits
+
+    def _run(self, ids, counts, cu, rows, slot_ids, starts, new_lens, device_ids) -> torch.Tensor:
+        T, B = int(cu[-1]), len(counts)
         # (more rows than the hand-written products take would put a library call into the graph)
         if self.graphs is not None and T == B and B <= GRAPH_MAX_BATCH and rows == list(range(B)) \
                 and self.cache.slots.n_slots == self._graph_slots():
@@ -228,8 +238,6 @@ class Engine:
                                           np.asarray(slot_ids, dtype=np.int32), self.cache.step_tables(slot_ids),
                                           device_ids)
                 logits = logits.clone()          # the graph's own buffer is overwritten by its next replay
-            self.cache.commit(slot_ids, new_lens)
-            self.steps_run += 1
             return logits
         tok_seq = np.repeat(np.arange(B, dtype=np.int32), counts)
         tok_pos = np.concatenate([np.arange(s, s + c, dtype=np.int32) for s, c in zip(starts, counts)])
@@ -248,8 +256,6 @@ class Engine:
             dev_tables = [d.view(t.shape) for d, t in zip(dev[6:6 + len(tables)], tables)]
             caches = self.cache.layer_caches(dev_tables)
             logits = self.model.forward(ctx, caches, dev[4] if len(rows) else None)
-        self.cache.commit(slot_ids, new_lens)
-        self.steps_run += 1
         return logits
 
     def _want_rows(self, want, counts: List[int], cu: np.ndarray) -> List[int]:

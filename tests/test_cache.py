@@ -183,3 +183,21 @@ def test_a_page_holds_every_element_once_and_a_fragment_is_one_run_of_memory(hd)
                 assert [values[16 * g + 8 * half + e][16 * db + i] for e in range(8)] == list(range(want, want + 8))
     with pytest.raises(ValueError):
         pages.page_offsets(40)
+
+
+def test_unreserve_gives_back_what_a_step_reserved_and_nothing_else():
+    c = _cache(max_tokens=64 * 8, windows=(0, 64), n_slots=2)
+    a, b = c.alloc_slot(), c.alloc_slot()
+    c.reserve([a], [200]); c.commit([a], [200])                             # the windowed group gives pages back at once
+    free = c.free_pages()
+    held = [list(g.pages.seqs[a].pages) for g in c.groups]
+    c.reserve([a, b], [260, 70])
+    assert c.free_pages() != free
+    c.unreserve([a, b])
+    assert c.free_pages() == free and c.length(a) == 200 and c.length(b) == 0
+    assert [list(g.pages.seqs[a].pages) for g in c.groups] == held
+    assert all(g.pages.seqs[b].pages == [] for g in c.groups)
+    t = c.step_tables([a, b])                                               # rows follow the lists after every change
+    assert [list(r[0][:len(h)]) for r, h in zip(t, held)] == held
+    c.free_slot(a); c.free_slot(b)
+    assert c.free_pages() == [g.pages.pool.n_pages for g in c.groups]

@@ -348,6 +348,30 @@ def test_step_errors():
     assert eng.cache.length(s) == 3
 
 
+def test_a_step_that_fails_while_it_runs_leaves_the_cache_as_it_was(monkeypatch):
+    """Pages are reserved before the model runs.  If the run raises (here: the model's forward
+    is made to), the sequences are as long as before and hold no page more; the next step runs."""
+    eng = H.engine("tiny_a", "float32", max_tokens=64 * 4, n_slots=2)
+    a, b = eng.alloc_slot(), eng.alloc_slot()
+    toks = [list(H.tokens("tiny_a", n, seed=21 + n)) for n in (70, 100)]
+    first = eng.step([(a, toks[0][:60])], want="last")
+    free = eng.cache.free_pages()
+    real = eng.model.forward
+    def broken(*args, **kwargs):
+        raise RuntimeError("stopped on purpose")
+    monkeypatch.setattr(eng.model, "forward", broken)
+    with pytest.raises(RuntimeError, match="on purpose"):
+        eng.step([(a, toks[0][60:70]), (b, toks[1])])                      # one page more for a, two for b
+    assert eng.cache.free_pages() == free and eng.cache.length(a) == 60 and eng.cache.length(b) == 0
+    monkeypatch.setattr(eng.model, "forward", real)
+    got = eng.step([(a, toks[0][60:70]), (b, toks[1])], want="last")
+    ref = H.engine("tiny_a", "float32", max_tokens=64 * 4, n_slots=2)
+    ra, rb = ref.alloc_slot(), ref.alloc_slot()
+    ref.step([(ra, toks[0][:60])])
+    assert torch.equal(got, ref.step([(ra, toks[0][60:70]), (rb, toks[1])], want="last"))
+    assert first.shape[0] == 1
+
+
 def test_a_sequence_cannot_grow_beyond_the_limit():
     """The engine's own limit (the command line's --max-context) within the model's positions:
     the step that would cross it is refused as a whole and nothing changes."""
