@@ -135,11 +135,12 @@ def visible(q_pos: int, k_pos: int, window: int = 0, sinks: int = 0) -> bool:
 
 def attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, n_heads: int, n_kv_heads: int,
               head_dim: int, scale: float | None = None, window: int = 0, sinks: int = 0,
-              positions=None) -> np.ndarray:
+              positions=None, rows=None) -> np.ndarray:
     """Causal grouped-query attention over one whole sequence.  Query head h reads
     KV head h // (n_heads / n_kv_heads); score = (q . k) * scale with scale =
     1/sqrt(head_dim) applied after the dot; softmax over the visible keys; o = sum p v.
-    Daisi.Llogos.Cpu/CpuBackend.cs:476-590 (group :510, scale :541, sum guard :581)."""
+    Daisi.Llogos.Cpu/CpuBackend.cs:476-590 (group :510, scale :541, sum guard :581).
+    rows: the queries to work out (all by default; the other rows of the result stay zero)."""
     t = q.shape[0]
     if scale is None:
         scale = 1.0 / math.sqrt(head_dim)
@@ -152,7 +153,7 @@ def attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, n_heads: int, n_kv_he
     out = np.zeros((t, n_heads, head_dim), dtype=np.float64)
     for h in range(n_heads):
         g = h // group
-        for i in range(t):
+        for i in (range(t) if rows is None else rows):
             keys = [j for j in range(t) if visible(positions[i], positions[j], window, sinks)]
             s = (kh[keys, g, :] @ qh[i, h, :]) * scale
             p = softmax(s)

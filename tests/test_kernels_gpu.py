@@ -331,7 +331,7 @@ def _plain_attention(c, nh, nkv, hd, window=0, sinks=0, scale=None):
         full_q = np.zeros((l, nh * hd))
         full_q[l - n:] = q[o:o + n]
         outs.append(pm.attention(full_q, c["ks"][b], c["vs"][b], nh, nkv, hd, scale=scale, window=window,
-                                 sinks=sinks)[l - n:])
+                                 sinks=sinks, rows=range(l - n, l))[l - n:])
         o += n
     return np.concatenate(outs)
 
@@ -356,14 +356,18 @@ def test_attention_whole_prompts_and_single_tokens(dtype, nh, nkv, hd):
         _close(out, _plain_attention(c, nh, nkv, hd), dtype)
 
 
-@pytest.mark.parametrize("nh,nkv,hd,batch,longest", [(8, 4, 128, 64, 700),      # 16 pages a block, no merge
-                                                     (8, 4, 64, 70, 1500),       # 16 pages a block, merged
-                                                     (16, 2, 64, 128, 700),      # 8 pages a block, merged
-                                                     (8, 4, 128, 4, 1500),       # 4 pages a block, 6 blocks merged
-                                                     (4, 1, 128, 4, 3300)])      # 13 blocks merged
-def test_single_token_attention_with_blocks_of_every_size(nh, nkv, hd, batch, longest):
-    """The decode kernel gives a block more pages when there are many blocks; every form must
-    agree with the plain attention, whatever the lengths of the other sequences."""
+@pytest.mark.parametrize("window,sinks", [(0, 0), (200, 70)])
+@pytest.mark.parametrize("nh,nkv,hd,batch,longest", [(8, 4, 128, 64, 700),      # one block a sequence, three pages a wave
+                                                     (8, 4, 64, 70, 1500),       # batches beyond the captured sizes
+                                                     (16, 2, 64, 128, 700),
+                                                     (8, 4, 128, 4, 1500),       # one page a wave, six blocks merged
+                                                     (4, 1, 128, 4, 3300),       # 13 blocks merged
+                                                     (8, 2, 128, 16, 5000)])     # several pages a wave and several blocks
+def test_single_token_attention_with_blocks_of_every_size(nh, nkv, hd, batch, longest, window, sinks):
+    """The decode kernel gives a wave more pages when there are many blocks; every form must
+    agree with the plain attention, whatever the lengths of the other sequences.  With a window
+    the pages between the sinks and the window are not the sequence's any more (the cache gives
+    them back): they hold NaN here, which would spoil the result if a wave took one of them."""
     rng = np.random.default_rng(batch)
     lens = [int(x) for x in rng.integers(1, longest // 3, batch)]
     lens[1], lens[batch // 2], lens[-1] = longest, 64, 65
@@ -374,13 +378,19 @@ def test_single_token_attention_with_blocks_of_every_size(nh, nkv, hd, batch, lo
             page = int(c["table"][b, l // 64])
             c["kp"][page][:, c["ki"][l % 64:]] = float("nan")
             c["vp"][page][:, c["vi"][l % 64:]] = float("nan")
+        for pi in range((l + 63) // 64 if window else 0):
+            if pi * 64 >= sinks and pi * 64 + 63 <= l - 1 - window:     # no key of the page is visible from position l - 1
+                page = int(c["table"][b, pi])
+                c["kp"][page] = float("nan")
+                c["vp"][page] = float("nan")
     ctx = type("Ctx", (), dict(tok_seq=_t(c["tok_seq"], torch.int32), tok_pos=_t(c["tok_pos"], torch.int32),
                                is_decode=True, max_context=max(lens), batch=batch, n_tokens=batch,
                                cu_seqlens=list(range(batch + 1)), cu_dev=None, starts=[l - 1 for l in lens],
                                shared={}))()
-    out = K.attention_mfma_bf16(ctx, c["q"], c["stride"], c["kp"], c["vp"], c["table"], nh, nkv, hd, 1 / math.sqrt(hd))
+    out = K.attention_mfma_bf16(ctx, c["q"], c["stride"], c["kp"], c["vp"], c["table"], nh, nkv, hd, 1 / math.sqrt(hd),
+                                window, sinks)
     assert out is not None
-    _close(out, _plain_attention(c, nh, nkv, hd), "bfloat16")
+    _close(out, _plain_attention(c, nh, nkv, hd, window, sinks), "bfloat16")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
