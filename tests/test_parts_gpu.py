@@ -148,11 +148,13 @@ def test_attention_part_alone(dtype, nh, nkv, hd, bias, qk_norm, window):
 @pytest.mark.parametrize("hd", [128, 64])
 @pytest.mark.parametrize("nh,nkv,bias,qk_norm,window", [(8, 2, True, True, 0), (16, 1, False, False, 0),
                                                         (5, 5, False, True, 70), (12, 4, True, False, 0)])
-def test_single_token_steps_from_the_projection_in_one_kernel(nh, nkv, bias, qk_norm, window, hd, monkeypatch):
+@pytest.mark.parametrize("lens", [[62, 130, 5], [700, 380, 5]])
+def test_single_token_steps_from_the_projection_in_one_kernel(nh, nkv, bias, qk_norm, window, hd, lens, monkeypatch):
     """Head sizes 128 and 64 in bfloat16: the attention kernel that makes its queries and the
     step's key and value from the projection itself gives, bit for bit, the outputs and the cache
     pages of the rotation kernel followed by the attention kernel, across a page's end, and both
-    agree with the plain parts."""
+    agree with the plain parts.  With the longer sequences the attention takes several blocks along
+    the context, whose results a second kernel merges."""
     dtype, hidden = "bfloat16", 72
     rng = np.random.default_rng(nh)
     rt = P.Runtime(DEV, DT[dtype])
@@ -168,13 +170,14 @@ def test_single_token_steps_from_the_projection_in_one_kernel(nh, nkv, bias, qk_
     taken = []
     fused_kernel = K.attention_decode_fused
     monkeypatch.setattr(K, "attention_decode_fused", lambda *a, **k: (taken.append(fused_kernel(*a, **k)), taken[-1])[1])
-    lens, steps = [62, 130, 5], 4
+    steps = 4
     xs = [_rand(rng, (l + steps, hidden), dtype) for l in lens]
-    table = torch.tensor([[5, 1, 7, 9], [0, 8, 2, 6], [4, 3, 10, 11]], dtype=torch.int32, device=DEV)
+    width = (max(lens) + steps + 63) // 64 + 1
+    table = torch.tensor(rng.permutation(3 * width).reshape(3, width), dtype=torch.int32, device=DEV)
     results = []
     for fused in (False, True):
         att.fuse_decode = fused
-        pool = lambda: torch.full((12, nkv, 64 * hd), float("nan"), dtype=DT[dtype], device=DEV)
+        pool = lambda: torch.full((3 * width, nkv, 64 * hd), float("nan"), dtype=DT[dtype], device=DEV)
         cache = P.LayerCache(k_pool=pool(), v_pool=pool(), table=table)
         x0 = torch.cat([x[:l] for (x, _), l in zip(xs, lens)]).to(DEV)
         outs = [K.sum_parts(att.forward(_ctx(rt, lens, lens), x0, cache), None, DT[dtype])]
