@@ -792,3 +792,131 @@ def test_captured_steps_of_a_mixer_with_state_advance_the_state_once(tmp_path):
         assert np.array_equal(outs[0], outs[1]), f"token {t}: replayed and launched steps differ by {np.abs(outs[0] - outs[1]).max()}"
         H.close(outs[0], np.stack([want[i][cut[i] + t] for i in live]), "float32", f"state on device, token {t}")
     assert len(engines[0].graphs.graphs) == 2
+
+
+# ---------------------------------------------------------------------------
+# a toy mixer with keys and values in the cache and a position scheme that is no rotation, defined here
+# ---------------------------------------------------------------------------
+@P.register_mixer("toy_distance_bias_attention")
+class DistanceBiasAttention(P.Mixer):
+    """Attention without rotation: the score of query i and key j is q . k / sqrt(hd) - slope_h (i - j).
+    It keeps its keys and values in the cache's pages, which it reaches through the cache's own
+    rule for where a (token, dimension) lies in a page (cache/pages.py), with plain tensor
+    operations: nothing of the framework knows of it."""
+
+    def __init__(self, prefix, hidden, n_heads, head_dim, slopes):
+        self.prefix, self.hidden, self.nh, self.hd, self.slopes = prefix, hidden, n_heads, head_dim, list(slopes)
+
+    def tensor_specs(self):
+        return [P.TensorSpec(self.prefix + n + ".weight", shape, "matrix")
+                for n, shape in (("q", (self.nh * self.hd, self.hidden)), ("k", (self.nh * self.hd, self.hidden)),
+                                 ("v", (self.nh * self.hd, self.hidden)), ("o", (self.hidden, self.nh * self.hd)))]
+
+    def kv_spec(self):
+        return P.KVSpec(self.nh, self.hd)
+
+    def bind(self, get, rt):
+        pages = importlib.import_module("daisi-llogos_amd.cache.pages")
+        self.rt = rt
+        self.w = {n: get(self.prefix + n + ".weight").to(device=rt.device, dtype=torch.float32) for n in "qkvo"}
+        ki, vi = pages.page_offsets(self.hd)
+        self.ki, self.vi = torch.tensor(ki, device=rt.device), torch.tensor(vi, device=rt.device)     # [64, hd]
+
+    def forward(self, ctx, h, cache):
+        nh, hd = self.nh, self.hd
+        x = h.float()
+        q, k, v = (x @ self.w[n].T for n in "qkv")
+        out = torch.empty((h.shape[0], nh * hd), dtype=torch.float32, device=h.device)
+        slopes = torch.tensor(self.slopes, device=h.device)[:, None, None]
+        for b in range(ctx.batch):
+            lo, hi = ctx.cu_seqlens[b], ctx.cu_seqlens[b + 1]
+            start, n = ctx.starts[b], ctx.cu_seqlens[b + 1] - ctx.cu_seqlens[b]
+            pos = torch.arange(start, start + n, device=h.device)
+            page, at = cache.table[b].long()[pos // 64], pos % 64
+            for pool, rule, rows in ((cache.k_pool, self.ki, k), (cache.v_pool, self.vi, v)):
+                flat = pool.view(pool.shape[0], nh, 64 * hd)
+                new = rows[lo:hi].view(n, nh, hd).to(pool.dtype)
+                flat[page[:, None, None], torch.arange(nh, device=h.device)[None, :, None], rule[at][:, None, :]] = new
+            every = torch.arange(0, start + n, device=h.device)                        # all positions so far, from the pages
+            page, at = cache.table[b].long()[every // 64], every % 64
+            heads = torch.arange(nh, device=h.device)[None, :, None]
+            keys = cache.k_pool[page[:, None, None], heads, self.ki[at][:, None, :]].float()      # [positions, heads, hd]
+            vals = cache.v_pool[page[:, None, None], heads, self.vi[at][:, None, :]].float()
+            s = torch.einsum("ihd,jhd->hij", q[lo:hi].view(n, nh, hd), keys) / hd ** 0.5
+            dist = (pos[:, None] - every[None, :]).float()
+            s = (s - slopes * dist).masked_fill(dist[None] < 0, float("-inf"))
+            out[lo:hi] = torch.einsum("hij,jhd->ihd", torch.softmax(s, -1), vals).reshape(n, nh * hd)
+        return (out @ self.w["o"].T).to(h.dtype)
+
+
+def _bias_spec(cfg, **kw):
+    models = importlib.import_module("daisi-llogos_amd.models")
+    layers = []
+    for i in range(cfg.n_layers):
+        p = f"layers.{i}."
+        layers.append(models.LayerSpec(
+            mixer=("toy_distance_bias_attention", dict(prefix=p + "mix.", hidden=cfg.hidden_size, n_heads=3, head_dim=16,
+                                                       slopes=[0.5, 0.125, 0.03125])),
+            ffn=("swiglu", dict(prefix=p + "ffn.", hidden=cfg.hidden_size, intermediate=56)),
+            mixer_norm=("rmsnorm", dict(name=p + "n1", width=cfg.hidden_size, eps=1e-6)),
+            ffn_norm=("rmsnorm", dict(name=p + "n2", width=cfg.hidden_size, eps=1e-6))))
+    return models.ModelSpec(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size, embed_name="embed.weight",
+                            layers=layers, final_norm=("rmsnorm", dict(name="norm", width=cfg.hidden_size, eps=1e-6)),
+                            head_name="head", tie_head=False)
+
+
+L.register_architecture("ToyDistanceBiasForCausalLM",
+                        lambda d: ToyConfig(d["vocab_size"], d["hidden_size"], d["n_layers"]), _bias_spec)
+
+
+def test_a_toy_mixer_with_cached_keys_and_a_position_scheme_of_its_own(tmp_path):
+    """A mixer whose positions enter as a bias on the scores (no rotation, no table of angles) and
+    whose keys and values live in the cache's pages is registered, built and stepped from here:
+    whole prompts, then token by token in a batch of unequal lengths across a page's end, with
+    slots and pages used again, against plain arithmetic."""
+    from safetensors.torch import load_file
+    cfg = {"architectures": ["ToyDistanceBiasForCausalLM"], "vocab_size": 70, "hidden_size": 40, "n_layers": 2,
+           "torch_dtype": "float32"}
+    folder = L.write_random_model(str(tmp_path / "bias"), cfg, seed=6)
+    w = {k: v.double().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    slopes = np.array([0.5, 0.125, 0.03125])
+
+    def plain(tokens):
+        T = len(tokens)
+        x = pm.embedding(w["embed.weight"], tokens)
+        dist = np.arange(T)[:, None] - np.arange(T)[None, :]
+        for i in range(2):
+            p = f"layers.{i}."
+            n = pm.rms_norm(x, w[p + "n1.weight"], 1e-6)
+            q, k, v = (pm.linear(n, w[p + f"mix.{m}.weight"]).reshape(T, 3, 16) for m in "qkv")
+            a = np.zeros((T, 3, 16))
+            for hh in range(3):
+                s = q[:, hh] @ k[:, hh].T / 4.0 - slopes[hh] * dist
+                s = np.where(dist < 0, -np.inf, s)
+                a[:, hh] = np.stack([pm.softmax(r) for r in s]) @ v[:, hh]
+            x = x + pm.linear(a.reshape(T, 48), w[p + "mix.o.weight"])
+            n = pm.rms_norm(x, w[p + "n2.weight"], 1e-6)
+            x = x + pm.swiglu_mlp(n, w[p + "ffn.gate_proj.weight"], w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
+        return pm.linear(pm.rms_norm(x, w["norm.weight"], 1e-6), w["head.weight"])
+
+    eng = L.Engine.from_folder(folder, dtype="float32", max_tokens=64 * 5, n_slots=3)
+    assert all(kv == P.KVSpec(3, 16) and st is None for kv, st in eng.model.cache_needs())
+    assert eng.graphs is None or not eng.model.graph_safe                 # the mixer reads the step on the host: never captured
+    rng = np.random.default_rng(1)
+    seqs = [rng.integers(0, 70, size=n).tolist() for n in (75, 9, 130)]
+    want = [plain(s) for s in seqs]
+    for s, wnt in zip(seqs[:2], want):
+        slot = eng.alloc_slot()
+        H.close(_np(eng.step([(slot, s)], want="all")), wnt, "float32", "distance bias, whole")
+        eng.free_slot(slot)
+    slots = [eng.alloc_slot() for _ in seqs]
+    cut = [60, 3, 120]
+    out = _np(eng.step([(sl, s[:c]) for sl, s, c in zip(slots, seqs, cut)], want="last"))
+    H.close(out, np.stack([wnt[c - 1] for wnt, c in zip(want, cut)]), "float32", "distance bias, prompts")
+    for t in range(10):                                                   # across the ends of pages at 64 and 128
+        live = [i for i in range(3) if cut[i] + t < len(seqs[i])]
+        got = _np(eng.step([(slots[i], [seqs[i][cut[i] + t]]) for i in live], want="last"))
+        H.close(got, np.stack([want[i][cut[i] + t] for i in live]), "float32", f"distance bias, token {t}")
+        for i in live:
+            if cut[i] + t + 1 == len(seqs[i]):
+                eng.free_slot(slots[i])
