@@ -226,6 +226,27 @@ def test_products_of_random_shapes_through_the_dispatch():
         assert np.abs(got - (want + _np(b))).max() <= 2e-5 * scale, (case, M, N, K_)
 
 
+@pytest.mark.parametrize("N,K_", [(70, 16), (2048, 8192), (17000, 1000), (33000, 2049), (66000, 530), (5, 4099), (300, 7)])
+def test_float32_product_of_few_rows_is_the_tiled_product_bit_for_bit(N, K_):
+    """Up to 32 rows in float32 go to a kernel of their own (a wave a few columns, the rows of a in
+    registers); it adds in the order of the tiled kernel, so a row's result is the same bits
+    whichever of the two a step's row count selects, alone or beside others, and right."""
+    rng = np.random.default_rng(N)
+    a = _t(rng.standard_normal((40, K_)))
+    w = _t(rng.standard_normal((N, K_)) * 0.05)
+    b = _t(rng.standard_normal(N))
+    tiled = K.gemm_generic(a, w, b, torch.float32)                         # 40 rows: the tiled kernel
+    want = pm.linear(_np(a), _np(w), _np(b))
+    assert np.abs(_np(tiled) - want).max() <= 2e-6 * max(1.0, np.abs(want).max()) * math.sqrt(K_)
+    for M in (1, 2, 3, 4, 7, 8, 9, 16, 31, 32):
+        few = K.gemm_generic(a[:M], w, b, torch.float32)
+        assert torch.equal(few, tiled[:M]), (M, N, K_, (few - tiled[:M]).abs().max().item())
+    wide = _t(rng.standard_normal((5, K_ + 3)))                            # rows that do not start at a multiple of 16 bytes
+    few = K.gemm_generic(wide[:, :K_], w, None, torch.float32)
+    many = K.gemm_generic(torch.cat([wide, wide * 0 + 1.0] * 4)[:, :K_], w, None, torch.float32)
+    assert torch.equal(few, many[:5])
+
+
 def test_rope_table_is_double_precision():
     pos = _t([0, 1, 4095, 100000], torch.int32)
     f = pm.rope_frequencies(64, 5e5)
