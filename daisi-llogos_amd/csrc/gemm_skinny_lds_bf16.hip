@@ -390,7 +390,7 @@ LLOGOS_EXPORT int llogos_gemm_packed_bf16(void* out, int out_dtype, const void* 
 #define BY_MODE(MB, CH) do { if (mode == PRODUCE_PLAIN) GO(MB, PRODUCE_PLAIN, CH); \
                              if (mode == PRODUCE_SWIGLU_F32) GO(MB, PRODUCE_SWIGLU_F32, CH); \
                              GO(MB, PRODUCE_SWIGLU_BF16, CH); } while (0)
-#define BY_ROWS(CH) do { if (mb == 1) BY_MODE(1, CH); if (mb == 2) BY_MODE(2, CH); BY_MODE(4, CH); } while (0)
+#define BY_ROWS(CH) do { if (mb == 1) BY_MODE(1, CH); if (mb == 2) BY_MODE(2, CH); if (mb == 3) BY_MODE(3, CH); BY_MODE(4, CH); } while (0)
     if (chunk == 128) BY_ROWS(128);
     BY_ROWS(256);
 #undef BY_ROWS
@@ -413,7 +413,7 @@ LLOGOS_EXPORT int llogos_gemm_packed_gated_bf16(void* out, int out_dtype, const 
     const int mb = (M + 15) / 16;
 #define GO(MB, CH) return launch_lds<1, MB, PRODUCE_PLAIN, CH, kLdsWaves, true, true>(out, out_dtype, src, W, nullptr, M, N, K, ldo, \
                                                                                      0, kpb, 1, stream)
-#define BY_ROWS(CH) do { if (mb == 1) GO(1, CH); if (mb == 2) GO(2, CH); GO(4, CH); } while (0)
+#define BY_ROWS(CH) do { if (mb == 1) GO(1, CH); if (mb == 2) GO(2, CH); if (mb == 3) GO(3, CH); GO(4, CH); } while (0)
     if (chunk == 128) BY_ROWS(128);
     BY_ROWS(256);
 #undef BY_ROWS
