@@ -872,7 +872,9 @@ static int decode_pages_per_wave(int table_width, int batch, int n_kv_heads) {
         if (rest > 0) {
             const long long room = full_rounds * units - pairs * full;    // places the last round of whole blocks leaves
             const long long more = pairs > room ? (pairs - room + units - 1) / units : 0;
-            steps += (double)more * ((rest + kDecodeWaves - 1) / kDecodeWaves);
+            // (blocks a quarter as long as the whole ones, or less, run beside the last of those: half a step each)
+            const int rest_steps = (rest + kDecodeWaves - 1) / kDecodeWaves;
+            steps += (double)more * rest_steps * (full > 0 && 4 * rest_steps <= ppw ? 0.5 : 1.0);
             rounds += (double)more;
         }
         const double cost = steps + 0.25 * rounds + (full + (rest > 0) > 1 ? 0.75 : 0.0);
