@@ -10,7 +10,7 @@ tests/Daisi.Llogos.Tests/Chat/LayerByLayerCompareTest.cs:43-111.)
 
 With LLOGOS_FULL_SIZE=1 also the whole Llama-3.1-8B configuration (32 layers) and the whole
 Qwen3-14B configuration (40 layers, per-head norms, vocabulary 151936): folders of 16 and 30
-GB, three minutes on the GPU box.
+GB, two minutes on the GPU box.
 
 The bfloat16 engine's distance from float64 arithmetic is set by where values are rounded to
 bfloat16, not by how the engine computes: the plain implementation with the same roundings
