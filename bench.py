@@ -229,14 +229,17 @@ def main(argv=None) -> int:
         print(f"[bench] generation loop b{args.batch}: {record['generate_loop']['value']:.1f} tok/s, "
               f"{record['generate_loop']['ms_per_step']:.3f} ms/step", file=sys.stderr, flush=True)
     if not args.no_points:
-        points = {}
+        points, fractions = {}, {}
         for b in (1, 64):
             steps = args.steps
-            d, _ = decode_run(b, steps, args.warmup)
+            d, mid = decode_run(b, steps, args.warmup)
             points[f"decode_b{b}"] = round(b * steps / d, 1)
-            print(f"[bench] decode b{b}: {points[f'decode_b{b}']:.1f} tok/s, {d / steps * 1e3:.3f} ms/step",
-                  file=sys.stderr, flush=True)
+            # the same account as for the headline step: every weight once and the live requests' cache
+            fractions[f"decode_b{b}"] = round((weight_bytes(cfg) + b * mid * kv_bytes_per_token(cfg)) / (d / steps) / HBM_PEAK, 4)
+            print(f"[bench] decode b{b}: {points[f'decode_b{b}']:.1f} tok/s, {d / steps * 1e3:.3f} ms/step, "
+                  f"{fractions[f'decode_b{b}']:.3f} of {HBM_PEAK / 1e12:g} TB/s", file=sys.stderr, flush=True)
         record["points"] = points
+        record["points_roofline_frac"] = fractions
         prompt = rng.integers(0, cfg["vocab_size"], size=prefill_tokens).tolist()
         times = []
         for it in range(5):                              # the first warms the library up; the best of the rest counts
