@@ -159,7 +159,7 @@ def main(argv=None) -> int:
             nonlocal ids
             for _ in range(n):
                 tokens = fetch_tokens(ids)
-                logits = eng.step(placeholders, want="last", device_ids=(ids, rows))
+                logits = eng.step(placeholders, want="last", device_ids=(ids, rows), borrow=True)
                 done[0] += 1
                 ids = pick(logits, done[0])
                 tokens()

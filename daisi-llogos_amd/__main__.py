@@ -184,15 +184,13 @@ def main(argv=None) -> int:
     llm = Llogos(args.model, dtype=args.dtype, max_context=args.max_context, max_batch=n_batch,
                  attention=args.attention)
     load_ms = (time.perf_counter() - t0) * 1000
-    cfg = llm.config
-    print(f"Loaded {cfg.architecture}: {cfg.num_hidden_layers} layers, hidden {cfg.hidden_size}, "
-          f"{cfg.num_attention_heads}/{cfg.num_key_value_heads} heads, vocab {cfg.vocab_size} "
-          f"in {load_ms:.0f} ms", file=sys.stderr)
+    model = llm.engine.model
+    print(f"Loaded {llm.engine.architecture}: {model.describe()} in {load_ms:.0f} ms", file=sys.stderr)
 
     if args.bench:
         if prompts is None:
             rng = np.random.default_rng(args.seed or 0)
-            prompts = [rng.integers(0, cfg.vocab_size, size=args.prompt_len).tolist() for _ in range(n_batch)]
+            prompts = [rng.integers(0, model.spec.vocab_size, size=args.prompt_len).tolist() for _ in range(n_batch)]
         print(f"Benchmarking with {len(prompts)} prompt(s) of {len(prompts[0])} tokens", file=sys.stderr)
         print(f"Backend: hip ({args.dtype}), Max tokens: {args.max_tokens}\n", file=sys.stderr)
         r = llm.benchmark(prompts, args.max_tokens)
@@ -204,11 +202,15 @@ def main(argv=None) -> int:
               f"({r.decode_tokens_per_second:8.1f} tok/s)", file=sys.stderr)
         print(f"  Total:    {r.prompt_tokens + r.generated_tokens:6d} tokens in {total_ms:8.1f} ms", file=sys.stderr)
         print(f"  Load:     {load_ms:8.1f} ms", file=sys.stderr)
-        # against the MI355X's published peaks: the prompt step's flops, and the bytes the decode steps had to read
+        # against the GPU's published peaks: the prompt step's flops, and the bytes the decode steps had to read
+        hbm = (r.peaks or {}).get("hbm", 0.0)
         print(f"  Roofline: prefill {r.prefill_flops / max(r.prefill_seconds, 1e-12) / 1e12:7.1f} TFLOP/s "
               f"({r.prefill_fraction_of_peak:.3f} of the {r.dtype} matrix peak)  "
-              f"decode {r.decode_bytes_per_second / 1e9:7.1f} GB/s ({r.decode_fraction_of_peak:.3f} of 8 TB/s)",
+              f"decode {r.decode_bytes_per_second / 1e9:7.1f} GB/s "
+              + (f"({r.decode_fraction_of_peak:.3f} of {hbm / 1e12:g} TB/s)" if hbm else "(no published peak for this GPU)"),
               file=sys.stderr)
+        print(f"  Memory:   weights {model.step_weight_bytes() / 1e9:.2f} GB, packed copies "
+              f"{model.packed_weight_bytes() / 1e9:.2f} GB, cache {llm.engine.cache.bytes() / 1e9:.2f} GB", file=sys.stderr)
         return 0
 
     params = GenerationParams(max_tokens=args.max_tokens, temperature=args.temperature, top_k=args.top_k,

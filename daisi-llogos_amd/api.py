@@ -21,8 +21,20 @@ from .sampling.params import GenerationParams
 _ATTENTION_FORMS = re.compile(r"^(?:(full)|window:(\d+)|sinks:(\d+),(\d+))$")
 
 
-HBM_PEAK_BYTES = 8.0e12                                                    # MI355X, bytes a second
-MFMA_PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}                       # dense, flops a second
+# Published peaks by GPU architecture name: memory bytes a second, dense matrix flops a second by type.
+# A GPU that is not listed here has no peaks, and fractions of peak are reported as 0 for it.
+DEVICE_PEAKS = {
+    "gfx950": {"hbm": 8.0e12, "bf16": 2.5e15, "fp32": 157.3e12},           # MI355X
+}
+
+
+def device_peaks(device: Union[str, torch.device, int, None] = None) -> dict:
+    """The published peaks of the GPU `device` (the current one when None), {} when unknown."""
+    if not torch.cuda.is_available():
+        return {}
+    name = torch.cuda.get_device_properties(torch.device(device) if device is not None else torch.cuda.current_device())
+    arch = getattr(name, "gcnArchName", "").split(":")[0]
+    return DEVICE_PEAKS.get(arch, {})
 
 
 def parse_attention(value: str) -> Tuple[Optional[int], int]:
@@ -51,6 +63,11 @@ class BenchmarkResult:
     prefill_flops: float = 0.0            # of the timed prompt step
     decode_bytes: float = 0.0             # every decode step's weights once + the cache of its live sequences
     dtype: str = "bf16"
+    peaks: Optional[dict] = None          # device_peaks() of the GPU it ran on; None: looked up when asked for
+
+    def _peak(self, key: str) -> float:
+        peaks = self.peaks if self.peaks is not None else device_peaks()
+        return float(peaks.get(key, 0.0))
 
     @property
     def prefill_tokens_per_second(self) -> float:
@@ -62,8 +79,9 @@ class BenchmarkResult:
 
     @property
     def prefill_fraction_of_peak(self) -> float:
-        """Flops of the prompt step / its time / the MI355X's published dense matrix peak for the type."""
-        peak = MFMA_PEAK_FLOPS.get(self.dtype, 0.0)
+        """Flops of the prompt step / its time / the GPU's published dense matrix peak for the type (0 for
+        a GPU whose peaks are not known)."""
+        peak = self._peak(self.dtype)
         return self.prefill_flops / self.prefill_seconds / peak if self.prefill_seconds > 0 and peak else 0.0
 
     @property
@@ -72,8 +90,10 @@ class BenchmarkResult:
 
     @property
     def decode_fraction_of_peak(self) -> float:
-        """Bytes the decode steps had to read / their time / the MI355X's published memory bandwidth."""
-        return self.decode_bytes_per_second / HBM_PEAK_BYTES
+        """Bytes the decode steps had to read / their time / the GPU's published memory bandwidth (0 for a
+        GPU whose peaks are not known)."""
+        peak = self._peak("hbm")
+        return self.decode_bytes_per_second / peak if peak else 0.0
 
 
 class Llogos:
@@ -92,9 +112,11 @@ class Llogos:
         if window is not None:
             options = dict(attention_window=window - sinks, attention_sinks=sinks)
         pool = max_tokens_in_cache or max_batch * pages_for(max_context) * PAGE_TOKENS
-        self.max_context, self.max_batch = max_context, max_batch
+        self.max_batch = max_batch
         self.engine = Engine.from_folder(model, dtype=dtype, max_tokens=pool, n_slots=max(max_batch, 1),
                                          device=device, max_seq=max_context, **options)
+        # the engine keeps the limit within the positions the model was made for
+        self.max_context = self.engine.max_seq or max_context
         self.config = self.engine.config
         self._generator = Generator(self.engine, max_batch=max_batch, synchronize=torch.cuda.synchronize)
 
@@ -110,7 +132,8 @@ class Llogos:
         elif options:
             raise ValueError("give either params or keyword options")
         for i, p in enumerate(prompts):
-            if len(p) + params.max_tokens > self.max_context:
+            # the last generated token is not fed back: a request comes to hold len(p) + max_tokens - 1 positions
+            if len(p) + max(params.max_tokens, 1) - 1 > self.max_context:
                 raise ValueError(f"prompt {i} ({len(p)} tokens) plus max_tokens {params.max_tokens} exceeds "
                                  f"max_context {self.max_context}")
         return self._generator.generate(prompts, params, on_token=on_token)
@@ -136,4 +159,4 @@ class Llogos:
         flops = sum(model.step_flops([lens[r] for r in batch], wanted_rows=len(batch)) for batch in res.batches)
         return BenchmarkResult(res.prompt_tokens, res.generated_tokens, res.prefill_seconds, res.decode_seconds,
                                prefill_flops=flops, decode_bytes=decode_bytes,
-                               dtype="fp32" if self.engine.rt.is_f32 else "bf16")
+                               dtype="fp32" if self.engine.rt.is_f32 else "bf16", peaks=device_peaks(self.engine.rt.device))

@@ -7,6 +7,10 @@ from typing import Dict, List
 # Positions a page holds.  This is the definition; the kernel library has the same number
 # compiled in (kPageTokens) and loading it fails if the two differ.
 PAGE_TOKENS = 64
+# A page holds a head's keys and values in fragments of 16 dimensions (key_offset, value_offset):
+# head sizes are multiples of this, up to the most the attention kernels take.
+HEAD_DIM_STEP = 16
+MAX_HEAD_DIM = 512
 
 
 class CacheError(RuntimeError):

@@ -166,6 +166,13 @@ class DenseDecoderConfig:
             raise ConfigError(
                 f"config: num_attention_heads ({self.num_attention_heads}) must be a multiple of "
                 f"num_key_value_heads ({self.num_key_value_heads})")
+        from ..cache.pages import HEAD_DIM_STEP, MAX_HEAD_DIM
+        if self.head_dim % HEAD_DIM_STEP or self.head_dim > MAX_HEAD_DIM:
+            how = "given as 'head_dim'" if self.head_dim * self.num_attention_heads != self.hidden_size else \
+                f"hidden_size {self.hidden_size} / num_attention_heads {self.num_attention_heads}"
+            raise ConfigError(f"config: 'head_dim' ({self.head_dim}, {how}) must be a multiple of {HEAD_DIM_STEP}, "
+                              f"at most {MAX_HEAD_DIM}: the cache's pages and the attention kernels work in "
+                              f"fragments of {HEAD_DIM_STEP} dimensions")
         if self.rotary_dim <= 0 or self.rotary_dim % 2 != 0 or self.rotary_dim > self.head_dim:
             raise ConfigError(f"config: rotary dimension {self.rotary_dim} must be even and within head_dim")
         if not self.rms_norm_eps > 0:

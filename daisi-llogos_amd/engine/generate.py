@@ -159,6 +159,7 @@ class Generator:
         their share of the cache allows: one that has its last permitted token coming is not
         stepped ahead."""
         eng = self.engine
+        lend = {"borrow": True} if getattr(eng, "lends_logits", False) else {}
         live = list(batch)
         need_history = params.has_penalties
         history = (lambda rs: [recent_tokens(prompts[r], result.tokens[r], params.penalty_count) for r in rs]) \
@@ -177,8 +178,9 @@ class Generator:
             ahead = [(r, i) for r, i in rows if len(result.tokens[r]) + 1 < params.max_tokens]
             logits = None
             if ahead:
+                # (the sampler reads these logits before the next step is queued: they may be the step's own buffer)
                 logits = eng.step([(slots[r], [0]) for r, _ in ahead], want="last",
-                                  device_ids=(ids, [i for _, i in ahead]))
+                                  device_ids=(ids, [i for _, i in ahead]), **lend)
             toks = fetch()
             if t1 is None and fetch is fetch_first:                       # the prompt step has ended
                 t1 = time.perf_counter()

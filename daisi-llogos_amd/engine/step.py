@@ -49,11 +49,15 @@ def resolve_dtype(dtype: Union[str, torch.dtype]) -> torch.dtype:
 
 def packed_weight_budget(model: Model, dtype: torch.dtype, max_tokens: int, device: torch.device) -> int:
     """Bytes that the packed copies of the bfloat16 matrices may take (the few-row products stream
-    a packed copy a quarter faster; prompts need the row-major one): what is left of 85 % of the
-    GPU's memory beside the matrices themselves and the cache.  At the Llama-3.1-70B sizes, 141 GB
-    of matrices, about two thirds of the layers get their packed copy; smaller models all."""
+    a packed copy a quarter faster; prompts need the row-major one): what is free on the GPU now,
+    when the model is about to be bound, less the matrices themselves and the cache, which are
+    still to be allocated, and less a margin of 15 % of the GPU's memory for activations and
+    workspaces.  At the Llama-3.1-70B sizes, 141 GB of matrices, about two thirds of the layers get
+    their packed copy; smaller models all.  Whatever else lives on the GPU (another engine in the
+    same process, another process) is not counted on: only free memory is."""
     if dtype != torch.bfloat16:
         return 0
+    element = torch.empty((), dtype=dtype).element_size()
     elements = 0
     for spec in model.tensor_specs():
         if spec.kind in ("matrix", "table"):
@@ -61,9 +65,11 @@ def packed_weight_budget(model: Model, dtype: torch.dtype, max_tokens: int, devi
             for d in spec.shape:
                 n *= int(d)
             elements += n
-    cache = max_tokens * sum(2 * kv.n_kv_heads * kv.head_dim * 2 for kv, _ in model.cache_needs() if kv is not None)
-    total = torch.cuda.get_device_properties(device).total_memory
-    return max(0, int(0.85 * total) - 2 * elements - cache)
+    cache = max_tokens * sum(2 * kv.n_kv_heads * kv.head_dim * element for kv, _ in model.cache_needs() if kv is not None)
+    with torch.cuda.device(device):
+        free, total = torch.cuda.mem_get_info()
+        free += torch.cuda.memory_reserved() - torch.cuda.memory_allocated()      # what torch holds but does not use
+    return max(0, int(free - 0.15 * total) - element * elements - cache)
 
 
 def _packing(rt: Runtime, model: Model, max_tokens: int, pack_weights: Optional[bool]) -> None:
@@ -86,8 +92,9 @@ class Engine:
     """A bound model with its cache.  `step` is the only way tokens reach the model."""
 
     def __init__(self, model: Model, rt: Runtime, max_tokens: int, n_slots: int = 64, config=None,
-                 use_graphs: Optional[bool] = None, max_seq: Optional[int] = None):
+                 use_graphs: Optional[bool] = None, max_seq: Optional[int] = None, architecture: str = ""):
         self.model, self.rt, self.config = model, rt, config
+        self.architecture = architecture or type(model).__name__      # the registry name the model was built under
         # The longest a sequence may become: the caller's limit (the reference's --max-context,
         # Daisi.Llogos.Cli/Program.cs:194-197, 805) within the positions the model was made for
         # (max_position_embeddings); a step that would go beyond is refused, nothing runs.
@@ -127,7 +134,7 @@ class Engine:
                 torch.cuda.synchronize()
         finally:
             ckpt.close()
-        return cls(model, rt, max_tokens, n_slots, config, use_graphs, max_seq)
+        return cls(model, rt, max_tokens, n_slots, config, use_graphs, max_seq, arch.name)
 
     @classmethod
     def from_config(cls, config: dict, seed: int = 0, dtype: Union[str, torch.dtype] = "bfloat16",
@@ -154,7 +161,7 @@ class Engine:
         with torch.cuda.device(dev):
             model.bind(get, rt)
             torch.cuda.synchronize()
-        return cls(model, rt, max_tokens, n_slots, typed, use_graphs, max_seq)
+        return cls(model, rt, max_tokens, n_slots, typed, use_graphs, max_seq, arch.name)
 
     # ---- slots ---------------------------------------------------------------------
     def _graph_slots(self) -> int:
@@ -175,10 +182,13 @@ class Engine:
     # ---- the step --------------------------------------------------------------------
     # single-token steps can take their token ids from device memory (`device_ids`)
     takes_device_ids = True
+    # step(..., borrow=True) may return a buffer that the next step overwrites
+    lends_logits = True
 
     def step(self, entries: Sequence[Tuple[int, Sequence[int]]],
              want: Union[str, Sequence[Sequence[int]], None] = "last",
-             device_ids: Optional[Tuple[torch.Tensor, Sequence[int]]] = None) -> Optional[torch.Tensor]:
+             device_ids: Optional[Tuple[torch.Tensor, Sequence[int]]] = None,
+             borrow: bool = False) -> Optional[torch.Tensor]:
         """entries: (slot, next tokens) for each sequence of the batch.  want: 'last', 'all',
         None, or for each entry the places among its tokens whose logits are asked for.
         Returns float32 logits [wanted places, vocab] in the order of the entries and of
@@ -187,7 +197,11 @@ class Engine:
         device_ids = (ids, rows): every entry brings one token, and entry i's token is
         ids[rows[i]] of an int32 vector on the device (what a sampler wrote after an earlier
         step); the tokens in `entries` are then placeholders.  The host need not know the
-        tokens, so the step can be queued while the earlier one still runs."""
+        tokens, so the step can be queued while the earlier one still runs.
+
+        borrow: the caller is done with the logits (on the device, in stream order) before it
+        asks for the next step, so a replayed step may hand out its own output buffer, which the
+        next replay overwrites, instead of a copy (33 MB a step at batch 64 and 128,256 tokens)."""
         if not entries:
             raise StepError("a step needs at least one sequence")
         slot_ids = [int(s) for s, _ in entries]
@@ -220,7 +234,7 @@ class Engine:
 
         self.cache.reserve(slot_ids, new_lens)
         try:
-            logits = self._run(ids, counts, cu, rows, slot_ids, starts, new_lens, device_ids)
+            logits = self._run(ids, counts, cu, rows, slot_ids, starts, new_lens, device_ids, borrow)
         except BaseException:
             self.cache.unreserve(slot_ids)             # the sequences are as long as before, and hold no page more
             raise
@@ -228,7 +242,7 @@ class Engine:
         self.steps_run += 1
         return logits
 
-    def _run(self, ids, counts, cu, rows, slot_ids, starts, new_lens, device_ids) -> torch.Tensor:
+    def _run(self, ids, counts, cu, rows, slot_ids, starts, new_lens, device_ids, borrow=False) -> torch.Tensor:
         T, B = int(cu[-1]), len(counts)
         # (more rows than the hand-written products take would put a library call into the graph)
         if self.graphs is not None and T == B and B <= GRAPH_MAX_BATCH and rows == list(range(B)) \
@@ -237,7 +251,8 @@ class Engine:
                 logits = self.graphs.step(ids.astype(np.int32), np.asarray(starts, dtype=np.int32),
                                           np.asarray(slot_ids, dtype=np.int32), self.cache.step_tables(slot_ids),
                                           device_ids)
-                logits = logits.clone()          # the graph's own buffer is overwritten by its next replay
+                if not borrow:
+                    logits = logits.clone()      # the graph's own buffer is overwritten by its next replay
             return logits
         tok_seq = np.repeat(np.arange(B, dtype=np.int32), counts)
         tok_pos = np.concatenate([np.arange(s, s + c, dtype=np.int32) for s, c in zip(starts, counts)])

@@ -161,12 +161,29 @@ class Model:
         else:
             self.head.bind(get, rt)
 
+    def describe(self) -> str:
+        """One line about the built model, from its own parts: layers, widths, vocabulary, and the
+        heads of the mixers that have any (no field of an architecture's configuration is asked for)."""
+        s = self.spec
+        text = f"{len(self.layers)} layers"
+        if len(self.schedule) != len(self.layers):
+            text += f" in {len(self.schedule)} runs"
+        text += f", hidden {s.hidden_size}"
+        heads = sorted({(m.n_heads, getattr(m, "n_kv_heads", m.n_heads)) for m in self.unit_mixers if hasattr(m, "n_heads")})
+        if heads:
+            text += ", " + " and ".join(f"{q}/{kv}" for q, kv in heads) + " heads"
+        return text + f", vocab {s.vocab_size}"
+
     # ---- what a step costs -----------------------------------------------------
     def step_weight_bytes(self) -> int:
         """Bytes of weights a step reads once: every scheduled run of a layer, the final norm and
         the head (of the embedding table a step reads a row a token, which is not counted)."""
         runs = sum(self.layers[e.layer].weight_bytes() for e in self.schedule)
         return runs + self.final_norm.weight_bytes() + self.head.weight_bytes()
+
+    def packed_weight_bytes(self) -> int:
+        """Bytes of device memory that the packed second copies of the matrices take (each layer once)."""
+        return sum(layer.packed_bytes() for layer in self.layers) + self.head.packed_bytes()
 
     def step_flops(self, lens: List[int], starts: Optional[List[int]] = None, wanted_rows: int = 0) -> float:
         """Floating-point operations of a step that brings lens[i] tokens to sequence i, which

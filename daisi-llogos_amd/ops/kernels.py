@@ -13,11 +13,10 @@ from typing import Optional, Sequence, Tuple
 import torch
 
 from . import library
-from ..cache.pages import PAGE_TOKENS      # the one definition; the library is checked against it when loaded
+from ..cache.pages import HEAD_DIM_STEP, MAX_HEAD_DIM, PAGE_TOKENS      # the one definition; the library is checked against PAGE_TOKENS when loaded
 
 F32, BF16 = 0, 1
 _DT = {torch.float32: F32, torch.bfloat16: BF16}
-MAX_HEAD_DIM = 512
 MAX_BANNED = 64             # ids one sampling call can set to -inf (kMaxBanned in csrc/sampling.hip)
 
 

@@ -140,8 +140,10 @@ def build(verbose: bool = True) -> str:
     # an empty or unwritable HOME must not stop the compiler from keeping its temporaries
     env.setdefault("TMPDIR", tempfile.gettempdir())
     srcs = sources()
-    obj_dir = os.path.join(out_dir, "obj")
-    os.makedirs(obj_dir, exist_ok=True)
+    # every build has object files of its own: two processes that build at once (test workers that
+    # both find a stale library) must not link each other's half-written objects
+    obj_dir = tempfile.mkdtemp(prefix=f"obj.{os.getpid()}.", dir=out_dir)
+    stamp = _source_hash()                               # of the sources as they are now, before they are compiled
     if verbose:
         _log(f"building {LIB_NAME} for {ARCH} from {len(srcs)} sources into {out_dir}")
     t0 = time.time()
@@ -158,19 +160,80 @@ def build(verbose: bool = True) -> str:
         return obj
 
     workers = max(1, min(len(srcs), int(os.environ.get("MAX_JOBS", os.cpu_count() or 4)), 16))
-    with ThreadPoolExecutor(max_workers=workers) as pool:
-        objs = list(pool.map(compile_one, srcs))
     tmp_lib = os.path.join(out_dir, f".{LIB_NAME}.{os.getpid()}")
-    _run_with_progress([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", tmp_lib, *objs], "link", env)
+    tmp_stamp = os.path.join(out_dir, f".sources.sha256.{os.getpid()}")
     lib_path = os.path.join(out_dir, LIB_NAME)
-    os.replace(tmp_lib, lib_path)
-    with open(os.path.join(out_dir, "sources.sha256"), "w") as fh:
-        fh.write(_source_hash())
+    try:
+        with ThreadPoolExecutor(max_workers=workers) as pool:
+            objs = list(pool.map(compile_one, srcs))
+        _run_with_progress([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", tmp_lib, *objs], "link", env)
+        with open(tmp_stamp, "w") as fh:
+            fh.write(stamp)
+        # A reader must never see a library under a stamp that is not its own: the old stamp is taken
+        # away first (a library without a stamp counts as stale), then the library is put in place,
+        # then its stamp; both are written beside their places and renamed, so neither is ever half there.
+        try:
+            os.remove(os.path.join(out_dir, "sources.sha256"))
+        except OSError:
+            pass
+        os.replace(tmp_lib, lib_path)
+        os.replace(tmp_stamp, os.path.join(out_dir, "sources.sha256"))
+    finally:
+        shutil.rmtree(obj_dir, ignore_errors=True)
+        for leftover in (tmp_lib, tmp_stamp):
+            try:
+                os.remove(leftover)
+            except OSError:
+                pass
     if verbose:
         _log(f"built {lib_path} in {time.time() - t0:.0f} s")
     global _lib
     _lib = None
     return lib_path
+
+
+_C_TYPES = {"int": ctypes.c_int, "float": ctypes.c_float, "double": ctypes.c_double, "long long": ctypes.c_longlong,
+            "unsigned": ctypes.c_uint, "hipStream_t": ctypes.c_void_p}
+
+
+def exported_signatures() -> dict:
+    """name -> (result type, [argument types]) of every entry point, read from the sources'
+    LLOGOS_EXPORT declarations (pointers of any kind are c_void_p).  An entry point whose
+    declaration uses a type this does not know raises: a wrong guess would pass wrong bits."""
+    import re
+    found = {}
+    for name in sources():
+        with open(os.path.join(_CSRC, name)) as fh:
+            text = fh.read()
+        for m in re.finditer(r"LLOGOS_EXPORT\s+([\w\s\*]+?)\s*\b(\w+)\s*\(([^)]*)\)", text):
+            ret, fn, args = m.groups()
+
+            def ctype(decl: str, named: bool):
+                decl = " ".join(decl.replace("*", " * ").split())
+                if "*" in decl:
+                    return ctypes.c_void_p
+                words = [w for w in decl.split() if w != "const"]
+                if named and len(words) > 1:
+                    words = words[:-1]                       # the parameter's name
+                key = " ".join(words)
+                if key not in _C_TYPES:
+                    raise KernelLibraryError(f"{name}: entry point {fn} uses the type '{key}', which has no ctypes counterpart here")
+                return _C_TYPES[key]
+            arg_list = [a for a in (x.strip() for x in args.split(",")) if a and a != "void"]
+            found[fn] = (ctype(ret, False), [ctype(a, True) for a in arg_list])
+    return found
+
+
+def declare(lib: ctypes.CDLL) -> None:
+    """Argument and result types for every entry point, so that a call with too few arguments,
+    an integer that does not fit or a tensor where a number belongs raises instead of passing
+    wrong bits to a kernel."""
+    for fn, (ret, args) in exported_signatures().items():
+        try:
+            f = getattr(lib, fn)
+        except AttributeError:
+            raise KernelLibraryError(f"the library has no entry point {fn}, which the sources declare") from None
+        f.restype, f.argtypes = ret, args
 
 
 def is_stale(lib_path: str) -> bool:
@@ -204,7 +267,7 @@ def load() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
     except OSError as e:
         raise KernelLibraryError(f"cannot load {path}: {e}") from e
-    lib.llogos_attn_decode_workspace.restype = ctypes.c_longlong       # every other entry returns an int code
+    declare(lib)
     from ..cache.pages import PAGE_TOKENS, key_offset, value_offset
     if lib.llogos_page_tokens() != PAGE_TOKENS:
         raise KernelLibraryError(f"{path} was built for pages of {lib.llogos_page_tokens()} positions, "

@@ -119,6 +119,17 @@ class Part:
                 total += sum(x.weight_bytes() for x in v if isinstance(x, Part))
         return total
 
+    def packed_bytes(self) -> int:
+        """Bytes of the second copies of matrices (in the matrix cores' operand order) that this
+        part and its sub-parts hold beside what weight_bytes() counts."""
+        total = 0
+        for v in vars(self).values():
+            if isinstance(v, Part):
+                total += v.packed_bytes()
+            elif isinstance(v, (list, tuple)):
+                total += sum(x.packed_bytes() for x in v if isinstance(x, Part))
+        return total
+
     def matrix_elements(self) -> int:
         """Elements of the matrices this part multiplies every token with (two flops each)."""
         total = 0

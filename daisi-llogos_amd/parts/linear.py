@@ -69,7 +69,18 @@ class Linear(Part):
             if need > rt.pack_budget:
                 return
             rt.pack_budget -= need
-        self.packed = K.pack_weights(self.weight, self.out_features[0] if self.gated else 0)
+        try:
+            self.packed = K.pack_weights(self.weight, self.out_features[0] if self.gated else 0)
+        except torch.cuda.OutOfMemoryError:
+            # no room for this copy after all (memory taken since the budget was worked out): the
+            # matrix keeps the row-major kernels, which give the same sums in the same order
+            self.packed = None
+            if rt.pack_budget is not None:
+                rt.pack_budget = 0
+
+    def packed_bytes(self) -> int:
+        """Bytes of the packed copy that this product holds beside the matrix (0 without one)."""
+        return 0 if self.packed is None else self.packed.data.numel() * self.packed.data.element_size()
 
     def _packed_rows(self, rows_out: Optional[int]) -> Optional[K.PackedWeight]:
         if self.packed is None or rows_out is None:

@@ -324,11 +324,12 @@ def argmax_first(values) -> int:
 def sample(logits, u: float, temperature: float = 0.8, top_k: int = 40, top_p: float = 0.95,
            repetition_penalty: float = 1.1, frequency_penalty: float = 0.0, presence_penalty: float = 0.0,
            min_p: float = 0.0, typical_p: float = 1.0, penalty_count: int = 64, min_keep: int = 1,
-           penalize_newline: bool = False, history=()) -> int:
+           penalize_newline: bool = False, history=(), candidates_out=None) -> int:
     """The reference's pipeline, Daisi.Llogos/Inference/Sampler.cs:26-85, with the uniform
     draw `u` given by the caller: penalties (:89-143), greedy short cut (:56-57), temperature
     (:60-62), top-k (:249-276), min-p (:157-174), softmax over candidates (:278-295),
-    typical-p (:182-230), top-p (:297-332), draw (:334-345).  float32 as in the reference."""
+    typical-p (:182-230), top-p (:297-332), draw (:334-345).  float32 as in the reference.
+    candidates_out: a list that receives the ids the draw chooses among (every id some `u` gives)."""
     work = np.array(logits, dtype=np.float32)
     n = len(work)
     f32 = np.float32
@@ -352,6 +353,8 @@ def sample(logits, u: float, temperature: float = 0.8, top_k: int = 40, top_p: f
                 work[t] -= f32(frequency_penalty) * f32(c)
                 work[t] -= f32(presence_penalty)
     if temperature == 0:
+        if candidates_out is not None:
+            candidates_out.append(argmax_first(work))
         return argmax_first(work)
     work = work * (f32(1.0) / f32(temperature))
     k = top_k if 0 < top_k < n else n
@@ -400,6 +403,8 @@ def sample(logits, u: float, temperature: float = 0.8, top_k: int = 40, top_p: f
         if s > 0:
             for c in cand:
                 probs[c] = f32(probs[c] / s)
+    if candidates_out is not None:
+        candidates_out.extend(cand)
     cum = 0.0
     for c in cand:
         cum += float(probs[c])

@@ -100,3 +100,12 @@ def test_a_library_built_from_other_sources_is_not_loaded(tmp_path, monkeypatch)
     with pytest.raises(library.KernelLibraryError, match="cannot load"):
         library.load()
     assert calls == [1]
+
+
+def test_fractions_of_peak_are_zero_for_a_gpu_without_published_peaks():
+    r = api.BenchmarkResult(100, 50, 0.1, 0.5, prefill_flops=1e12, decode_bytes=1e9, peaks={})
+    assert r.prefill_fraction_of_peak == 0.0 and r.decode_fraction_of_peak == 0.0
+    assert r.decode_bytes_per_second == 2e9 and r.prefill_tokens_per_second == 1000
+    known = api.BenchmarkResult(100, 50, 0.1, 0.5, prefill_flops=1e12, decode_bytes=1e9, peaks=api.DEVICE_PEAKS["gfx950"])
+    assert known.decode_fraction_of_peak == 2e9 / 8e12 and known.prefill_fraction_of_peak == 1e13 / 2.5e15
+    assert api.device_peaks() == {} or "hbm" in api.device_peaks()      # no GPU here: nothing is assumed

@@ -71,6 +71,14 @@ def test_wrong_types_and_sizes(llogos):
         read(num_key_value_heads=3)
     with pytest.raises(llogos.ConfigError, match="head_dim"):
         read(hidden_size=66)                                            # 66 / 4 heads and no head_dim
+    # head sizes are refused where the configuration is read, with the key's name: a multiple of 16 ...
+    with pytest.raises(llogos.ConfigError, match=r"'head_dim' \(40, hidden_size 320 / num_attention_heads 8\) must be a multiple of 16"):
+        read(hidden_size=320, num_attention_heads=8, num_key_value_heads=8)
+    with pytest.raises(llogos.ConfigError, match=r"'head_dim' \(24, given as 'head_dim'\)"):
+        read(head_dim=24)
+    with pytest.raises(llogos.ConfigError, match="at most 512"):
+        read(head_dim=528)                                              # ... within what the attention kernels take
+    assert read(head_dim=48).head_dim == 48
     with pytest.raises(llogos.ConfigError, match="rms_norm_eps"):
         read(rms_norm_eps=0)
     with pytest.raises(llogos.ConfigError, match="hidden_act"):

@@ -359,9 +359,6 @@ class ToyConfig:
     hidden_size: int
     n_layers: int
     architecture: str = "ToyStateForCausalLM"
-    num_hidden_layers: int = 0
-    num_attention_heads: int = 2
-    num_key_value_heads: int = 1
 
 
 def _toy_spec(cfg, **kw):
@@ -448,6 +445,27 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
         s = eng.alloc_slot(); eng.step([(s, [1, 2, 3])]); eng.cache.truncate(s, 1)
 
 
+def test_the_command_line_runs_a_toy_architecture(tmp_path, capsys):
+    """The command line describes and runs a model from what the built model says of itself: the toy
+    configuration has none of the dense decoder's fields."""
+    cli = importlib.import_module("daisi-llogos_amd.__main__")
+    from safetensors.torch import load_file
+    cfg = {"architectures": ["ToyStateForCausalLM"], "vocab_size": 90, "hidden_size": 40, "n_layers": 3,
+           "torch_dtype": "float32"}
+    folder = L.write_random_model(str(tmp_path / "toy"), cfg, seed=2)
+    w = {k: v.double().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    prompt = [5, 17, 3, 80, 41]
+    assert cli.main(["--model", folder, "--prompt", " ".join(map(str, prompt)), "-n", "6", "-t", "0",
+                     "--repeat-penalty", "1.0", "--dtype", "float32", "--max-context", "64"]) == 0
+    io = capsys.readouterr()
+    assert "Loaded ToyStateForCausalLM: 3 layers, hidden 40, 2/1 heads, vocab 90" in io.err
+    got = [int(t) for t in io.out.split()]
+    seq = list(prompt)
+    for _ in range(6):
+        seq.append(int(np.argmax(_plain_toy(w, seq, 3)[-1])))
+    assert got == seq[len(prompt):]
+
+
 # ---------------------------------------------------------------------------
 # a toy feed-forward with routing and a toy position encoding, defined here
 # ---------------------------------------------------------------------------
@@ -503,9 +521,6 @@ class RoutedConfig:
     vocab_size: int
     hidden_size: int
     n_layers: int
-    num_hidden_layers: int = 0
-    num_attention_heads: int = 4
-    num_key_value_heads: int = 2
 
 
 def _routed_spec(cfg, **kw):
@@ -622,9 +637,6 @@ class TwoMixerConfig:
     vocab_size: int
     hidden_size: int
     n_layers: int
-    num_hidden_layers: int = 0
-    num_attention_heads: int = 2
-    num_key_value_heads: int = 1
 
 
 def _two_mixer_spec(cfg, **kw):
@@ -792,6 +804,60 @@ def test_captured_steps_of_a_mixer_with_state_advance_the_state_once(tmp_path):
         assert np.array_equal(outs[0], outs[1]), f"token {t}: replayed and launched steps differ by {np.abs(outs[0] - outs[1]).max()}"
         H.close(outs[0], np.stack([want[i][cut[i] + t] for i in live]), "float32", f"state on device, token {t}")
     assert len(engines[0].graphs.graphs) == 2
+
+
+def test_a_slot_beyond_the_first_count_between_replays_of_a_captured_step(tmp_path):
+    """The cache starts with two slots.  Two sequences are stepped through captured graphs; then a
+    third sequence takes a slot the cache did not have, which makes the per-slot state tensors
+    anew (the captured graphs hold the old ones' addresses and must be dropped), and all three go
+    on.  Replayed steps against launched ones bit for bit, and against the plain running mean: a
+    graph that still wrote the old state tensor, or a state that did not move with its slot,
+    would show at the first token after the growth."""
+    from safetensors.torch import load_file
+    cfg = {"architectures": ["ToyStateOnDeviceForCausalLM"], "vocab_size": 60, "hidden_size": 40, "n_layers": 2,
+           "torch_dtype": "float32"}
+    folder = L.write_random_model(str(tmp_path / "grow"), cfg, seed=12)
+    w = {k: v.double().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+
+    def plain(tokens):
+        x = pm.embedding(w["embed.weight"], tokens)
+        for i in range(2):
+            p = f"layers.{i}."
+            n = pm.rms_norm(x, w[p + "n1.weight"], 1e-6)
+            x = x + np.cumsum(n, axis=0) / np.arange(1, len(tokens) + 1)[:, None] * w[p + "gain.weight"]
+            n = pm.rms_norm(x, w[p + "n2.weight"], 1e-6)
+            x = x + pm.swiglu_mlp(n, w[p + "ffn.gate_proj.weight"], w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
+        return pm.linear(pm.rms_norm(x, w["norm.weight"], 1e-6), w["head.weight"])
+
+    engines = [L.Engine.from_folder(folder, dtype="float32", max_tokens=512, n_slots=2, use_graphs=g) for g in (True, False)]
+    rng = np.random.default_rng(6)
+    seqs = [rng.integers(0, 60, size=n).tolist() for n in (24, 20, 18)]
+    want = [plain(s) for s in seqs]
+    cut = [7, 3, 5]
+    slots = [[e.alloc_slot() for _ in range(2)] for e in engines]
+    for e, sl in zip(engines, slots):
+        e.step([(s, q[:c]) for s, q, c in zip(sl, seqs, cut)], want=None)
+    fed = list(cut)
+
+    def one_token_each(live, what):
+        outs = [_np(e.step([(sl[i], [seqs[i][fed[i]]]) for i in live], want="last")) for e, sl in zip(engines, slots)]
+        assert np.array_equal(outs[0], outs[1]), f"{what}: replayed and launched steps differ by {np.abs(outs[0] - outs[1]).max()}"
+        H.close(outs[0], np.stack([want[i][fed[i]] for i in live]), "float32", what)
+        for i in live:
+            fed[i] += 1
+
+    for t in range(4):
+        one_token_each([0, 1], f"two sequences, token {t}")
+    held = engines[0].cache.states[0]
+    assert engines[0].cache.slots.n_slots == 2 and len(engines[0].graphs.graphs) == 1
+    for e, sl in zip(engines, slots):
+        sl.append(e.alloc_slot())                                           # the third slot: the cache grows
+        e.step([(sl[2], seqs[2][:cut[2]])], want=None)
+    assert engines[0].cache.slots.n_slots > 2 and engines[0].cache.states[0] is not held
+    for t in range(6):
+        one_token_each([0, 1, 2], f"three sequences after the growth, token {t}")
+    one_token_each([2, 0], "two of them, in another order")
+    assert set(engines[0].graphs.graphs) == {(3, ()), (2, ())}             # the graphs of before the growth are gone
 
 
 # ---------------------------------------------------------------------------

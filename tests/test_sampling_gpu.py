@@ -96,23 +96,54 @@ def test_large_vocabulary_and_batch_rows_are_independent():
         assert tok in np.argsort(-row)[:40]
 
 
-def test_prevent_eos_and_sampled_generation():
+TINY_B_RUN = dict(max_tokens=24, temperature=0.8, seed=1234, stop_tokens=())      # 3 prompts of 40 / 3 / 9 tokens
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+@pytest.mark.parametrize("filters", [dict(top_k=0, top_p=1.0, repetition_penalty=1.0),            # temperature alone
+                                     dict(top_k=40, top_p=0.95, repetition_penalty=1.1)],          # the reference's defaults
+                         ids=["temperature", "defaults"])
+def test_sampled_generation_draw_by_draw(dtype, filters):
+    """Three prompts of 40, 3 and 9 tokens, 24 tokens each at temperature 0.8 with a fixed seed, through the
+    entry point; then every generated token again from the plain sampler on the plain logits of the
+    same context with the same uniform number (seed, request, index of the token).  float32: the same
+    token, but for at most one a sequence whose uniform number lies within rounding of a boundary of
+    the cumulative sum.  bfloat16 (logits differ by roundings, so a boundary may move past the
+    uniform number): every token is one the plain sampler chooses among, and most are the same."""
+    rng_mod = importlib.import_module("daisi-llogos_amd.sampling.rng")
+    name = "tiny_b"
+    llm = H.llogos.Llogos(H.folder(name), dtype=dtype, max_context=96, max_batch=3)
+    prompts = [list(H.tokens(name, n, 60 + n)) for n in (40, 3, 9)]
+    kw = dict(TINY_B_RUN, **filters)
+    got = llm.generate(prompts, **kw).tokens
+    assert [len(t) for t in got] == [24, 24, 24]
+    assert got == llm.generate(prompts, **kw).tokens                    # a fixed seed repeats
+    assert got != llm.generate(prompts, **dict(kw, seed=99)).tokens
+    cfg, w = H.plain(name)
+    same_all = 0
+    for r, (p, toks) in enumerate(zip(prompts, got)):
+        logits = pm.forward(cfg, w, p + toks)
+        same = 0
+        for i, t in enumerate(toks):
+            cands = []
+            want = pm.sample(logits[len(p) + i - 1], rng_mod.uniform(kw["seed"], r, i), temperature=kw["temperature"],
+                             top_k=kw["top_k"], top_p=kw["top_p"], repetition_penalty=kw["repetition_penalty"],
+                             history=(p + toks[:i]), candidates_out=cands)
+            assert t in cands, (dtype, r, i, t, want)
+            same += t == want
+        if dtype == "float32":
+            assert same >= len(toks) - 1, (r, same)
+        same_all += same
+    assert same_all >= 60, same_all                                     # of 72 (bfloat16: 66 to 70 when this was written)
+
+
+def test_prevent_eos():
     name = "tiny_b"
     llm = H.llogos.Llogos(H.folder(name), dtype="float32", max_context=96, max_batch=3)
-    prompts = [list(H.tokens(name, n, 60 + n)) for n in (40, 3, 9)]
-    kw = dict(max_tokens=24, temperature=0.8, top_k=40, top_p=0.95, repetition_penalty=1.1, seed=1234, stop_tokens=())
-    a = llm.generate(prompts, **kw).tokens
-    assert a == llm.generate(prompts, **kw).tokens                      # a fixed seed repeats
-    assert a != llm.generate(prompts, **dict(kw, seed=99)).tokens
-    # every sampled token is one the plain sampler could draw: within the top 40 of the plain logits
-    cfg, w = H.plain(name)
-    for p, toks in zip(prompts, a):
-        logits = pm.forward(cfg, w, p + toks)
-        for i, t in enumerate(toks):
-            row = logits[len(p) + i - 1].copy()
-            assert t in np.argsort(-row)[:60]
-    banned = a[0][0]
-    b = llm.generate([prompts[0]], max_tokens=8, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0,
+    prompt = list(H.tokens(name, 40, 100))
+    banned = llm.generate([prompt], max_tokens=1, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0,
+                          stop_tokens=()).tokens[0][0]
+    b = llm.generate([prompt], max_tokens=8, temperature=0.0, top_k=0, top_p=1.0, repetition_penalty=1.0,
                      stop_tokens=(banned,), prevent_eos=True).tokens[0]
     assert len(b) == 8 and banned not in b
 
