@@ -666,17 +666,47 @@ def gemm_packed_bf16(a: torch.Tensor, pw: PackedWeight, bias: Optional[torch.Ten
     return out
 
 
-# Which product serves more than 64 rows of bfloat16 (prompts): "library" (the default: the library's
-# product on the row-major matrix, as the reference uses a library there) or "tiles" (gemm_tiles_bf16
-# on the packed copy: hand-written, with the SwiGLU epilogue, measured at two thirds of the library's
-# speed at the 8B sizes).  LLOGOS_PROMPT_PRODUCT in the environment sets the default.
-PROMPT_PRODUCT = os.environ.get("LLOGOS_PROMPT_PRODUCT", "library")
+# Which product serves many rows of bfloat16 (prompts): "auto" (the default): the hand-written tiled
+# product (gemm_tiles_bf16 on the packed copy) where it was measured faster than the library's, which is
+# the gate/up product with its SwiGLU epilogue from TILES_MIN_ROWS rows on, and the library's product
+# elsewhere (as the reference uses a library there); "tiles": the hand-written one wherever it applies;
+# "library": the library's everywhere.  LLOGOS_PROMPT_PRODUCT in the environment sets the default.
+PROMPT_PRODUCT = os.environ.get("LLOGOS_PROMPT_PRODUCT", "auto")
+TILES_MIN_ROWS = 1024
 
 
-def gemm_tiles_bf16(a: torch.Tensor, pw: PackedWeight, bias: Optional[torch.Tensor], out_dtype: torch.dtype) -> Optional[torch.Tensor]:
-    """a [M, K] . w^T on the packed copy of w for any number of rows (tiles of 128 tokens x 256 rows,
+def tiles_serve_gated(M: int) -> bool:
+    """Whether the tiled product makes silu(gate) * up for M rows (rather than the library's product and a
+    SwiGLU pass)."""
+    return PROMPT_PRODUCT == "tiles" or (PROMPT_PRODUCT == "auto" and M >= TILES_MIN_ROWS)
+
+
+def tiles_plan(M: int, N: int, K: int) -> Optional[Tuple[int, int]]:
+    """(parts of k, token_tiles) with which the tiled product serves a plain product of M rows, or None where
+    the library's does.  Measured on the MI355X at the layer sizes of 8B, 14B and 70B models: a matrix that
+    is much longer than high (a feed-forward's down projection) with 129 to 1,024 rows of activations is where
+    the library is furthest from its best (14B, 256 rows: 119 us against 65; 70B: 291 against 143; 8B, 512 rows:
+    88 against 68), and blocks along k fill the compute units that its few row tiles leave idle.  Elsewhere
+    the library's product was level or ahead (by 10 to 25 % from 2,048 rows on)."""
+    if PROMPT_PRODUCT == "library" or M <= SKINNY_MAX_ROWS or K % 64:
+        return None
+    if PROMPT_PRODUCT == "tiles":
+        return 1, 0
+    if K >= 2 * N and LDS_MAX_ROWS < M <= 1024:
+        parts, token_tiles = (4, 2) if M <= 256 else ((4, 0) if M <= 512 else (2, 0))
+        while parts > 1 and (K // 64) // parts < 2:
+            parts //= 2
+        return parts, token_tiles
+    return None
+
+
+def gemm_tiles_bf16(a: torch.Tensor, pw: PackedWeight, bias: Optional[torch.Tensor], out_dtype: torch.dtype,
+                    parts: int = 1, token_tiles: int = 0) -> Optional[torch.Tensor]:
+    """a [M, K] . w^T on the packed copy of w for any number of rows (tiles of 256 or 128 tokens x 256 rows,
     v_mfma_f32_32x32x16_bf16): [M, N] with the bias added, or, for a matrix packed with gate_rows,
-    [M, gate_rows] = silu(gate) * up.  None for shapes it does not take (K no multiple of 64)."""
+    [M, gate_rows] = silu(gate) * up; with parts > 1 float32 partial sums [parts, M, N] over ranges of k.
+    token_tiles: 4 or 2 force tiles of 256 or 128 tokens, 0 lets the launch choose.
+    None for shapes it does not take (K no multiple of 64, parts of fewer than 128 values of k)."""
     if a.dtype != torch.bfloat16 or a.dim() != 2:
         return None
     M, K = a.shape
@@ -686,15 +716,21 @@ def gemm_tiles_bf16(a: torch.Tensor, pw: PackedWeight, bias: Optional[torch.Tens
     _dev(pw.data, bias)
     _need(a.is_cuda and a.device == pw.data.device, "gemm: a and w must be on the same GPU")
     _need(not (gated and bias is not None), "gemm: the gated product takes no bias")
+    _need(parts >= 1 and not (gated and parts > 1), "gemm: the gated product comes in one part")
     if bias is not None:
         _need(bias.dtype == torch.float32 and bias.shape == (pw.N,), "gemm: bias must be float32 [N]")
-    out = torch.empty((M, pw.gate_rows if gated else pw.N), dtype=out_dtype, device=a.device)
+        _need(parts == 1, "gemm: a product in parts leaves the bias to its consumer")
+    if parts > 1:
+        out_dtype = torch.float32
+    width = pw.gate_rows if gated else pw.N
+    out = torch.empty((parts, M, width), dtype=out_dtype, device=a.device)
     code = _lib().llogos_gemm_tiles_bf16(_p(out), _DT[out_dtype], _p(a), a.stride(0), _p(pw.data), _p(bias), M, pw.N, K,
-                                         out.stride(0), int(gated), 4, _stream())
+                                         width, ctypes.c_longlong(M * width), int(gated), int(parts), int(token_tiles),
+                                         compute_units(a.device), _stream())
     if code == -2:
         return None
     _check(code, "gemm_tiles_bf16")
-    return out
+    return out[0] if parts == 1 else out
 
 
 def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swiglu_input: bool = False,
@@ -707,7 +743,8 @@ def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swigl
 
     float32 operands: plain FMAs in 32-bit throughout.  bfloat16 operands: up to 64 rows the
     hand-written weight-streaming kernels (on the packed copy of w when there is one: `packed`),
-    up to 128 rows too where w is much longer than it has rows (see long_inner); otherwise the
+    up to 128 rows too where w is much longer than it has rows (see long_inner); for more rows the
+    hand-written tiled product where it was measured ahead (see tiles_plan); otherwise the
     library product (as the reference uses a library for its prompt products,
     Daisi.Llogos.Cuda/CudaBackend.cs:158-316)."""
     M = a.shape[-2]
@@ -762,8 +799,9 @@ def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swigl
                                    lds_splits(M, w.shape[0], w.shape[1]), 1)
         if out is not None:
             return out
-    if packed is not None and PROMPT_PRODUCT == "tiles" and M > SKINNY_MAX_ROWS and out_dtype == torch.bfloat16:
-        out = gemm_tiles_bf16(a, packed, None, torch.float32 if f32_ok else out_dtype)
+    plan = tiles_plan(M, packed.N, packed.K) if packed is not None else None
+    if plan is not None and out_dtype == torch.bfloat16 and a.dtype == torch.bfloat16 and a.dim() == 2:
+        out = gemm_tiles_bf16(a, packed, None, torch.float32 if f32_ok else out_dtype, parts=plan[0], token_tiles=plan[1])
         if out is not None:
             return out
     if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out_dtype == torch.bfloat16 and a.is_contiguous() \

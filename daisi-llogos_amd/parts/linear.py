@@ -104,11 +104,13 @@ class Linear(Part):
 
     def gated_product(self, a: torch.Tensor) -> Optional[torch.Tensor]:
         """silu(a . gate^T) * (a . up^T) as [M, out] in the runtime's type, made in one kernel from the
-        packed copy; None where that does not apply (no packed copy, more than 64 rows, float32)."""
+        packed copy (up to 64 rows the weight-streaming product, for prompts the tiled one); None where that
+        does not apply (no packed copy, float32, row counts at which the library's product and a SwiGLU pass
+        are faster)."""
         if self.packed is None or not self.packed.gate_rows or a.dim() != 2:
             return None
         if a.shape[0] > K.SKINNY_MAX_ROWS:
-            return K.gemm_tiles_bf16(a, self.packed, None, self.rt.dtype) if K.PROMPT_PRODUCT == "tiles" else None
+            return K.gemm_tiles_bf16(a, self.packed, None, self.rt.dtype) if K.tiles_serve_gated(a.shape[0]) else None
         return K.gemm_packed_gated_bf16(a, self.packed, self.rt.dtype, K.packed_plan(a.shape[0], self.packed.N, self.packed.K)[1])
 
     def bias_rows(self, rows_out: Optional[int] = None) -> Optional[torch.Tensor]:

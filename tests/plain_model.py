@@ -324,12 +324,14 @@ def argmax_first(values) -> int:
 def sample(logits, u: float, temperature: float = 0.8, top_k: int = 40, top_p: float = 0.95,
            repetition_penalty: float = 1.1, frequency_penalty: float = 0.0, presence_penalty: float = 0.0,
            min_p: float = 0.0, typical_p: float = 1.0, penalty_count: int = 64, min_keep: int = 1,
-           penalize_newline: bool = False, history=(), candidates_out=None) -> int:
+           penalize_newline: bool = False, history=(), candidates_out=None,
+           intervals_out=None) -> int:
     """The reference's pipeline, Daisi.Llogos/Inference/Sampler.cs:26-85, with the uniform
     draw `u` given by the caller: penalties (:89-143), greedy short cut (:56-57), temperature
     (:60-62), top-k (:249-276), min-p (:157-174), softmax over candidates (:278-295),
     typical-p (:182-230), top-p (:297-332), draw (:334-345).  float32 as in the reference.
-    candidates_out: a list that receives the ids the draw chooses among (every id some `u` gives)."""
+    candidates_out: a list that receives the ids the draw chooses among (every id some `u` gives);
+    intervals_out: a dict that receives id -> (lo, hi), the part of [0, 1) whose `u` draw that id."""
     work = np.array(logits, dtype=np.float32)
     n = len(work)
     f32 = np.float32
@@ -355,6 +357,8 @@ def sample(logits, u: float, temperature: float = 0.8, top_k: int = 40, top_p: f
     if temperature == 0:
         if candidates_out is not None:
             candidates_out.append(argmax_first(work))
+        if intervals_out is not None:
+            intervals_out[argmax_first(work)] = (0.0, 1.0)
         return argmax_first(work)
     work = work * (f32(1.0) / f32(temperature))
     k = top_k if 0 < top_k < n else n
@@ -405,6 +409,11 @@ def sample(logits, u: float, temperature: float = 0.8, top_k: int = 40, top_p: f
                 probs[c] = f32(probs[c] / s)
     if candidates_out is not None:
         candidates_out.extend(cand)
+    if intervals_out is not None:
+        lo = 0.0
+        for c in cand:
+            intervals_out[c] = (lo, lo + float(probs[c]))
+            lo += float(probs[c])
     cum = 0.0
     for c in cand:
         cum += float(probs[c])

@@ -652,31 +652,67 @@ def test_gate_up_product_with_the_swiglu_epilogue(M, I, H):
         K.pack_weights(w, gate_rows=I + 16)
 
 
-@pytest.mark.parametrize("M,N,K_", [(65, 256, 64), (300, 1000, 512), (2048, 4096, 4096), (129, 6144, 1024), (700, 130, 192)])
-def test_tiled_product_for_many_rows_on_packed_weights(M, N, K_):
-    """The hand-written prompt-size product (tiles of 128 tokens x 256 rows, 32x32x16 MFMAs on the
-    packed copy): token counts and heights that fill no tile, float32 and bfloat16 results, bias."""
+@pytest.mark.parametrize("M,N,K_", [(65, 256, 64), (300, 1000, 512), (2048, 4096, 4096), (129, 6144, 1024), (700, 130, 192),
+                                    (1500, 2300, 640)])
+@pytest.mark.parametrize("token_tiles", [0, 4, 2])
+def test_tiled_product_for_many_rows_on_packed_weights(M, N, K_, token_tiles):
+    """The hand-written prompt-size product (tiles of 256 or 128 tokens x 256 rows, 32x32x16 MFMAs on the
+    packed copy): token counts and heights that fill no tile, float32 and bfloat16 results, bias, parts of k."""
     rng = np.random.default_rng(M + N)
     a, w = _t(rng.standard_normal((M, K_)), torch.bfloat16), _t(rng.standard_normal((N, K_)) * 0.05, torch.bfloat16)
     bias = _t(rng.standard_normal(N))
     want = _np(a) @ _np(w).T
     pw = K.pack_weights(w)
-    _close(K.gemm_tiles_bf16(a, pw, None, torch.float32), want, "float32", scale=np.abs(want).max() * 10)
-    _close(K.gemm_tiles_bf16(a, pw, bias, torch.bfloat16), want + _np(bias), "bfloat16")
+    _close(K.gemm_tiles_bf16(a, pw, None, torch.float32, token_tiles=token_tiles), want, "float32", scale=np.abs(want).max() * 10)
+    _close(K.gemm_tiles_bf16(a, pw, bias, torch.bfloat16, token_tiles=token_tiles), want + _np(bias), "bfloat16")
     assert K.gemm_tiles_bf16(a[:, :K_ - 8].contiguous(), K.pack_weights(w[:, :K_ - 8].contiguous()), None, torch.float32) is None
+    for parts in (2, 3):
+        got = K.gemm_tiles_bf16(a, pw, None, torch.bfloat16, parts=parts, token_tiles=token_tiles)
+        if K_ // 64 // parts < 2:
+            assert got is None                                          # a part would hold less than two stages of 64
+            continue
+        assert got.shape == (parts, M, N) and got.dtype == torch.float32
+        if parts == 2:                                                  # the first part is the product over the first half of k
+            half = -(-(K_ // 64) // 2) * 64
+            _close(got[0], _np(a)[:, :half] @ _np(w)[:, :half].T, "float32", scale=np.abs(want).max() * 10)
+        _close(got.sum(0), want, "float32", scale=np.abs(want).max() * 10)
+        _close(K.sum_parts(got, bias, torch.float32), want + _np(bias), "float32", scale=np.abs(want).max() * 10)
 
 
-@pytest.mark.parametrize("M,I,H", [(200, 1008, 256), (2048, 14336, 4096), (65, 16, 64)])
+def test_tiled_product_cuts_the_last_round_into_smaller_tiles():
+    """2,048 tokens by 7,168 rows are 8 x 28 tiles of 256 tokens: on 64 compute units 224 tiles are three
+    rounds and a half, and the launch takes the row tiles of the half round in tiles of 128 tokens.  The
+    result does not depend on the cut (every element's sum runs over k in the same order)."""
+    rng = np.random.default_rng(3)
+    M, N, K_ = 2048, 7168, 256
+    a, w = _t(rng.standard_normal((M, K_)), torch.bfloat16), _t(rng.standard_normal((N, K_)) * 0.05, torch.bfloat16)
+    pw = K.pack_weights(w)
+    lib = K._lib()
+    outs = []
+    for units in (64, 256, 1):                    # 224 tiles: 3.5 rounds of 64 (cut), less than one round of 256, whole rounds of 1
+        out = torch.empty((M, N), dtype=torch.float32, device=a.device)
+        code = lib.llogos_gemm_tiles_bf16(K._p(out), K.F32, K._p(a), a.stride(0), K._p(pw.data), None, M, N, K_, N, M * N, 0, 1, 0,
+                                          units, K._stream())
+        assert code == 0
+        outs.append(out)
+    _close(outs[0], _np(a) @ _np(w).T, "float32", scale=np.abs(_np(a) @ _np(w).T).max() * 10)
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+
+
+@pytest.mark.parametrize("M,I,H", [(200, 1008, 256), (2048, 14336, 4096), (65, 16, 64), (1000, 7200, 320)])
 def test_tiled_product_with_the_swiglu_epilogue(M, I, H):
     rng = np.random.default_rng(M + I)
     wg, wu = (_t(rng.standard_normal((I, H)) * 0.08, torch.bfloat16) for _ in range(2))
     a = _t(rng.standard_normal((M, H)) * (0.25 if H > 1000 else 1.0), torch.bfloat16)
     pw = K.pack_weights(torch.cat([wg, wu]).contiguous(), gate_rows=I)
     want = pm.silu(_np(a) @ _np(wg).T) * (_np(a) @ _np(wu).T)
-    got = K.gemm_tiles_bf16(a, pw, None, torch.float32)
-    assert got.shape == (M, I)
-    _close(got, want, "float32", scale=np.abs(want).max() * 50)
-    _close(K.gemm_tiles_bf16(a, pw, None, torch.bfloat16), want, "bfloat16")
+    for token_tiles in (0, 4, 2):
+        got = K.gemm_tiles_bf16(a, pw, None, torch.float32, token_tiles=token_tiles)
+        assert got.shape == (M, I)
+        _close(got, want, "float32", scale=np.abs(want).max() * 50)
+        _close(K.gemm_tiles_bf16(a, pw, None, torch.bfloat16, token_tiles=token_tiles), want, "bfloat16")
+    with pytest.raises(K.KernelError):
+        K.gemm_tiles_bf16(a, pw, None, torch.float32, parts=2)
 
 
 def test_prompts_through_the_tiled_product(monkeypatch):
@@ -690,3 +726,24 @@ def test_prompts_through_the_tiled_product(monkeypatch):
     s = eng.alloc_slot()
     got = eng.step([(s, toks)], want="all").cpu().double().numpy()
     H.close(got, H.plain_logits(name, toks), "bfloat16", "prompt through the tiled product", config=name)
+
+
+def test_long_prompts_take_the_tiled_gate_up_product_by_default():
+    """From TILES_MIN_ROWS tokens on the gate/up product with its SwiGLU epilogue is the hand-written one;
+    the logits are the plain ones either way, and the two ways agree within bfloat16 rounding."""
+    import gpu_helpers as H
+    assert K.PROMPT_PRODUCT == "auto" and K.tiles_serve_gated(K.TILES_MIN_ROWS) and not K.tiles_serve_gated(K.TILES_MIN_ROWS - 1)
+    name = "layer_8b"
+    eng = H.engine(name, "bfloat16", max_tokens=64 * 18, n_slots=1)
+    toks = H.tokens(name, K.TILES_MIN_ROWS + 40, 2)
+    calls = []
+    real = K.gemm_tiles_bf16
+    K.gemm_tiles_bf16 = lambda *a, **kw: (calls.append((a[0].shape[0], a[1].gate_rows > 0)), real(*a, **kw))[1]
+    try:
+        s = eng.alloc_slot()
+        got = eng.step([(s, toks)], want=[[0, 100, len(toks) - 1]]).cpu().double().numpy()
+    finally:
+        K.gemm_tiles_bf16 = real
+    assert calls == [(len(toks), True)] * 2                                # the gate/up product of both layers
+    want = H.plain_logits(name, toks)[[0, 100, len(toks) - 1]]
+    H.close(got, want, "bfloat16", "long prompt, tiled gate/up product", config=name)

@@ -73,3 +73,23 @@ def test_sets_of_waves_of_the_prompt_attention():
         assert K.prefill_halves(lens, None, 32) == want, lens
     # a continued prompt counts the pages before it
     assert K.prefill_halves([128], [4000], 32) == 2 and K.prefill_halves([128] * 64, [4000] * 64, 32) == 1
+
+
+def test_where_the_tiled_product_serves_prompts(monkeypatch):
+    """By default the tiled product takes the gate/up product with its SwiGLU epilogue from TILES_MIN_ROWS rows
+    on, and plain products only for matrices much longer than high at 129 to 1,024 rows, in parts of k that
+    hold at least two stages of 64."""
+    assert K.PROMPT_PRODUCT == "auto"
+    assert K.tiles_serve_gated(K.TILES_MIN_ROWS) and not K.tiles_serve_gated(K.TILES_MIN_ROWS - 1)
+    down = (4096, 14336)
+    assert K.tiles_plan(64, *down) is None and K.tiles_plan(128, *down) is None          # the few-row products' rows
+    assert K.tiles_plan(129, *down) == (4, 2) and K.tiles_plan(256, *down) == (4, 2)
+    assert K.tiles_plan(300, *down) == (4, 0) and K.tiles_plan(1024, *down) == (2, 0)
+    assert K.tiles_plan(1025, *down) is None
+    assert K.tiles_plan(300, 4096, 4096) is None and K.tiles_plan(300, 6144, 4096) is None   # o, qkv: the library's
+    assert K.tiles_plan(300, 64, 320) == (2, 0)                                          # 5 stages of 64: not 4 parts
+    assert K.tiles_plan(300, 64, 200) is None                                            # k no multiple of 64
+    monkeypatch.setattr(K, "PROMPT_PRODUCT", "library")
+    assert K.tiles_plan(300, *down) is None and not K.tiles_serve_gated(4096)
+    monkeypatch.setattr(K, "PROMPT_PRODUCT", "tiles")
+    assert K.tiles_plan(300, 4096, 4096) == (1, 0) and K.tiles_serve_gated(65)
