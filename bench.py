@@ -11,7 +11,13 @@ against 8 TB/s, "points" = decoding at batch 1 and 64.  Beside the published pea
 holds what this GPU was measured to do at best in the same run ("measured_peak": a kernel that
 only reads the weights' bytes; v_mfma_f32_16x16x32_bf16 issued back to back) and the fractions
 of those; "generate_loop" is the same decode through the product's generation loop
-(Generator.generate: its batching, stop checks and bookkeeping inside the timed region).
+(Generator.generate: its batching, stop checks and bookkeeping inside the timed region);
+"spread" = the headline decode measured three times; "kernels" = where a decode step at the
+headline batch and the 2,048-token prompt spend their time, part by part, from events on the
+stream (microseconds a call, GB/s of the bytes a part has to read or TFLOP/s of its products);
+"sizes" = decoding at further sizes and contexts (the same model at 16,384 positions and at
+batch 64 with 4,096 positions; the Qwen3-14B layer sizes at batch 8 and 32), each with its
+fraction of the memory roofline.
 
     python bench.py --ceilings      # the measured ceilings alone, at several buffer sizes"""
 import argparse
@@ -83,6 +89,7 @@ def main(argv=None) -> int:
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS, help="tokens of the timed prompt")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration has (0 = all)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    ap.add_argument("--no-sizes", action="store_true", help="skip the further sizes and contexts")
     ap.add_argument("--only-prefill", action="store_true", help="time the 2,048-token prompt alone (for profiling)")
     ap.add_argument("--ceilings", action="store_true", help="measure the read bandwidth and the MFMA rate of this GPU and exit")
     ap.add_argument("--temperature", type=float, default=0.0, help="0 = greedy (the default run); above 0 the sampler draws")
@@ -116,14 +123,18 @@ def main(argv=None) -> int:
 
     model_name, cfg = MODELS[args.model]
     cfg = dict(cfg)
+    cfg0 = cfg
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
     max_batch = max(args.batch, 1 if (args.no_points or args.only_prefill) else 64)
     per_seq = args.prompt_len + args.steps + args.warmup + 64
+    sizes_on = not (args.no_points or args.only_prefill or args.no_sizes or args.temperature > 0)
+    long_runs = [(8, 16384), (64, 4096)] if sizes_on else []        # (batch, positions) of the same model
     t0 = time.time()
-    eng = llogos.Engine.from_config(cfg, seed=0, dtype="bfloat16",
-                                    max_tokens=max(max_batch * (per_seq + 64), prefill_tokens + 128), n_slots=max_batch)
+    eng = eng0 = llogos.Engine.from_config(cfg, seed=0, dtype="bfloat16",
+                                    max_tokens=max([max_batch * (per_seq + 64), prefill_tokens + 128] +
+                                                   [b * (n + 64) for b, n in long_runs]), n_slots=max_batch)
     print(f"[bench] model ready in {time.time() - t0:.1f} s; weights {weight_bytes(cfg) / 1e9:.2f} GB, "
           f"cache {eng.cache.bytes() / 1e9:.2f} GB", file=sys.stderr, flush=True)
     rng = np.random.default_rng(0)
@@ -142,11 +153,14 @@ def main(argv=None) -> int:
         n = logits.shape[0]
         return sampler.sample(logits, list(range(n)), [step] * n, None)
 
-    def decode_run(batch, steps, warmup):
-        """Prompts in one step, then greedy single-token steps: `warmup` untimed, `steps` timed."""
+    def decode_run(batch, steps, warmup, eng=None, cfg=None, prompt_len=None, prompts_per_step=None):
+        """Prompts in one step (or `prompts_per_step` at a time), then greedy single-token steps:
+        `warmup` untimed, `steps` timed."""
+        eng, cfg, prompt_len = eng or eng0, cfg or cfg0, prompt_len or args.prompt_len
         slots = [eng.alloc_slot() for _ in range(batch)]
-        prompts = [rng.integers(0, cfg["vocab_size"], size=args.prompt_len).tolist() for _ in range(batch)]
-        logits = eng.step(list(zip(slots, prompts)), want="last")
+        prompts = [rng.integers(0, cfg["vocab_size"], size=prompt_len).tolist() for _ in range(batch)]
+        per = prompts_per_step or batch
+        logits = torch.cat([eng.step(list(zip(slots[i:i + per], prompts[i:i + per])), want="last") for i in range(0, batch, per)])
         ids = pick(logits, 0)
         rows = list(range(batch))
         placeholders = [(s, [0]) for s in slots]
@@ -169,10 +183,78 @@ def main(argv=None) -> int:
         run(steps)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
-        ctx_mid = args.prompt_len + warmup + steps / 2.0
+        ctx_mid = prompt_len + warmup + steps / 2.0
         for s in slots:
             eng.free_slot(s)
         return dt, ctx_mid
+
+    def bytes_of_step(cfg, batch, ctx_mid):
+        """What a decode step has to read: every weight it uses once, and the cache of the live requests."""
+        return weight_bytes(cfg) + batch * ctx_mid * kv_bytes_per_token(cfg)
+
+    def part_costs(cfg, tokens, batch, context):
+        """Per part of a layer: bytes of its weights (and of the cache it reads), flops of `tokens` tokens."""
+        h, i, v = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+        q, kv = cfg["num_attention_heads"] * cfg["head_dim"], cfg["num_key_value_heads"] * cfg["head_dim"]
+        mats = {"qkv": h * (q + 2 * kv), "o": q * h, "gate_up": 2 * h * i, "down": h * i, "head": v * h}
+        costs = {k: (2.0 * n, 2.0 * n * (batch if k == "head" else tokens)) for k, n in mats.items()}
+        # attention: keys and values of the live context; products with keys and values over the causal half
+        pairs = batch * context if tokens == batch else tokens * (tokens + 1) / 2.0
+        costs["attention"] = (batch * context * 2.0 * kv * 2, 4.0 * q * pairs)
+        return costs
+
+    def prompt_rates(eng, cfg, entries, tokens):
+        """A prompt step launched kernel by kernel with a probe: per part microseconds a call and TFLOP/s."""
+        probe = llogos.StepProbe()
+        probe.hold()
+        probe.start()
+        eng.step(entries, want="last", probe=probe)
+        us = probe.microseconds_per_call()
+        out = {}
+        for name, (_, flops) in part_costs(cfg, tokens, 1, tokens).items():
+            if name in us:
+                out[name + "_us"] = round(us[name], 1)
+                out[name + "_TFLOPs"] = round(flops / us[name] / 1e6, 1)
+        for name in ("norm", "rotation"):
+            if name in us:
+                out[name + "_us"] = round(us[name], 1)
+        return out
+
+    def decode_rates(eng, cfg, slots, context, step_us):
+        """The parts of a single-token step of the sequences in `slots`: the products and the norm each run
+        for every layer in a row (the weights come from memory, nothing lies between the kernels, as in the
+        replayed step): microseconds a call and GB/s of the bytes the part has to read.  The attention
+        (rotation, cache write, attention, merge) is what is left of the replayed step (`step_us`, less the
+        head) per layer beside those; launched kernel by kernel its four short kernels would be measured
+        with the gaps between them, and a record between every two kernels costs them more than they take."""
+        batch = len(slots)
+        probe = llogos.StepProbe()
+        eng.step([(sl, [1]) for sl in slots], want="last", probe=probe)     # (gives the step's context to the probe)
+        layers = eng.model.layers
+        dev = eng.rt.device
+        h = torch.randn(batch, cfg["hidden_size"], device=dev).to(torch.bfloat16)
+        a = torch.randn(batch, cfg["num_attention_heads"] * cfg["head_dim"], device=dev).to(torch.bfloat16)
+        act = torch.randn(batch, cfg["intermediate_size"], device=dev).to(torch.bfloat16)
+
+        def gate_up(layer):
+            out = layer.ffn.gate_up.gated_product(h)
+            return out if out is not None else layer.ffn.gate_up.product(h)
+        us = {
+            "qkv": probe.repeat([lambda l=l: l.mixer.qkv.product(h, f32_ok=True) for l in layers]),
+            "o": probe.repeat([lambda l=l: l.mixer.o.product(a, f32_ok=True) for l in layers]),
+            "gate_up": probe.repeat([lambda l=l: gate_up(l) for l in layers]),
+            "down": probe.repeat([lambda l=l: l.ffn.down.product(act, f32_ok=True) for l in layers]),
+            "head": probe.repeat([lambda: eng.model.head.forward(h, out_dtype=torch.float32)] * 3),
+            "norm": probe.repeat([lambda l=l: l.mixer_norm.forward(torch.zeros(batch, cfg["hidden_size"], device=dev), None)
+                                  for l in layers]) ,
+        }
+        us["attention"] = (step_us - us["head"]) / len(layers) - us["qkv"] - us["o"] - us["gate_up"] - us["down"] - 2 * us["norm"]
+        out = {}
+        for name, (nbytes, _) in part_costs(cfg, batch, batch, context).items():
+            out[name + "_us"] = round(us[name], 1)
+            out[name + "_GBps"] = round(nbytes / us[name] / 1e3, 1)
+        out["norm_us"] = round(us["norm"], 1)
+        return out
 
     if args.only_prefill:
         prompt = rng.integers(0, cfg["vocab_size"], size=prefill_tokens).tolist()
@@ -215,6 +297,10 @@ def main(argv=None) -> int:
     print(f"[bench] decode b{args.batch}: {value:.1f} tok/s, {ms_per_step:.3f} ms/step, "
           f"{achieved / 1e12:.2f} TB/s", file=sys.stderr, flush=True)
 
+    if not args.no_points:
+        runs = [value] + [args.batch * args.steps / decode_run(args.batch, args.steps, args.warmup)[0] for _ in range(2)]
+        record["spread"] = {"runs": 3, "min": round(min(runs), 1), "max": round(max(runs), 1)}
+        print(f"[bench] decode b{args.batch}, three runs: {min(runs):.1f} to {max(runs):.1f} tok/s", file=sys.stderr, flush=True)
     if not args.no_points and sampler is None:
         # the same decode through the product's own loop: prompts in one step, then greedy tokens with
         # the loop's batching, stop checks, slot bookkeeping and token fetches inside the timed region
@@ -256,8 +342,47 @@ def main(argv=None) -> int:
                              "frac": round(flops / pt / MFMA_PEAK["bf16"], 4),
                              "measured_peak_tflops": round(mfma_peak / 1e12, 1),
                              "frac_of_measured": round(flops / pt / mfma_peak, 4)}
-        print(f"[bench] prefill {prefill_tokens}: {prefill_tokens / pt:.0f} tok/s, {pt * 1e3:.2f} ms", file=sys.stderr,
-              flush=True)
+        print(f"[bench] prefill {prefill_tokens}: {prefill_tokens / pt:.0f} tok/s, {pt * 1e3:.2f} ms (five runs: "
+              f"{min(times) * 1e3:.2f} to {max(times[1:]) * 1e3:.2f} after the first)", file=sys.stderr, flush=True)
+        record["prefill"]["ms_max"] = round(max(times[1:]) * 1e3, 3)
+        # where the time goes: a decode step of the headline batch and the prompt, part by part
+        slots = [eng.alloc_slot() for _ in range(args.batch)]
+        eng.step([(sl, rng.integers(0, cfg["vocab_size"], size=args.prompt_len).tolist()) for sl in slots], want="last")
+        kernels = {f"decode_b{args.batch}": decode_rates(eng, cfg, slots, args.prompt_len + 1, ms_per_step * 1e3)}
+        for sl in slots:
+            eng.free_slot(sl)
+        s = eng.alloc_slot()
+        kernels[f"prefill_{prefill_tokens}"] = prompt_rates(eng, cfg, [(s, prompt)], prefill_tokens)
+        eng.free_slot(s)
+        record["kernels"] = kernels
+        for k, v in kernels.items():
+            print(f"[bench] {k}: {v}", file=sys.stderr, flush=True)
+    if sizes_on:
+        sizes = {}
+
+        def size_point(label, eng, cfg, batch, prompt_len, steps, per_step):
+            d, mid = decode_run(batch, steps, 4, eng=eng, cfg=cfg, prompt_len=prompt_len, prompts_per_step=per_step)
+            frac = bytes_of_step(cfg, batch, mid) / (d / steps) / HBM_PEAK
+            sizes[label] = {"value": round(batch * steps / d, 1), "ms_per_step": round(d / steps * 1e3, 3), "frac": round(frac, 4)}
+            print(f"[bench] {label}: {sizes[label]['value']:.1f} tok/s, {d / steps * 1e3:.3f} ms/step, {frac:.3f} of "
+                  f"{HBM_PEAK / 1e12:g} TB/s", file=sys.stderr, flush=True)
+
+        short = model_name.lower().replace("-", "").replace(".", "")
+        for b, n in long_runs:                               # the context is n positions in the middle of the timed steps
+            size_point(f"{short}_b{b}_ctx{n}", eng, cfg, b, n - 4 - 16, 32, max(1, 32768 // n))
+        if args.model == "llama-3.1-8b" and not args.layers:
+            # another model's sizes: the engine above gives its memory back first
+            del eng, eng0, generator
+            import gc
+            gc.collect()
+            torch.cuda.empty_cache()
+            name2, cfg2 = MODELS["qwen3-14b"]
+            t0 = time.time()
+            eng2 = llogos.Engine.from_config(dict(cfg2), seed=0, dtype="bfloat16", max_tokens=32 * (1024 + 128 + 64), n_slots=32)
+            print(f"[bench] {name2} ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+            for b in (8, 32):
+                size_point(f"qwen314b_b{b}_p1024", eng2, cfg2, b, 1024, 64, 8)
+        record["sizes"] = sizes
     print(json.dumps(record), flush=True)
     return 0
 

@@ -11,14 +11,14 @@ from .config import (ARCHITECTURES, ConfigError, DenseDecoderConfig, RopeScaling
 from .weights import Checkpoint, WeightError, write_random_model
 from .models import LayerSpec, Model, ModelSpec, ScheduleEntry, dense_decoder_spec
 from .cache import Cache, CacheError, CacheFull
-from .engine import Engine, GenerationResult, Generator, StepError, plan_batches
+from .engine import Engine, GenerationResult, Generator, StepError, StepProbe, plan_batches
 from .sampling import GenerationParams, Sampler
 from .api import BenchmarkResult, Llogos, parse_attention
 
 __all__ = [
     "ARCHITECTURES", "ConfigError", "DenseDecoderConfig", "RopeScaling", "architecture_of", "read_config_json",
     "register_architecture", "Checkpoint", "WeightError", "write_random_model", "LayerSpec", "Model",
-    "ModelSpec", "ScheduleEntry", "dense_decoder_spec", "Cache", "CacheError", "CacheFull", "Engine", "StepError",
+    "ModelSpec", "ScheduleEntry", "dense_decoder_spec", "Cache", "CacheError", "CacheFull", "Engine", "StepError", "StepProbe",
     "GenerationResult", "Generator", "plan_batches", "GenerationParams", "Sampler", "BenchmarkResult", "Llogos",
     "parse_attention",
 ]

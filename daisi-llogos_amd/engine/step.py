@@ -188,7 +188,7 @@ class Engine:
     def step(self, entries: Sequence[Tuple[int, Sequence[int]]],
              want: Union[str, Sequence[Sequence[int]], None] = "last",
              device_ids: Optional[Tuple[torch.Tensor, Sequence[int]]] = None,
-             borrow: bool = False) -> Optional[torch.Tensor]:
+             borrow: bool = False, probe=None) -> Optional[torch.Tensor]:
         """entries: (slot, next tokens) for each sequence of the batch.  want: 'last', 'all',
         None, or for each entry the places among its tokens whose logits are asked for.
         Returns float32 logits [wanted places, vocab] in the order of the entries and of
@@ -201,7 +201,11 @@ class Engine:
 
         borrow: the caller is done with the logits (on the device, in stream order) before it
         asks for the next step, so a replayed step may hand out its own output buffer, which the
-        next replay overwrites, instead of a copy (33 MB a step at batch 64 and 128,256 tokens)."""
+        next replay overwrites, instead of a copy (33 MB a step at batch 64 and 128,256 tokens).
+
+        probe: a callable that the model's parts call with their name when their kernels are
+        queued (engine/probe.py: StepProbe times the step part by part); such a step is launched
+        kernel by kernel, not replayed."""
         if not entries:
             raise StepError("a step needs at least one sequence")
         slot_ids = [int(s) for s, _ in entries]
@@ -234,7 +238,7 @@ class Engine:
 
         self.cache.reserve(slot_ids, new_lens)
         try:
-            logits = self._run(ids, counts, cu, rows, slot_ids, starts, new_lens, device_ids, borrow)
+            logits = self._run(ids, counts, cu, rows, slot_ids, starts, new_lens, device_ids, borrow, probe)
         except BaseException:
             self.cache.unreserve(slot_ids)             # the sequences are as long as before, and hold no page more
             raise
@@ -242,10 +246,10 @@ class Engine:
         self.steps_run += 1
         return logits
 
-    def _run(self, ids, counts, cu, rows, slot_ids, starts, new_lens, device_ids, borrow=False) -> torch.Tensor:
+    def _run(self, ids, counts, cu, rows, slot_ids, starts, new_lens, device_ids, borrow=False, probe=None) -> torch.Tensor:
         T, B = int(cu[-1]), len(counts)
         # (more rows than the hand-written products take would put a library call into the graph)
-        if self.graphs is not None and T == B and B <= GRAPH_MAX_BATCH and rows == list(range(B)) \
+        if self.graphs is not None and probe is None and T == B and B <= GRAPH_MAX_BATCH and rows == list(range(B)) \
                 and self.cache.slots.n_slots == self._graph_slots():
             with torch.cuda.device(self.rt.device):
                 logits = self.graphs.step(ids.astype(np.int32), np.asarray(starts, dtype=np.int32),
@@ -267,9 +271,11 @@ class Engine:
                 K.gather_i32(dev[0], device_ids[0], dev[-1])
             ctx = StepContext(runtime=self.rt, n_tokens=T, batch=B, ids=dev[0], tok_seq=dev[1], tok_pos=dev[2],
                               slots=dev[3], cu_seqlens=[int(c) for c in cu], starts=starts, slot_ids=slot_ids,
-                              is_decode=max(counts) == 1, max_context=max(new_lens), cu_dev=dev[5])
+                              is_decode=max(counts) == 1, max_context=max(new_lens), cu_dev=dev[5], probe=probe)
             dev_tables = [d.view(t.shape) for d, t in zip(dev[6:6 + len(tables)], tables)]
             caches = self.cache.layer_caches(dev_tables)
+            if probe is not None and hasattr(probe, "context"):
+                probe.context(ctx, caches)               # (a probe that wants to run parts of this step again by itself)
             logits = self.model.forward(ctx, caches, dev[4] if len(rows) else None)
         return logits
 

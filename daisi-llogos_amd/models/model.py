@@ -206,13 +206,16 @@ class Model:
         None when nothing is wanted."""
         s = self.spec
         x = K.embed(self.embed_table, ctx.ids, s.embed_scale)
+        ctx.mark("embed")
         pending = None
         for entry, units in zip(self.schedule, self.entry_units):
             x, pending = self.layers[entry.layer].forward(ctx, x, pending, [caches[u] for u in units])
         if want_rows is None or want_rows.numel() == 0:
             return None
         n = self.final_norm.forward(x, pending, rows=want_rows, write_back=False)
+        ctx.mark("norm")
         logits = self.head.forward(n, out_dtype=torch.float32)
+        ctx.mark("head")
         if s.logit_scale != 1.0 or s.logit_softcap > 0.0:
             K.scale_softcap(logits, s.logit_scale, s.logit_softcap)
         return logits

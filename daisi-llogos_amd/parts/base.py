@@ -93,6 +93,12 @@ class StepContext:
     cu_dev: Optional[torch.Tensor] = None   # int32 [B + 1] token offsets on the device (None in a captured step)
     in_graph: bool = False              # the step is being captured for replay: host lists are not valid
     shared: Dict[object, object] = field(default_factory=dict)   # per-step tables shared by layers
+    probe: Optional[Callable[[str], None]] = None                 # called with a part's name when its kernels are queued
+
+    def mark(self, name: str) -> None:
+        """A part has queued its kernels (for a step that is timed part by part, engine/probe.py)."""
+        if self.probe is not None:
+            self.probe(name)
 
 
 class Part:

@@ -32,6 +32,11 @@ class PreNormBlock(Block):
                 caches) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
         cache = caches[0] if isinstance(caches, (list, tuple)) else caches
         h = self.mixer_norm.forward(x, pending)
+        ctx.mark("norm")
         a = self.mixer.forward(ctx, h, cache)
+        ctx.mark("mixer")
         h = self.ffn_norm.forward(x, a)
-        return x, self.ffn.forward(ctx, h)
+        ctx.mark("norm")
+        d = self.ffn.forward(ctx, h)
+        ctx.mark("feed_forward")
+        return x, d

@@ -32,10 +32,16 @@ class SwiGLU(FeedForward):
     def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
         act = self.gate_up.gated_product(h)
         if act is not None:
-            # up to 64 rows on packed weights: silu(gate) * up is the epilogue of the gate/up product
+            # on packed weights silu(gate) * up is the epilogue of the gate/up product
             # (the reference's MatMulSwiGLU, Daisi.Llogos/IComputeBackend.cs:448-456)
-            return self.down.product(act, f32_ok=True)
+            ctx.mark("gate_up")
+            out = self.down.product(act, f32_ok=True)
+            ctx.mark("down")
+            return out
         gu = self.gate_up.product(h)
+        ctx.mark("gate_up")
         # otherwise silu(gate) * up is made inside the down product where its kernel can (few rows), by a
         # kernel of its own for many; the residual sum that follows adds the product's parts
-        return self.down.product(gu, swiglu_input=True, f32_ok=True)
+        out = self.down.product(gu, swiglu_input=True, f32_ok=True)
+        ctx.mark("down")
+        return out
