@@ -346,53 +346,146 @@ __global__ void qk_rope_cache_kernel(const TI* __restrict__ qkv, int parts, size
     }
 }
 
-// The same for head_dim = rot = 128 with split-half pairing, without LDS or block barriers:
-// lane l of a wave holds dimensions 2 l and 2 l + 1 of its head, and the rotation partner
-// (64 dimensions away) sits in lane l ^ 32.
+// The same for head_dim = rot = 128 with split-half pairing, without LDS or block barriers, for
+// prompts.  With one (token, head) a wave and two values a lane this kernel took 29.5 us for 2,048
+// tokens of the 8B head shape (2.6 TB/s) and 20 us of that with every store left out: its time
+// was the number of its load instructions (five a token and head, of 4 and 8 bytes a lane), not
+// bytes or latency.  So a lane takes four consecutive dimensions (one 16-byte load), half a
+// wave a head (the rotation partner, 64 dimensions away, sits 16 lanes away), and a wave its two
+// heads for kRopeTokens tokens in a row, all of whose values it asks for before it works on the
+// first.  Values of eight consecutive positions are neighbours in a value page, so when the
+// wave's tokens are such a run its value stores are 16 bytes (otherwise one element each).
+constexpr int kRopeTokens = 8;
+constexpr int kRopeHeadsPerBlock = 8;                 // four waves of two heads
+
+template <typename TI> __device__ __forceinline__ float4 load4_f32(const TI* p);
+template <> __device__ __forceinline__ float4 load4_f32<float>(const float* p) { return *reinterpret_cast<const float4*>(p); }
+template <> __device__ __forceinline__ float4 load4_f32<bf16_t>(const bf16_t* p) {
+    const uint2 v = *reinterpret_cast<const uint2*>(p);
+    return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u),
+                       __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));
+}
+template <typename T> __device__ __forceinline__ void store4_f32(T* p, float a, float b, float c, float d);
+template <> __device__ __forceinline__ void store4_f32<float>(float* p, float a, float b, float c, float d) {
+    *reinterpret_cast<float4*>(p) = make_float4(a, b, c, d);
+}
+template <> __device__ __forceinline__ void store4_f32<bf16_t>(bf16_t* p, float a, float b, float c, float d) {
+    uint2 v;
+    v.x = (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+    v.y = (uint32_t)f32_to_bf16(c) | ((uint32_t)f32_to_bf16(d) << 16);
+    *reinterpret_cast<uint2*>(p) = v;
+}
+
 template <typename TI, typename T>
-__global__ void qk_rope_cache_hd128_kernel(const TI* __restrict__ qkv, int parts, size_t part_stride, int row_stride,
-                                           const float* __restrict__ bias, T* __restrict__ q_out,
-                                           int n_heads, int n_kv_heads,
-                                           const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w,
-                                           float eps, const float2* __restrict__ cs,
-                                           T* __restrict__ k_pool, T* __restrict__ v_pool, PagedKV cache,
-                                           const int* __restrict__ tok_seq, const int* __restrict__ tok_pos) {
+__global__ __launch_bounds__(kWave * kRopeHeadsPerBlock / 2) void qk_rope_cache_hd128_kernel(
+        const TI* __restrict__ qkv, int parts, size_t part_stride, int row_stride,
+        const float* __restrict__ bias, T* __restrict__ q_out, int n_heads, int n_kv_heads,
+        const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w,
+        float eps, const float2* __restrict__ cs, T* __restrict__ k_pool, T* __restrict__ v_pool, PagedKV cache,
+        const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, int n_tokens) {
     constexpr int HD = 128;
-    const int t = blockIdx.x;
-    const int head = blockIdx.y * kHeadsPerBlock + threadIdx.y;
-    const int lane = threadIdx.x;
-    if (head >= n_heads + 2 * n_kv_heads) return;
-    const int d = 2 * lane;
-    const size_t col = (size_t)head * HD + d;
-    const TI* src = qkv + (size_t)t * row_stride + col;
-    float x0 = sum_parts(src, 0, parts, part_stride), x1 = sum_parts(src, 1, parts, part_stride);
-    if (bias) { x0 += bias[col]; x1 += bias[col + 1]; }
-    const bool is_q = head < n_heads;
-    const bool is_k = !is_q && head < n_heads + n_kv_heads;
-    if (!is_q && !is_k) {
-        T* vdst = v_pool + paged_base(cache, tok_seq[t], head - n_heads - n_kv_heads, tok_pos[t]);
-        store_f32(vdst + page_value_offset(tok_pos[t] % kPageTokens, d), x0);
-        store_f32(vdst + page_value_offset(tok_pos[t] % kPageTokens, d + 1), x1);
+    const int t0 = blockIdx.x * kRopeTokens;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int l = lane & 31;
+    const int head = blockIdx.y * kRopeHeadsPerBlock + 2 * wave + (lane >> 5);
+    const int total_heads = n_heads + 2 * n_kv_heads;
+    const bool live = head < total_heads;              // (a wave's second head may lie past the last one)
+    const int hsafe = live ? head : total_heads - 1;
+    const int d = 4 * l;
+    const size_t col = (size_t)hsafe * HD + d;
+    const bool is_q = hsafe < n_heads;
+    const bool is_k = !is_q && hsafe < n_heads + n_kv_heads;
+    const bool is_v = !is_q && !is_k;
+    float4 x[kRopeTokens], ca[kRopeTokens], cb[kRopeTokens];
+    int seq[kRopeTokens], pos[kRopeTokens];
+#pragma unroll
+    for (int i = 0; i < kRopeTokens; ++i) {
+        const int t = min(t0 + i, n_tokens - 1);       // (tokens past the end: the last one again, not stored)
+        const TI* src = qkv + (size_t)t * row_stride + col;
+        x[i] = load4_f32<TI>(src);
+        for (int q = 1; q < parts; ++q) {
+            const float4 more = load4_f32<TI>(src + q * part_stride);
+            x[i].x += more.x; x[i].y += more.y; x[i].z += more.z; x[i].w += more.w;
+        }
+        // (cos, sin) of dimensions d & 63 .. + 3: two 16-byte loads
+        const float4* c4 = reinterpret_cast<const float4*>(cs + (size_t)t * 64 + (d & 63));
+        ca[i] = c4[0];
+        cb[i] = c4[1];
+        seq[i] = tok_seq[t];
+        pos[i] = tok_pos[t];
+    }
+    float4 b = make_float4(0.f, 0.f, 0.f, 0.f), w = make_float4(1.f, 1.f, 1.f, 1.f);
+    if (bias) b = *reinterpret_cast<const float4*>(bias + col);
+    const float* norm_w = is_q ? q_norm_w : (is_k ? k_norm_w : nullptr);
+    if (norm_w) w = *reinterpret_cast<const float4*>(norm_w + d);
+    // whether the wave's tokens are eight consecutive positions of one sequence that start at a multiple of eight
+    bool run = t0 + kRopeTokens <= n_tokens && (pos[0] & 7) == 0;
+#pragma unroll
+    for (int i = 1; i < kRopeTokens; ++i) run = run && seq[i] == seq[0] && pos[i] == pos[0] + i;
+#pragma unroll
+    for (int i = 0; i < kRopeTokens; ++i) {
+        x[i].x += b.x; x[i].y += b.y; x[i].z += b.z; x[i].w += b.w;
+    }
+    if (is_v) {
+        if (!live) return;
+        if (run) {
+            T* vdst = v_pool + paged_base(cache, seq[0], hsafe - n_heads - n_kv_heads, pos[0]);
+            const int at = pos[0] % kPageTokens;
+            // eight positions of one dimension lie side by side
+            T* p0 = vdst + page_value_offset(at, d);
+            store4_f32<T>(p0, x[0].x, x[1].x, x[2].x, x[3].x);       store4_f32<T>(p0 + 4, x[4].x, x[5].x, x[6].x, x[7].x);
+            T* p1 = vdst + page_value_offset(at, d + 1);
+            store4_f32<T>(p1, x[0].y, x[1].y, x[2].y, x[3].y);       store4_f32<T>(p1 + 4, x[4].y, x[5].y, x[6].y, x[7].y);
+            T* p2 = vdst + page_value_offset(at, d + 2);
+            store4_f32<T>(p2, x[0].z, x[1].z, x[2].z, x[3].z);       store4_f32<T>(p2 + 4, x[4].z, x[5].z, x[6].z, x[7].z);
+            T* p3 = vdst + page_value_offset(at, d + 3);
+            store4_f32<T>(p3, x[0].w, x[1].w, x[2].w, x[3].w);       store4_f32<T>(p3 + 4, x[4].w, x[5].w, x[6].w, x[7].w);
+            return;
+        }
+#pragma unroll
+        for (int i = 0; i < kRopeTokens; ++i) {
+            if (t0 + i >= n_tokens) break;
+            T* vdst = v_pool + paged_base(cache, seq[i], hsafe - n_heads - n_kv_heads, pos[i]);
+            const int at = pos[i] % kPageTokens;
+            store_f32(vdst + page_value_offset(at, d), x[i].x);
+            store_f32(vdst + page_value_offset(at, d + 1), x[i].y);
+            store_f32(vdst + page_value_offset(at, d + 2), x[i].z);
+            store_f32(vdst + page_value_offset(at, d + 3), x[i].w);
+        }
         return;
     }
-    const float* norm_w = is_q ? q_norm_w : k_norm_w;
-    if (norm_w) {
-        const float ss = wave_sum(x0 * x0 + x1 * x1);
-        const float inv = 1.0f / sqrtf(ss / (float)HD + eps);
-        x0 = x0 * inv * norm_w[d];
-        x1 = x1 * inv * norm_w[d + 1];
+    // (both heads of a wave take the same path from here on, or the other one is a value head and has left:
+    // the exchanges below stay within a head's 32 lanes)
+#pragma unroll
+    for (int i = 0; i < kRopeTokens; ++i) {
+        const int t = t0 + i;
+        if (t >= n_tokens) break;
+        float4 a = x[i];
+        if (norm_w) {
+            float ss = a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w;
+#pragma unroll
+            for (int o = 16; o > 0; o >>= 1) ss += __shfl_xor(ss, o, kWave);
+            const float inv = 1.0f / sqrtf(ss / (float)HD + eps);
+            a.x = a.x * inv * w.x; a.y = a.y * inv * w.y; a.z = a.z * inv * w.z; a.w = a.w * inv * w.w;
+        }
+        float4 p;
+        p.x = __shfl_xor(a.x, 16, kWave); p.y = __shfl_xor(a.y, 16, kWave);
+        p.z = __shfl_xor(a.z, 16, kWave); p.w = __shfl_xor(a.w, 16, kWave);
+        float4 y;
+        if (l < 16) {
+            y.x = a.x * ca[i].x - p.x * ca[i].y; y.y = a.y * ca[i].z - p.y * ca[i].w;
+            y.z = a.z * cb[i].x - p.z * cb[i].y; y.w = a.w * cb[i].z - p.w * cb[i].w;
+        } else {
+            y.x = p.x * ca[i].y + a.x * ca[i].x; y.y = p.y * ca[i].w + a.y * ca[i].z;
+            y.z = p.z * cb[i].y + a.z * cb[i].x; y.w = p.w * cb[i].w + a.w * cb[i].z;
+        }
+        if (!live) continue;
+        // (four consecutive dimensions are neighbours in a key page too)
+        T* dst = is_q ? q_out + ((size_t)t * n_heads + hsafe) * HD + d
+                      : k_pool + paged_base(cache, seq[i], hsafe - n_heads, pos[i])
+                               + page_key_offset(pos[i] % kPageTokens, d, HD);
+        store4_f32<T>(dst, y.x, y.y, y.z, y.w);
     }
-    const float p0 = __shfl_xor(x0, 32, kWave), p1 = __shfl_xor(x1, 32, kWave);
-    const float2 c0 = cs[(size_t)t * 64 + (d & 63)], c1 = cs[(size_t)t * 64 + (d & 63) + 1];
-    float y0, y1;
-    if (lane < 32) { y0 = x0 * c0.x - p0 * c0.y; y1 = x1 * c1.x - p1 * c1.y; }
-    else           { y0 = p0 * c0.y + x0 * c0.x; y1 = p1 * c1.y + x1 * c1.x; }
-    // (dimensions 2 l and 2 l + 1 are neighbours in a key page too)
-    T* dst = is_q ? q_out + ((size_t)t * n_heads + head) * HD + d
-                  : k_pool + paged_base(cache, tok_seq[t], head - n_heads, tok_pos[t])
-                           + page_key_offset(tok_pos[t] % kPageTokens, d, HD);
-    store_f32(dst, y0);
-    store_f32(dst + 1, y1);
 }
 
 // qkv: the fused projection [parts][T][row_stride] in float32 or in the cache's type (parts are
@@ -412,12 +505,18 @@ LLOGOS_EXPORT int llogos_qk_rope_cache(const void* qkv, int in_dtype, int parts,
     PagedKV cache{table, table_stride, n_kv_heads, head_dim};
     const int total_heads = n_heads + 2 * n_kv_heads;
     dim3 grid(T, (total_heads + kHeadsPerBlock - 1) / kHeadsPerBlock), block(kWave, kHeadsPerBlock);
+    dim3 grid128((T + kRopeTokens - 1) / kRopeTokens, (total_heads + kRopeHeadsPerBlock - 1) / kRopeHeadsPerBlock);
+    // (the wide form takes 16-byte steps through rows, tables and pools)
+    const bool wide = head_dim == 128 && rot == 128 && pairing == 0 && (row_stride % 4) == 0 && (part_stride % 4) == 0 &&
+                      ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)q_out % 16) == 0 && ((uintptr_t)cs % 16) == 0 &&
+                      ((uintptr_t)bias % 16) == 0 && ((uintptr_t)k_pool % 16) == 0 && ((uintptr_t)v_pool % 16) == 0 &&
+                      ((uintptr_t)q_norm_w % 16) == 0 && ((uintptr_t)k_norm_w % 16) == 0;
     const size_t smem = (size_t)kHeadsPerBlock * head_dim * sizeof(float);
 #define LAUNCH(TI, T_) do { \
-        if (head_dim == 128 && rot == 128 && pairing == 0) \
-            qk_rope_cache_hd128_kernel<TI, T_><<<grid, block, 0, stream>>>( \
+        if (wide) \
+            qk_rope_cache_hd128_kernel<TI, T_><<<grid128, kWave * kRopeHeadsPerBlock / 2, 0, stream>>>( \
                 (const TI*)qkv, parts, (size_t)part_stride, row_stride, bias, (T_*)q_out, n_heads, n_kv_heads, \
-                q_norm_w, k_norm_w, eps, (const float2*)cs, (T_*)k_pool, (T_*)v_pool, cache, tok_seq, tok_pos); \
+                q_norm_w, k_norm_w, eps, (const float2*)cs, (T_*)k_pool, (T_*)v_pool, cache, tok_seq, tok_pos, T); \
         else \
             qk_rope_cache_kernel<TI, T_><<<grid, block, smem, stream>>>( \
                 (const TI*)qkv, parts, (size_t)part_stride, row_stride, bias, (T_*)q_out, n_heads, n_kv_heads, head_dim, \

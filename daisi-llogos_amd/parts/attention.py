@@ -14,7 +14,7 @@ from typing import Callable, List, Optional
 import torch
 
 from ..ops import kernels as K
-from .base import KVSpec, LayerCache, Mixer, Runtime, StepContext, TensorSpec, register_mixer
+from .base import KVSpec, LayerCache, Mixer, Runtime, StepContext, TensorSpec, mark, register_mixer
 from .linear import Linear
 from .rope import Rotary
 
@@ -71,7 +71,7 @@ class Attention(Mixer):
         cs = self.position.prepare(ctx)
         if cache.writes:
             qkv = self.qkv.product(h, f32_ok=True)                      # [(parts,) T, (nh + 2 nkv) hd]
-            ctx.mark("qkv")
+            mark(ctx, "qkv")
             if ctx.is_decode and self.fuse_decode:
                 # one token a sequence: norm, rotation and cache write inside the attention kernel
                 a = K.attention_decode_fused(ctx, qkv, self.qkv.bias_rows(), nh, nkv, hd, self.position.rot,
@@ -79,7 +79,7 @@ class Attention(Mixer):
                                              cache.k_pool, cache.v_pool, cache.table, self.scale, self.window,
                                              self.sinks)
                 if a is not None:
-                    ctx.mark("attention")
+                    mark(ctx, "attention")
                     return self._project(ctx, a)
             q = K.qk_rope_cache(qkv, self.qkv.bias_rows(), self.rt.dtype, nh, nkv, hd, self.position.rot,
                                 self.position.pairing, self.q_norm_w, self.k_norm_w, self.eps, cs,
@@ -87,17 +87,17 @@ class Attention(Mixer):
         else:
             # the keys and values of these positions are another layer's: project q alone
             qkv = self.qkv.product(h, rows_out=nh * hd, f32_ok=True)
-            ctx.mark("qkv")
+            mark(ctx, "qkv")
             q = K.qk_rope_cache(qkv, self.qkv.bias_rows(nh * hd), self.rt.dtype, nh, 0, hd, self.position.rot,
                                 self.position.pairing, self.q_norm_w, None, self.eps, cs, None, None, None,
                                 ctx.tok_seq, ctx.tok_pos)
-        ctx.mark("rotation")
+        mark(ctx, "rotation")
         a = K.attention(ctx, q, q.stride(0), cache.k_pool, cache.v_pool, cache.table,
                         nh, nkv, hd, self.scale, self.window, self.sinks)
-        ctx.mark("attention")
+        mark(ctx, "attention")
         return self._project(ctx, a)
 
     def _project(self, ctx: StepContext, a: torch.Tensor) -> torch.Tensor:
         out = self.o.product(a, f32_ok=True)    # the residual sum that follows adds the parts
-        ctx.mark("o")
+        mark(ctx, "o")
         return out

@@ -101,6 +101,12 @@ class StepContext:
             self.probe(name)
 
 
+def mark(ctx: Optional[StepContext], name: str) -> None:
+    """ctx.mark(name) for a part that may be run without a step around it (ctx None)."""
+    if ctx is not None and ctx.probe is not None:
+        ctx.probe(name)
+
+
 class Part:
     """Base of mixers, feed-forwards, norms and position encodings."""
 

@@ -11,7 +11,7 @@ from typing import Callable, List, Optional, Tuple
 
 import torch
 
-from .base import Block, FeedForward, LayerCache, Mixer, Norm, Part, Runtime, StepContext, TensorSpec, register_block
+from .base import Block, FeedForward, LayerCache, Mixer, Norm, Part, Runtime, StepContext, TensorSpec, mark, register_block
 
 
 @register_block("pre_norm")
@@ -32,11 +32,11 @@ class PreNormBlock(Block):
                 caches) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
         cache = caches[0] if isinstance(caches, (list, tuple)) else caches
         h = self.mixer_norm.forward(x, pending)
-        ctx.mark("norm")
+        mark(ctx, "norm")
         a = self.mixer.forward(ctx, h, cache)
-        ctx.mark("mixer")
+        mark(ctx, "mixer")
         h = self.ffn_norm.forward(x, a)
-        ctx.mark("norm")
+        mark(ctx, "norm")
         d = self.ffn.forward(ctx, h)
-        ctx.mark("feed_forward")
+        mark(ctx, "feed_forward")
         return x, d

@@ -7,7 +7,7 @@ from typing import Callable, List, Optional
 
 import torch
 
-from .base import FeedForward, Runtime, StepContext, TensorSpec, register_feed_forward
+from .base import FeedForward, Runtime, StepContext, TensorSpec, mark, register_feed_forward
 from .linear import Linear
 
 
@@ -34,14 +34,14 @@ class SwiGLU(FeedForward):
         if act is not None:
             # on packed weights silu(gate) * up is the epilogue of the gate/up product
             # (the reference's MatMulSwiGLU, Daisi.Llogos/IComputeBackend.cs:448-456)
-            ctx.mark("gate_up")
+            mark(ctx, "gate_up")
             out = self.down.product(act, f32_ok=True)
-            ctx.mark("down")
+            mark(ctx, "down")
             return out
         gu = self.gate_up.product(h)
-        ctx.mark("gate_up")
+        mark(ctx, "gate_up")
         # otherwise silu(gate) * up is made inside the down product where its kernel can (few rows), by a
         # kernel of its own for many; the residual sum that follows adds the product's parts
         out = self.down.product(gu, swiglu_input=True, f32_ok=True)
-        ctx.mark("down")
+        mark(ctx, "down")
         return out

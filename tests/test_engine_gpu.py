@@ -659,6 +659,37 @@ def test_a_model_made_on_the_device_is_the_model_written_to_a_folder(dtype):
     H.close(outs[1], H.plain_logits(name, toks), dtype, "model made on the device", config=name)
 
 
+@pytest.mark.parametrize("dtype", H.DTYPES)
+def test_a_step_timed_part_by_part_is_the_same_step(dtype):
+    """A step run with a probe is launched kernel by kernel and marked by its parts; its logits are those of
+    the replayed step, and every layer's parts appear once in the account."""
+    name = "tiny_d"
+    engines = [H.engine(name, dtype, n_slots=2) for _ in range(2)]
+    toks = [H.tokens(name, 40, 5), H.tokens(name, 9, 6)]
+    slots = [[e.alloc_slot() for _ in toks] for e in engines]
+    probe = H.llogos.StepProbe()
+    probe.start()
+    outs = [engines[0].step([(s, t[:-2]) for s, t in zip(slots[0], toks)], want="last", probe=probe),
+            engines[1].step([(s, t[:-2]) for s, t in zip(slots[1], toks)], want="last")]
+    assert torch.equal(outs[0], outs[1])
+    layers = tc.ALL[name]["num_hidden_layers"]
+    totals = probe.totals()
+    assert {k: n for k, (n, _) in totals.items()} == {
+        "embed": 1, "norm": 2 * layers + 1, "qkv": layers, "rotation": layers, "attention": layers, "o": layers,
+        "mixer": layers, "gate_up": layers, "down": layers, "feed_forward": layers, "head": 1}
+    assert all(ms >= 0 for _, ms in totals.values())
+    for t in range(2):                                                  # single tokens: replayed against launched with a probe
+        probe = H.llogos.StepProbe()
+        probe.hold(1.0)
+        probe.start()
+        a = engines[0].step([(s, [tk[-2 + t]]) for s, tk in zip(slots[0], toks)], want="last", probe=probe)
+        b = engines[1].step([(s, [tk[-2 + t]]) for s, tk in zip(slots[1], toks)], want="last")
+        assert torch.equal(a, b)
+        assert probe.totals()["attention"][0] == layers
+        assert ("rotation" in probe.totals()) == (dtype == "float32")   # bfloat16: one kernel from the projection to the output
+    assert probe.repeat([lambda: engines[0].model.layers[0].mixer_norm.forward(torch.zeros(2, 120, device="cuda"), None)] * 3) > 0
+
+
 def test_benchmark_reports_bytes_and_flops_of_its_steps():
     """Llogos.benchmark's roofline inputs for tiny_a, worked by hand: two layers of
     qkv (128 x 64 + bias 128), o (64 x 64), gate/up (352 x 64), down (64 x 176), two norms (64 each), the
