@@ -236,18 +236,35 @@ def main(argv=None) -> int:
         a = torch.randn(batch, cfg["num_attention_heads"] * cfg["head_dim"], device=dev).to(torch.bfloat16)
         act = torch.randn(batch, cfg["intermediate_size"], device=dev).to(torch.bfloat16)
 
-        def gate_up(layer):
-            out = layer.ffn.gate_up.gated_product(h)
-            return out if out is not None else layer.ffn.gate_up.product(h)
-        us = {
-            "qkv": probe.repeat([lambda l=l: l.mixer.qkv.product(h, f32_ok=True) for l in layers]),
-            "o": probe.repeat([lambda l=l: l.mixer.o.product(a, f32_ok=True) for l in layers]),
-            "gate_up": probe.repeat([lambda l=l: gate_up(l) for l in layers]),
-            "down": probe.repeat([lambda l=l: l.ffn.down.product(act, f32_ok=True) for l in layers]),
-            "head": probe.repeat([lambda: eng.model.head.forward(h, out_dtype=torch.float32)] * 3),
-            "norm": probe.repeat([lambda l=l: l.mixer_norm.forward(torch.zeros(batch, cfg["hidden_size"], device=dev), None)
-                                  for l in layers]) ,
-        }
+        def gate_up(layer, rows):
+            out = layer.ffn.gate_up.gated_product(rows)
+            return out if out is not None else layer.ffn.gate_up.product(rows)
+        P = llogos.parts
+        x = torch.randn(batch, cfg["hidden_size"], device=dev)
+        # steps of few rows: o and down add themselves to the stream and leave the next norm's rows, which
+        # gate/up and qkv take as they are (no norm kernel between); otherwise products in parts and the norm
+        left = [l.mixer.o.add_to(a, P.Residual(x, l.ffn_norm)) for l in layers]
+        if all(v is not None for v in left):
+            rows_ffn = [l.ffn_norm.forward(x, v, lazy=True) for l, v in zip(layers, left)]
+            left = [l.ffn.down.add_to(act, P.Residual(x, l.mixer_norm)) for l in layers]
+            rows_mixer = [l.mixer_norm.forward(x, v, lazy=True) for l, v in zip(layers, left)]
+            us = {
+                "qkv": probe.repeat([lambda l=l, r=r: l.mixer.qkv.product(r, f32_ok=True) for l, r in zip(layers, rows_mixer)]),
+                "o": probe.repeat([lambda l=l: l.mixer.o.add_to(a, P.Residual(x, l.ffn_norm)) for l in layers]),
+                "gate_up": probe.repeat([lambda l=l, r=r: gate_up(l, r) for l, r in zip(layers, rows_ffn)]),
+                "down": probe.repeat([lambda l=l: l.ffn.down.add_to(act, P.Residual(x, l.mixer_norm)) for l in layers]),
+                "norm": 0.0,
+            }
+        else:
+            us = {
+                "qkv": probe.repeat([lambda l=l: l.mixer.qkv.product(h, f32_ok=True) for l in layers]),
+                "o": probe.repeat([lambda l=l: l.mixer.o.product(a, f32_ok=True) for l in layers]),
+                "gate_up": probe.repeat([lambda l=l: gate_up(l, h) for l in layers]),
+                "down": probe.repeat([lambda l=l: l.ffn.down.product(act, f32_ok=True) for l in layers]),
+                "norm": probe.repeat([lambda l=l: l.mixer_norm.forward(torch.zeros(batch, cfg["hidden_size"], device=dev), None)
+                                      for l in layers]),
+            }
+        us["head"] = probe.repeat([lambda: eng.model.head.forward(h, out_dtype=torch.float32)] * 3)
         us["attention"] = (step_us - us["head"]) / len(layers) - us["qkv"] - us["o"] - us["gate_up"] - us["down"] - 2 * us["norm"]
         out = {}
         for name, (nbytes, _) in part_costs(cfg, batch, batch, context).items():

@@ -1,0 +1,139 @@
+// x[M, N] += a[M, K] . w[N, K]^T (+ bias) for up to 16 rows, on packed weights, in one pass:
+// the product that closes a mixer or a feed-forward adds itself to the residual stream and
+// leaves, beside the stream, what the norm that follows needs of it.
+//
+// A block owns 16 rows of w (16 columns of x) and the whole of k: its waves take equal runs of
+// k, each with one MFMA accumulator; LDS adds the waves' sums in ascending order of k, the
+// block adds them to its 16 columns of x (float32, in place) and writes for every row of x the
+// sum of the squares of its 16 new values: sums[strip][16], and x * norm_w in bfloat16, the rows
+// of the rmsnorm that follows without their scale.  The product that takes norm(x) as its
+// activations (gemm_skinny_lds_bf16.hip, PRODUCE_UNSCALED) multiplies these rows, adds the strips'
+// sums in ascending order and applies 1 / rms to its result: no other pass over x and no kernel
+// between the two products.  Nothing here depends on what else runs: the order of every addition is
+// fixed by N, K and the number of waves.
+//
+// (With k divided over blocks instead, as the few-row product with partial sums does, a row of x
+// is complete only after a kernel boundary, and the norm has to be a kernel of its own: at 8
+// rows two such kernels were 9.6 of a layer's 102 us.)
+//
+// Weights: llogos_pack_weights' layout, [N / 64][K / 32][4 strips][64 lanes] fragments of 16
+// bytes; strip s of a 64-row group is every fourth KB of the group's run.  Activations: each
+// wave loads its own MFMA operand from a (rows beyond M: zero); with at most 16 rows that is
+// at most as many bytes as the weights and they come from the L2.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kResidualRows = 16;      // rows of a (tokens) at most
+constexpr int kAhead = 4;              // MFMA steps whose operands a wave asks for together
+
+constexpr int kActRow = kAhead * 32 + 8;   // bf16 of a wave's LDS row: 4 steps and 16 bytes of padding (rows 4 banks apart)
+
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void gemm_residual_kernel(
+        float* __restrict__ x, int ldx, float* __restrict__ sums, bf16_t* __restrict__ unscaled, int ldu,
+        const float* __restrict__ norm_w, const bf16_t* __restrict__ a, int lda,
+        const u32x4* __restrict__ wp, const float* __restrict__ bias, int M, int N, int K) {
+    __shared__ float red[WAVES][4][kWave];
+    __shared__ __attribute__((aligned(16))) bf16_t acts[WAVES][kResidualRows][kActRow];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int r = lane & 15, g = lane >> 4;
+    const int strip = blockIdx.x;
+    const int steps = (K + 31) / 32;
+    const int s_begin = (int)((long long)steps * wave / WAVES), s_end = (int)((long long)steps * (wave + 1) / WAVES);
+    const u32x4* wsrc = wp + ((size_t)(strip >> 2) * steps * 4 + (strip & 3)) * kWave + lane;
+    // Activations: a wave copies the 4 steps' 128 values of k of four rows with one load (16 lanes a row,
+    // whole cache lines), through registers into its own rows of LDS, and reads its MFMA operands from
+    // there.  (Loading the operands themselves, 16 rows x 64 bytes a step, asked for twice the lines: the
+    // 8B down projection took 23.0 us at 8 rows, 20.6 without its activations; with this copy ...)
+    const int quads = (M + 3) / 4;                       // loads of four rows
+    const bf16_t* asrc = a + (size_t)g * lda + r * 8;
+    const int k_end = min(K, s_end * 32);
+
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    u32x4 wf[2][kAhead];
+    uint4 af[2][kResidualRows / 4];
+    auto fetch = [&](int buf, int s0) {
+#pragma unroll
+        for (int j = 0; j < kAhead; ++j) {
+            u32x4 v = {0, 0, 0, 0};
+            if (s0 + j < s_end) v = __builtin_nontemporal_load(wsrc + (size_t)(s0 + j) * (4 * kWave));
+            wf[buf][j] = v;
+        }
+#pragma unroll
+        for (int q = 0; q < kResidualRows / 4; ++q) {
+            uint4 t = make_uint4(0, 0, 0, 0);
+            if (q < quads && 4 * q + g < M && s0 * 32 + r * 8 < k_end)
+                t = *reinterpret_cast<const uint4*>(asrc + (size_t)(4 * q) * lda + s0 * 32);
+            af[buf][q] = t;
+        }
+    };
+    auto multiply = [&](int buf) {
+#pragma unroll
+        for (int q = 0; q < kResidualRows / 4; ++q)
+            *reinterpret_cast<uint4*>(&acts[wave][4 * q + g][r * 8]) = af[buf][q];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int j = 0; j < kAhead; ++j) {
+            const uint4 t = *reinterpret_cast<const uint4*>(&acts[wave][r][j * 32 + g * 8]);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wf[buf][j]),
+                                                          __builtin_bit_cast(bf16x8, t), acc, 0, 0, 0);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+    if (s_begin < s_end) fetch(0, s_begin);
+    for (int s = s_begin; s < s_end; s += 2 * kAhead) {
+        if (s + kAhead < s_end) fetch(1, s + kAhead);
+        multiply(0);
+        if (s + 2 * kAhead < s_end) fetch(0, s + 2 * kAhead);
+        if (s + kAhead < s_end) multiply(1);
+    }
+
+    // acc[i]: column 16 strip + 4 g + i of x, row r
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][i][lane] = acc[i];
+    __syncthreads();
+    if (threadIdx.x >= 256) return;
+    const int m = threadIdx.x >> 4, c = threadIdx.x & 15;
+    const int src_lane = (c >> 2) * 16 + m, i = c & 3;
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) v += red[w][i][src_lane];
+    const int n = strip * 16 + c;
+    float sq = 0.f;
+    if (m < M && n < N) {
+        float* xp = x + (size_t)m * ldx + n;
+        const float y = *xp + (v + (bias ? bias[n] : 0.f));
+        *xp = y;
+        sq = y * y;
+        if (unscaled) unscaled[(size_t)m * ldu + n] = f32_to_bf16(y * norm_w[n]);
+    }
+    // the 16 lanes of a row are neighbours: a fixed tree of additions
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) sq += __shfl_xor(sq, o, kWave);
+    if (c == 0) sums[(size_t)strip * kResidualRows + m] = sq;
+}
+
+// sums: float32 [ceil(N / 16)][16], written whole (rows from M on hold 0).  unscaled (optional, with norm_w
+// [N]): bfloat16 [M][ldu] = x * norm_w of the new x, the rows of an rmsnorm that still lack their scale.
+LLOGOS_EXPORT int llogos_gemm_residual_bf16(float* x, int ldx, float* sums, void* unscaled, int ldu, const float* norm_w,
+                                            const void* act, int lda, const void* packed_w, const float* bias,
+                                            int M, int N, int K, int waves, hipStream_t stream) {
+    if (M <= 0 || N <= 0 || K <= 0 || ldx < N || lda < K || x == nullptr || sums == nullptr) return LLOGOS_BAD_ARGUMENT;
+    if (unscaled != nullptr && (norm_w == nullptr || ldu < N)) return LLOGOS_BAD_ARGUMENT;
+    if (M > kResidualRows || (K % 8) || (lda % 8) || ((uintptr_t)act % 16) || ((uintptr_t)packed_w % 16))
+        return LLOGOS_UNSUPPORTED;
+    const int strips = (N + 15) / 16;
+    const u32x4* W = (const u32x4*)packed_w;
+    const bf16_t* A = (const bf16_t*)act;
+    if (waves == 4) gemm_residual_kernel<4><<<strips, 4 * kWave, 0, stream>>>(x, ldx, sums, (bf16_t*)unscaled, ldu, norm_w, A, lda, W, bias, M, N, K);
+    else if (waves == 8) gemm_residual_kernel<8><<<strips, 8 * kWave, 0, stream>>>(x, ldx, sums, (bf16_t*)unscaled, ldu, norm_w, A, lda, W, bias, M, N, K);
+    else if (waves == 16) gemm_residual_kernel<16><<<strips, 16 * kWave, 0, stream>>>(x, ldx, sums, (bf16_t*)unscaled, ldu, norm_w, A, lda, W, bias, M, N, K);
+    else return LLOGOS_BAD_ARGUMENT;
+    return LLOGOS_LAUNCH_CHECK();
+}

@@ -36,19 +36,27 @@ constexpr int kChunkSteps = kChunkK / 32;    // MFMA steps per chunk
 constexpr int kLdsMaxRows = 128;            // rows of activations (64 with a fused producer)
 constexpr int kRowPad = 16;                  // bf16 of padding per LDS row (32 bytes)
 
-enum { PRODUCE_PLAIN = 0, PRODUCE_SWIGLU_F32 = 1, PRODUCE_SWIGLU_BF16 = 2 };
+enum { PRODUCE_PLAIN = 0, PRODUCE_SWIGLU_F32 = 1, PRODUCE_SWIGLU_BF16 = 2, PRODUCE_UNSCALED = 3 };
+constexpr int kNormRows = 16;        // rows at most when the activations are rows of a norm without their scale
 
 struct ActSource {
-    const void* ptr;        // plain: bf16 [M][lda]; swiglu: [parts][M][2 K] float32 or bf16
-    int lda;                // plain: row stride in elements; swiglu: 2 K
+    const void* ptr;        // plain, unscaled: bf16 [M][lda]; swiglu: [parts][M][2 K] float32 or bf16
+    int lda;                // plain, unscaled: row stride in elements; swiglu: 2 K
     int parts;              // swiglu: partial products to add
     size_t part_stride;     // elements between parts
+    // unscaled: the activations are x * w of an rmsnorm over rows x of `width` values whose sums of squares
+    // lie in sums [n_sums][kNormRows] by parts (llogos_gemm_residual_bf16); the product of row m is
+    // multiplied by 1 / sqrt(sum_m / width + eps) in the epilogue
+    const float* sums;
+    int n_sums;
+    int width;
+    float eps;
 };
 
 // eight consecutive activations (k .. k + 7 of row m) as bf16
 template <int MODE>
 __device__ __forceinline__ uint4 produce8(const ActSource& src, int m, int k, int K) {
-    if (MODE == PRODUCE_PLAIN) {
+    if (MODE == PRODUCE_PLAIN || MODE == PRODUCE_UNSCALED) {
         return *reinterpret_cast<const uint4*>((const bf16_t*)src.ptr + (size_t)m * src.lda + k);
     } else {
         float g[8], u[8];
@@ -102,6 +110,7 @@ __global__ __launch_bounds__(WAVES * kWave) void gemm_skinny_lds_kernel(
     constexpr int kPieces = kRows * (CHUNK / 8);                    // 16-byte pieces of a chunk
     constexpr int kPiecesPerThread = (kPieces + WAVES * kWave - 1) / (WAVES * kWave);
     __shared__ __attribute__((aligned(16))) bf16_t lds[2][kRows][kRowLen];
+    __shared__ float inv_rms[kNormRows], squares_by_part[16 * kNormRows];
 
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int r = lane & 15, g = lane >> 4;
@@ -183,10 +192,31 @@ __global__ __launch_bounds__(WAVES * kWave) void gemm_skinny_lds_kernel(
         }
     };
 
+    // PRODUCE_UNSCALED: thread (j, m) adds parts j, j + 16, ... of row m's sum of squares; its loads go out
+    // first, so that they have arrived with the first activations and cost no wait of their own; thread m adds
+    // the 16 sums in ascending j at the end: the same additions in every block
+    float row_squares = 0.f, early[16];
+    if (MODE == PRODUCE_UNSCALED && threadIdx.x < 16 * kNormRows) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int p = threadIdx.x / kNormRows + 16 * i;
+            early[i] = p < src.n_sums ? src.sums[(size_t)p * kNormRows + (threadIdx.x & (kNormRows - 1))] : 0.f;
+        }
+    }
+    auto add_row_squares = [&]() {
+        if (MODE == PRODUCE_UNSCALED && threadIdx.x < 16 * kNormRows) {
+            const int m = threadIdx.x & (kNormRows - 1), j = threadIdx.x / kNormRows;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) row_squares += early[i];
+            for (int p = j + 256; p < src.n_sums; p += 16) row_squares += src.sums[(size_t)p * kNormRows + m];
+            squares_by_part[threadIdx.x] = row_squares;
+        }
+    };
     if (n_chunks > 0) {
         fetch_acts(k_begin);
         fetch_w(wf0, k_begin);
         store_acts(0);
+        add_row_squares();
         __syncthreads();
     }
     for (int c = 0; c < n_chunks; c += 2) {
@@ -202,6 +232,16 @@ __global__ __launch_bounds__(WAVES * kWave) void gemm_skinny_lds_kernel(
         __syncthreads();
     }
 
+    if (MODE == PRODUCE_UNSCALED) {
+        if (n_chunks <= 0) { add_row_squares(); __syncthreads(); }
+        if (threadIdx.x < kNormRows) {
+            float t = 0.f;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) t += squares_by_part[j * kNormRows + threadIdx.x];
+            inv_rms[threadIdx.x] = 1.0f / sqrtf(t / (float)src.width + src.eps);
+        }
+        __syncthreads();
+    }
     if (GATED) {
         // The packed strips alternate between 16 gate rows and the 16 up rows of the same columns
         // (llogos_pack_weights with gate_rows): waves 0 and 2 hold gate values, waves 1 and 3 the up
@@ -225,7 +265,8 @@ __global__ __launch_bounds__(WAVES * kWave) void gemm_skinny_lds_kernel(
             if (m >= M) continue;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float gate = acc[0][mb][i], up = xch[(((wave >> 1) * MB + mb) * 4 + i) * kWave + lane];
+                const float row_scale = MODE == PRODUCE_UNSCALED ? inv_rms[m] : 1.0f;
+                const float gate = acc[0][mb][i] * row_scale, up = xch[(((wave >> 1) * MB + mb) * 4 + i) * kWave + lane] * row_scale;
                 const float y = gate * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * gate)) * up;
                 if (col0 + i < N / 2) store_f32(out + (size_t)m * ldo + col0 + i, y);
             }
@@ -240,10 +281,11 @@ __global__ __launch_bounds__(WAVES * kWave) void gemm_skinny_lds_kernel(
         for (int mb = 0; mb < MB; ++mb) {
             const int m = mb * 16 + r;
             if (m >= M) continue;
+            const float row_scale = MODE == PRODUCE_UNSCALED ? inv_rms[m] : 1.0f;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int n = n0 + rb * 16 + 4 * g + i;
-                if (n < N) store_f32(dst + (size_t)m * ldo + n, acc[rb][mb][i] + (bias ? bias[n] : 0.f));
+                if (n < N) store_f32(dst + (size_t)m * ldo + n, acc[rb][mb][i] * row_scale + (bias ? bias[n] : 0.f));
             }
         }
 }
@@ -417,5 +459,38 @@ LLOGOS_EXPORT int llogos_gemm_packed_gated_bf16(void* out, int out_dtype, const 
     if (chunk == 128) BY_ROWS(128);
     BY_ROWS(256);
 #undef BY_ROWS
+#undef GO
+}
+
+// The same two products on the rows of an rmsnorm that still lack their scale: act [M][lda] = x * norm_w in
+// bfloat16, for up to 16 rows, and sums [n_sums][16] the partial sums of squares of the rows of x over
+// `width` values, both left by the product that completed x (llogos_gemm_residual_bf16).  The scale
+// 1 / sqrt(sum / width + eps) is a factor of the whole row, so it is applied to the product in the
+// epilogue, in float32: no kernel between the product that completes x and this one.  gated = 0: out
+// [parts][M][ldo] as llogos_gemm_packed_bf16 (a bias is added after the scale); gated = 1: out [M][ldo] =
+// silu(gate) * up as llogos_gemm_packed_gated_bf16.
+LLOGOS_EXPORT int llogos_gemm_packed_unscaled_bf16(void* out, int out_dtype, const void* act, int lda, const float* sums,
+                                                   int n_sums, int width, float eps, const void* packed_w,
+                                                   const float* bias, int M, int N, int K, int ldo,
+                                                   long long part_stride, int splits, int chunk, int gated,
+                                                   hipStream_t stream) {
+    if (M <= 0 || N <= 0 || K <= 0 || splits < 1 || n_sums < 1 || width < 1 || act == nullptr || sums == nullptr)
+        return LLOGOS_BAD_ARGUMENT;
+    if (out_dtype != DT_BF16 && out_dtype != DT_F32) return LLOGOS_BAD_ARGUMENT;
+    if (chunk != 128 && chunk != 256) return LLOGOS_BAD_ARGUMENT;
+    if (gated ? ((N % 32) || ldo < N / 2 || bias != nullptr) : ldo < N) return LLOGOS_BAD_ARGUMENT;
+    if (M > kNormRows || (K % 8) || (lda % 8) || lda < K || ((uintptr_t)act % 16) || ((uintptr_t)packed_w % 16))
+        return LLOGOS_UNSUPPORTED;
+    const int parts = gated ? 1 : llogos_gemm_packed_parts(K, splits, chunk);
+    if (parts > 1 && (out_dtype != DT_F32 || bias != nullptr || part_stride < (long long)M * ldo))
+        return LLOGOS_BAD_ARGUMENT;
+    const int kpb = packed_k_per_block(K, parts, chunk);
+    ActSource src{act, lda, 1, 0, sums, n_sums, width, eps};
+    const bf16_t* W = (const bf16_t*)packed_w;
+#define GO(CH, GATED) return launch_lds<1, 1, PRODUCE_UNSCALED, CH, kLdsWaves, true, GATED>(out, out_dtype, src, W, bias, M, N, K, ldo, \
+                                                                                            (size_t)part_stride, kpb, parts, stream)
+    if (gated) { if (chunk == 128) GO(128, true); GO(256, true); }
+    if (chunk == 128) GO(128, false);
+    GO(256, false);
 #undef GO
 }

@@ -208,8 +208,15 @@ class Model:
         x = K.embed(self.embed_table, ctx.ids, s.embed_scale)
         ctx.mark("embed")
         pending = None
-        for entry, units in zip(self.schedule, self.entry_units):
-            x, pending = self.layers[entry.layer].forward(ctx, x, pending, [caches[u] for u in units])
+        blocks = [self.layers[entry.layer] for entry in self.schedule]
+        for i, (block, units) in enumerate(zip(blocks, self.entry_units)):
+            if block.takes_next_norm:
+                # the norm that reads the stream after this block: the next block's first one (the final
+                # norm reads only the wanted rows and prepares its own)
+                next_norm = blocks[i + 1].entry_norm() if i + 1 < len(blocks) else None
+                x, pending = block.forward(ctx, x, pending, [caches[u] for u in units], next_norm=next_norm)
+            else:
+                x, pending = block.forward(ctx, x, pending, [caches[u] for u in units])
         if want_rows is None or want_rows.numel() == 0:
             return None
         n = self.final_norm.forward(x, pending, rows=want_rows, write_back=False)

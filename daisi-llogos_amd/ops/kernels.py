@@ -7,6 +7,7 @@ tensors used as device memory; launches go to torch's current stream.
 from __future__ import annotations
 
 import ctypes
+from dataclasses import dataclass
 import os
 from typing import Optional, Sequence, Tuple
 
@@ -663,6 +664,122 @@ def gemm_packed_bf16(a: torch.Tensor, pw: PackedWeight, bias: Optional[torch.Ten
     if code == -2:
         return None
     _check(code, "gemm_packed_bf16")
+    return out
+
+
+RESIDUAL_MAX_ROWS = 16     # rows at most of the product that adds itself to the residual stream
+# "on" (the default): steps of up to 16 rows close a mixer and a feed-forward with gemm_residual_bf16 and
+# open the next with gemm_packed_unscaled_bf16 where the shapes allow; "off": the products in parts and
+# the norm's own kernel everywhere.  LLOGOS_RESIDUAL_PRODUCT in the environment sets the default.
+RESIDUAL_PRODUCT = os.environ.get("LLOGOS_RESIDUAL_PRODUCT", "on")
+
+
+@dataclass
+class RowSquares:
+    """What a product that has added itself to the residual stream x leaves beside it: sums [strips, 16],
+    float32, strip s holding for each row of x the sum of the squares of columns 16 s .. 16 s + 15.  A
+    norm over the rows of x needs no other pass over them (gemm_packed_normed_bf16)."""
+    sums: torch.Tensor
+    width: int                                  # columns of x that the sums cover
+    unscaled: Optional[torch.Tensor] = None     # bfloat16 [M, width]: x * norm_w, the rmsnorm's rows without their scale
+    norm_w: Optional[torch.Tensor] = None       # the weight that `unscaled` was made with
+
+
+def residual_plan(M: int, N: int, K: int, n_cus: Optional[int] = None) -> int:
+    """Waves of a block of gemm_residual_bf16 (0: not served; then the product in parts over k and the norm's
+    own kernel do the work).  A block owns 16 rows of w and all of k, so there are N / 16 blocks, and a
+    compute unit streams what its blocks own at a bounded rate: the blocks have to fill the units evenly.
+    Measured on the MI355X (256 units) at 1, 8 and 16 rows against the product in parts plus the norm kernel:
+      N / 16 <= units (1B, 3B, 8B widths): always ahead, 8 waves a block (8B at 8 rows: o 8.9 us against 12.4,
+        down 20.9 against 24.2);
+      N / 16 a multiple of the units (70B: 512): ahead with 4 waves (o 22.5 against 27.3, down 75.6 against
+        78.8), but behind at 16 rows with k beyond 16K (83 against 79), where a block's copy of the
+        activations is as many bytes as its weights;
+      N / 16 = 1.25 units (14B: 320): a quarter of the units get two blocks; ahead only for the small
+        matrix (o 14.0 against 16.1; down 38 against 33)."""
+    if RESIDUAL_PRODUCT != "on" or not (0 < M <= RESIDUAL_MAX_ROWS and K % 8 == 0):
+        return 0
+    n_cus = n_cus or compute_units()
+    strips = -(-N // 16)
+    if N * K > (1 << 22):                     # (smaller ones: only the number of kernels counts)
+        if strips < n_cus // 2:
+            return 0
+        if strips > n_cus and strips % n_cus and N * K > (1 << 25):
+            return 0
+        if M > 8 and K > 16384:
+            return 0
+    return 8 if strips <= n_cus and K >= 1024 else 4
+
+
+def gemm_residual_bf16(x: torch.Tensor, a: torch.Tensor, pw: PackedWeight, bias: Optional[torch.Tensor],
+                       waves: int, norm_w: Optional[torch.Tensor] = None) -> Optional[RowSquares]:
+    """x [M, N] (float32, in place) += a [M, K] . w^T (+ bias) for up to 16 rows of bfloat16 activations in
+    one kernel, every sum in an order fixed by the shapes; returns the sums of squares of x's new rows, by
+    strips of 16 columns, and with `norm_w` [N] also x * norm_w in bfloat16 (the rows of the rmsnorm with
+    that weight, without their scale).  None for shapes it does not take."""
+    if a.dtype != torch.bfloat16 or a.dim() != 2 or x.dim() != 2 or x.dtype != torch.float32 or pw.gate_rows:
+        return None
+    M, K = a.shape
+    N = pw.N
+    if not (K == pw.K and x.shape == (M, N) and 0 < M <= RESIDUAL_MAX_ROWS and K % 8 == 0 and a.stride(1) == 1
+            and a.stride(0) % 8 == 0 and x.stride(1) == 1 and a.data_ptr() % 16 == 0 and pw.data.data_ptr() % 16 == 0):
+        return None
+    _dev(x, a, pw.data, bias, norm_w)
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.shape == (N,), "gemm: bias must be float32 [N]")
+    unscaled = None
+    if norm_w is not None:
+        _need(norm_w.dtype == torch.float32 and norm_w.shape == (N,) and norm_w.is_contiguous(), "gemm: norm weight must be float32 [N]")
+        unscaled = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    sums = torch.empty((-(-N // 16), 16), dtype=torch.float32, device=x.device)
+    code = _lib().llogos_gemm_residual_bf16(_p(x), x.stride(0), _p(sums), _p(unscaled), N, _p(norm_w), _p(a), a.stride(0),
+                                            _p(pw.data), _p(bias), M, N, K, int(waves), _stream())
+    if code == -2:
+        return None
+    _check(code, "gemm_residual_bf16")
+    return RowSquares(sums, N, unscaled, norm_w)
+
+
+def gemm_packed_unscaled_bf16(squares: RowSquares, eps: float, pw: PackedWeight, bias: Optional[torch.Tensor],
+                              out_dtype: torch.dtype, splits: int = 1, chunk: int = 128) -> Optional[torch.Tensor]:
+    """The few-row product on packed weights with an rmsnorm's rows as its activations, of which `squares`
+    holds x * norm_w in bfloat16 and the sums of squares of x (gemm_residual_bf16 with norm_w): the rows'
+    scale 1 / sqrt(mean square + eps) is applied to the product, in float32.  On a matrix packed with
+    gate_rows the result is silu(gate) * up [M, gate_rows], otherwise [parts, M, N] as gemm_packed_bf16 (a
+    bias is added after the scale).  None for shapes it does not take."""
+    a = squares.unscaled
+    if a is None:
+        return None
+    M, K = a.shape
+    N = pw.N
+    if not (K == pw.K and squares.width == K and 0 < M <= RESIDUAL_MAX_ROWS and K % 8 == 0 and a.stride(1) == 1
+            and a.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and pw.data.data_ptr() % 16 == 0):
+        return None
+    _dev(a, squares.sums, pw.data, bias)
+    lib = _lib()
+    gated = pw.gate_rows > 0
+    if gated:
+        if bias is not None:
+            return None
+        parts, cols = 1, pw.gate_rows
+        out = torch.empty((M, cols), dtype=out_dtype, device=a.device)
+    else:
+        if bias is not None:
+            _need(bias.dtype == torch.float32 and bias.shape == (N,), "gemm: bias must be float32 [N]")
+        parts = lib.llogos_gemm_packed_parts(K, int(splits), int(chunk))
+        _need(parts >= 1, "gemm: the LDS buffer holds 128 or 256 values of k")
+        if parts > 1:
+            _need(bias is None, "gemm: a product in parts leaves the bias to its consumer")
+            out_dtype = torch.float32
+        cols = N
+        out = torch.empty((parts, M, N), dtype=out_dtype, device=a.device)
+    code = lib.llogos_gemm_packed_unscaled_bf16(
+        _p(out), _DT[out_dtype], _p(a), a.stride(0), _p(squares.sums), squares.sums.shape[0], K,
+        ctypes.c_float(eps), _p(pw.data), _p(bias), M, N, K, cols, ctypes.c_longlong(M * N), int(splits), int(chunk),
+        int(gated), _stream())
+    if code == -2:
+        return None
+    _check(code, "gemm_packed_unscaled_bf16")
     return out
 
 

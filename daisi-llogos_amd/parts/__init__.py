@@ -1,6 +1,6 @@
 """Parts a layer is put together from; importing the package registers the built-in ones."""
 from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITIONS, Block, FeedForward, GroupView, KVSpec, LayerCache,
-                   Mixer, Norm, Part, PositionEncoding, Runtime, StateSpec, StepContext, TensorSpec, make,
+                   Mixer, Norm, NormedRows, Part, PositionEncoding, Residual, Runtime, StateSpec, StepContext, TensorSpec, make,
                    register_block, register_feed_forward, register_mixer, register_norm, register_position)
 from .linear import Linear
 from .norm import RMSNorm

@@ -14,7 +14,7 @@ from typing import Callable, List, Optional
 import torch
 
 from ..ops import kernels as K
-from .base import KVSpec, LayerCache, Mixer, Runtime, StepContext, TensorSpec, mark, register_mixer
+from .base import KVSpec, LayerCache, Mixer, Residual, Runtime, StepContext, TensorSpec, mark, register_mixer
 from .linear import Linear
 from .rope import Rotary
 
@@ -22,6 +22,8 @@ from .rope import Rotary
 @register_mixer("attention")
 class Attention(Mixer):
     graph_safe = True
+    takes_normed_rows = True       # h goes into the q/k/v product alone
+    adds_to_residual = True        # the output projection can add itself to the stream
 
     def __init__(self, prefix: str, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int,
                  position: Rotary, bias: bool = False, qk_norm: bool = False, eps: float = 1e-6,
@@ -66,7 +68,7 @@ class Attention(Mixer):
         if getattr(self.position, "inv_freq", None) is None:
             self.position.bind(get, rt)
 
-    def forward(self, ctx: StepContext, h: torch.Tensor, cache: LayerCache) -> torch.Tensor:
+    def forward(self, ctx: StepContext, h, cache: LayerCache, residual: Optional[Residual] = None):
         nh, nkv, hd = self.n_heads, self.n_kv_heads, self.head_dim
         cs = self.position.prepare(ctx)
         if cache.writes:
@@ -80,7 +82,7 @@ class Attention(Mixer):
                                              self.sinks)
                 if a is not None:
                     mark(ctx, "attention")
-                    return self._project(ctx, a)
+                    return self._project(ctx, a, residual)
             q = K.qk_rope_cache(qkv, self.qkv.bias_rows(), self.rt.dtype, nh, nkv, hd, self.position.rot,
                                 self.position.pairing, self.q_norm_w, self.k_norm_w, self.eps, cs,
                                 cache.k_pool, cache.v_pool, cache.table, ctx.tok_seq, ctx.tok_pos)
@@ -95,9 +97,11 @@ class Attention(Mixer):
         a = K.attention(ctx, q, q.stride(0), cache.k_pool, cache.v_pool, cache.table,
                         nh, nkv, hd, self.scale, self.window, self.sinks)
         mark(ctx, "attention")
-        return self._project(ctx, a)
+        return self._project(ctx, a, residual)
 
-    def _project(self, ctx: StepContext, a: torch.Tensor) -> torch.Tensor:
-        out = self.o.product(a, f32_ok=True)    # the residual sum that follows adds the parts
+    def _project(self, ctx: StepContext, a: torch.Tensor, residual: Optional[Residual] = None):
+        out = self.o.add_to(a, residual) if residual is not None else None
+        if out is None:
+            out = self.o.product(a, f32_ok=True)    # the residual sum that follows adds the parts
         mark(ctx, "o")
         return out

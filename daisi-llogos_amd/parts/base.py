@@ -153,9 +153,39 @@ class Part:
         return total
 
 
+@dataclass
+class Residual:
+    """The float32 residual stream x [T, H] offered to a part whose last product may add itself to it,
+    with the norm that reads the stream next (None when its rows are not wanted in advance)."""
+    x: torch.Tensor
+    norm: Optional["Norm"] = None
+
+
+@dataclass
+class NormedRows:
+    """A norm's rows that still lack their scale: `squares` holds x * weight in bfloat16 and the sums of
+    squares of the rows of x (ops.kernels.RowSquares), left by the product that completed x.  A product
+    that takes them applies the scale to its result; tensor() runs the norm's own kernel instead."""
+    squares: object
+    eps: float
+    norm: "Norm"
+    x: torch.Tensor
+
+    def tensor(self) -> torch.Tensor:
+        return self.norm.forward(self.x)
+
+
 class Mixer(Part):
     """Token mixer: forward(ctx, h [T, H] in the runtime's type, cache) -> [T, H], or float32
-    partial sums [parts, T, H] that the residual sum after it adds."""
+    partial sums [parts, T, H] that the residual sum after it adds.
+
+    Two optional agreements with the block, each announced by a class attribute:
+    takes_normed_rows: h may be a NormedRows instead of a tensor;
+    adds_to_residual: forward takes `residual=Residual(...)` and may add its output to residual.x
+    itself, returning what the product left (ops.kernels.RowSquares) instead of a tensor."""
+
+    takes_normed_rows = False
+    adds_to_residual = False
 
     def kv_spec(self) -> Optional[KVSpec]:
         return None
@@ -175,7 +205,11 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    """forward(ctx, h [T, H]) -> [T, H], or float32 partial sums [parts, T, H]."""
+    """forward(ctx, h [T, H]) -> [T, H], or float32 partial sums [parts, T, H].  The optional agreements
+    of a Mixer (takes_normed_rows, adds_to_residual) hold here too."""
+
+    takes_normed_rows = False
+    adds_to_residual = False
 
     # True when forward launches the same kernels with the same shapes whatever the tokens are
     # (no routing decided on the host), so that a captured single-token step can be replayed.
@@ -188,11 +222,18 @@ class FeedForward(Part):
 class Norm(Part):
     """forward(x, delta, rows) -> normed rows in the runtime's type.  `x` is the float32
     residual stream; a pending `delta` ([T, H] or partial sums [parts, T, H]) is added to it
-    first (in place)."""
+    first (in place).  `delta` may also be what a product that has already added itself to x left
+    (ops.kernels.RowSquares): then x is complete, and with `lazy` a norm that can do so returns
+    NormedRows for a consumer that takes them."""
 
-    def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None,
-                rows: Optional[torch.Tensor] = None, write_back: bool = True) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, delta=None, rows: Optional[torch.Tensor] = None,
+                write_back: bool = True, lazy: bool = False):
         raise NotImplementedError
+
+    def row_weight(self) -> Optional[torch.Tensor]:
+        """float32 [H]: the weight w of a norm of the form x * w * (a scale of the whole row from the
+        row's mean square and eps); None for any other norm."""
+        return None
 
 
 class Block(Part):
@@ -201,7 +242,17 @@ class Block(Part):
 
     forward(ctx, x, pending, caches) -> (x, pending): `x` is the float32 residual stream
     [T, H], `pending` a delta that is still to be added to it ([T, H] or partial sums
-    [parts, T, H], or None), `caches` one LayerCache for each of mixers(), in that order."""
+    [parts, T, H], or None), `caches` one LayerCache for each of mixers(), in that order.
+    `pending` is handed to the block's first norm as its delta and may be whatever that norm takes.
+
+    A block that sets takes_next_norm is also given `next_norm`, the norm that reads the stream after
+    this block (entry_norm() of the block that runs next), for parts that prepare its rows."""
+
+    takes_next_norm = False
+
+    def entry_norm(self) -> Optional["Norm"]:
+        """The norm that takes `pending` (None if the block has no such norm)."""
+        return None
 
     def mixers(self) -> List["Mixer"]:
         return []

@@ -4,14 +4,16 @@
 
 Each residual sum is done inside the following norm's kernel, in float32, so the
 feed-forward's output is handed on as `pending` and added by whoever norms next
-(reference: the deferred adds of Daisi.Llogos/Inference/ForwardPass.cs:214-252)."""
+(reference: the deferred adds of Daisi.Llogos/Inference/ForwardPass.cs:214-252); or, for
+steps of few rows, by the product that closes the mixer or the feed-forward, which then also
+leaves the following norm's rows for the product that opens the next part."""
 from __future__ import annotations
 
 from typing import Callable, List, Optional, Tuple
 
 import torch
 
-from .base import Block, FeedForward, LayerCache, Mixer, Norm, Part, Runtime, StepContext, TensorSpec, mark, register_block
+from .base import Block, FeedForward, LayerCache, Mixer, Norm, Part, Residual, Runtime, StepContext, TensorSpec, mark, register_block
 
 
 @register_block("pre_norm")
@@ -28,15 +30,27 @@ class PreNormBlock(Block):
     def parts(self) -> List[Part]:
         return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn]
 
-    def forward(self, ctx: StepContext, x: torch.Tensor, pending: Optional[torch.Tensor],
-                caches) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    takes_next_norm = True
+
+    def entry_norm(self) -> Optional[Norm]:
+        return self.mixer_norm
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, pending, caches, next_norm: Optional[Norm] = None):
         cache = caches[0] if isinstance(caches, (list, tuple)) else caches
-        h = self.mixer_norm.forward(x, pending)
+        # A part that says so may add its output to x itself and leave the next norm's rows half made
+        # (then `a` or `d` is what it left, and the norm that takes it needs no kernel of its own).
+        h = self.mixer_norm.forward(x, pending, lazy=self.mixer.takes_normed_rows)
         mark(ctx, "norm")
-        a = self.mixer.forward(ctx, h, cache)
+        if self.mixer.adds_to_residual:
+            a = self.mixer.forward(ctx, h, cache, residual=Residual(x, self.ffn_norm))
+        else:
+            a = self.mixer.forward(ctx, h, cache)
         mark(ctx, "mixer")
-        h = self.ffn_norm.forward(x, a)
+        h = self.ffn_norm.forward(x, a, lazy=self.ffn.takes_normed_rows)
         mark(ctx, "norm")
-        d = self.ffn.forward(ctx, h)
+        if self.ffn.adds_to_residual:
+            d = self.ffn.forward(ctx, h, residual=Residual(x, next_norm))
+        else:
+            d = self.ffn.forward(ctx, h)
         mark(ctx, "feed_forward")
         return x, d

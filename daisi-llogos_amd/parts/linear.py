@@ -7,7 +7,7 @@ from typing import Callable, List, Optional, Sequence
 import torch
 
 from ..ops import kernels as K
-from .base import Part, Runtime, TensorSpec
+from .base import NormedRows, Part, Residual, Runtime, TensorSpec
 
 
 class Linear(Part):
@@ -92,22 +92,53 @@ class Linear(Part):
         total = self.weight.numel() * self.weight.element_size() if self.weight is not None else 0
         return total + (self.bias.numel() * self.bias.element_size() if self.bias is not None else 0)
 
-    def product(self, a: torch.Tensor, rows_out: Optional[int] = None, swiglu_input: bool = False,
+    def product(self, a, rows_out: Optional[int] = None, swiglu_input: bool = False,
                 f32_ok: bool = False) -> torch.Tensor:
         """a . W^T without the bias, as [M, out] or as float32 partial sums [parts, M, out] for a
         consumer kernel that adds parts (and the bias, `bias_rows`).  With `swiglu_input`, `a` is a
         fused gate/up product (maybe in parts) and W is applied to silu(gate) * up; with `f32_ok`
-        the consumer also takes a float32 result."""
+        the consumer also takes a float32 result.  `a` may be a norm's rows without their scale
+        (NormedRows), which the product on the packed copy then applies to its result."""
+        if isinstance(a, NormedRows):
+            pw = self._packed_rows(rows_out)
+            if pw is not None and not pw.gate_rows and not swiglu_input:
+                splits, chunk = K.packed_plan(a.x.shape[0], pw.N, pw.K)
+                out = K.gemm_packed_unscaled_bf16(a.squares, a.eps, pw, None, torch.float32 if f32_ok else self.rt.dtype,
+                                                  splits, chunk)
+                if out is not None:
+                    return out
+            a = a.tensor()
         w = self.weight if rows_out is None else self.weight[:rows_out]
         return K.gemm_product(a, w, self.rt.dtype, swiglu_input=swiglu_input, f32_ok=f32_ok,
                               packed=self._packed_rows(rows_out))
 
-    def gated_product(self, a: torch.Tensor) -> Optional[torch.Tensor]:
+    def add_to(self, a: torch.Tensor, residual: Residual):
+        """residual.x += a . W^T + bias in one kernel, for the few rows and the shapes that
+        gemm_residual_bf16 serves: returns what it left for the norm that follows (RowSquares, with that
+        norm's rows without their scale if residual.norm has a row weight), or None when x is untouched
+        and the caller takes the product as a tensor."""
+        if self.packed is None or self.packed.gate_rows or not isinstance(a, torch.Tensor) or a.dim() != 2:
+            return None
+        x = residual.x
+        if x.dim() != 2 or x.shape != (a.shape[0], self.packed.N):
+            return None
+        waves = K.residual_plan(a.shape[0], self.packed.N, self.packed.K)
+        if not waves:
+            return None
+        norm_w = residual.norm.row_weight() if residual.norm is not None else None
+        return K.gemm_residual_bf16(x, a, self.packed, self.bias, waves, norm_w)
+
+    def gated_product(self, a) -> Optional[torch.Tensor]:
         """silu(a . gate^T) * (a . up^T) as [M, out] in the runtime's type, made in one kernel from the
         packed copy (up to 64 rows the weight-streaming product, for prompts the tiled one); None where that
         does not apply (no packed copy, float32, row counts at which the library's product and a SwiGLU pass
         are faster)."""
-        if self.packed is None or not self.packed.gate_rows or a.dim() != 2:
+        if self.packed is None or not self.packed.gate_rows:
+            return None
+        if isinstance(a, NormedRows):
+            return K.gemm_packed_unscaled_bf16(a.squares, a.eps, self.packed, None, self.rt.dtype, 1,
+                                               K.packed_plan(a.x.shape[0], self.packed.N, self.packed.K)[1])
+        if a.dim() != 2:
             return None
         if a.shape[0] > K.SKINNY_MAX_ROWS:
             return K.gemm_tiles_bf16(a, self.packed, None, self.rt.dtype) if K.tiles_serve_gated(a.shape[0]) else None

@@ -7,13 +7,15 @@ from typing import Callable, List, Optional
 
 import torch
 
-from .base import FeedForward, Runtime, StepContext, TensorSpec, mark, register_feed_forward
+from .base import FeedForward, Residual, Runtime, StepContext, TensorSpec, mark, register_feed_forward
 from .linear import Linear
 
 
 @register_feed_forward("swiglu")
 class SwiGLU(FeedForward):
     graph_safe = True
+    takes_normed_rows = True
+    adds_to_residual = True
 
     def __init__(self, prefix: str, hidden: int, intermediate: int):
         self.prefix = prefix
@@ -29,13 +31,15 @@ class SwiGLU(FeedForward):
         self.gate_up.bind(get, rt)
         self.down.bind(get, rt)
 
-    def forward(self, ctx: StepContext, h: torch.Tensor) -> torch.Tensor:
+    def forward(self, ctx: StepContext, h, residual: Optional[Residual] = None):
         act = self.gate_up.gated_product(h)
         if act is not None:
             # on packed weights silu(gate) * up is the epilogue of the gate/up product
             # (the reference's MatMulSwiGLU, Daisi.Llogos/IComputeBackend.cs:448-456)
             mark(ctx, "gate_up")
-            out = self.down.product(act, f32_ok=True)
+            out = self.down.add_to(act, residual) if residual is not None else None
+            if out is None:
+                out = self.down.product(act, f32_ok=True)
             mark(ctx, "down")
             return out
         gu = self.gate_up.product(h)

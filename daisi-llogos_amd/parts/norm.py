@@ -9,7 +9,7 @@ from typing import Callable, List, Optional
 import torch
 
 from ..ops import kernels as K
-from .base import Norm, Runtime, TensorSpec, register_norm
+from .base import Norm, NormedRows, Runtime, TensorSpec, register_norm
 
 
 @register_norm("rmsnorm")
@@ -27,6 +27,15 @@ class RMSNorm(Norm):
         super().bind(get, rt)
         self.weight = get(self.name + ".weight").to(device=rt.device, dtype=torch.float32).contiguous()
 
-    def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None,
-                rows: Optional[torch.Tensor] = None, write_back: bool = True) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, delta=None, rows: Optional[torch.Tensor] = None,
+                write_back: bool = True, lazy: bool = False):
+        if isinstance(delta, K.RowSquares):
+            # the product before has added itself to x; if it also left this norm's rows without their
+            # scale, a consumer that takes them needs no kernel here
+            if lazy and rows is None and delta.unscaled is not None and delta.norm_w is self.weight:
+                return NormedRows(delta, self.eps, self, x)
+            delta = None
         return K.rmsnorm(x, self.weight, self.eps, self.rt.dtype, delta=delta, rows=rows, write_back=write_back)
+
+    def row_weight(self) -> Optional[torch.Tensor]:
+        return self.weight

@@ -690,6 +690,33 @@ def test_a_step_timed_part_by_part_is_the_same_step(dtype):
     assert probe.repeat([lambda: engines[0].model.layers[0].mixer_norm.forward(torch.zeros(2, 120, device="cuda"), None)] * 3) > 0
 
 
+@pytest.mark.parametrize("name", ["tiny_a", "tiny_b", "tiny_d"])
+def test_single_tokens_with_products_that_add_themselves_to_the_stream(name, monkeypatch):
+    """In bfloat16, steps of up to 16 single tokens close every mixer and feed-forward with the product that adds
+    itself to the residual stream, and the norm between two products has no kernel of its own: only the first
+    layer's first norm and the final one are launched.  With more rows, or with the switch off, every norm is a
+    kernel.  Both ways give the plain model's logits, sequence by sequence.  (tiny_d's feed-forward width is no
+    multiple of 16, so its gate/up product has no SwiGLU epilogue and its down projection, which makes silu(gate) *
+    up on the way in, hands its sums to the next layer's norm as before: one kernel a layer.)"""
+    layers = tc.ALL[name]["num_hidden_layers"]
+    fused = 2 if tc.ALL[name]["intermediate_size"] % 16 == 0 else layers + 1
+    toks = [H.tokens(name, 30 + 3 * i, 20 + i) for i in range(18)]
+    calls = []
+    real = K.rmsnorm
+    monkeypatch.setattr(K, "rmsnorm", lambda *a, **kw: (calls.append(1), real(*a, **kw))[1])
+    for mode, n_seq in (("on", 16), ("on", 5), ("off", 5), ("on", 18)):
+        monkeypatch.setattr(K, "RESIDUAL_PRODUCT", mode)
+        eng = H.engine(name, "bfloat16", max_tokens=64 * 40, n_slots=20, use_graphs=False)
+        slots = [eng.alloc_slot() for _ in range(n_seq)]
+        eng.step([(s, t[:-3]) for s, t in zip(slots, toks)], want="last")
+        for j in (3, 2, 1):
+            del calls[:]
+            out = _np(eng.step([(s, [t[-j]]) for s, t in zip(slots, toks)], want="last"))
+            assert len(calls) == (fused if mode == "on" and n_seq <= 16 else 2 * layers + 1), (mode, n_seq, len(calls))
+        for i in range(n_seq):
+            H.close(out[i], H.plain_logits(name, toks[i])[-1], "bfloat16", f"{mode}, {n_seq} sequences, sequence {i}", config=name)
+
+
 def test_benchmark_reports_bytes_and_flops_of_its_steps():
     """Llogos.benchmark's roofline inputs for tiny_a, worked by hand: two layers of
     qkv (128 x 64 + bias 128), o (64 x 64), gate/up (352 x 64), down (64 x 176), two norms (64 each), the

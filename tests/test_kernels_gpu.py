@@ -652,6 +652,101 @@ def test_gate_up_product_with_the_swiglu_epilogue(M, I, H):
         K.pack_weights(w, gate_rows=I + 16)
 
 
+@pytest.mark.parametrize("M,N,K_", [(1, 4096, 4096), (8, 4096, 14336), (16, 48, 200), (5, 80, 8), (13, 5120, 1000), (3, 16, 72), (9, 120, 200),
+                                    (2, 7, 16)])
+@pytest.mark.parametrize("waves", [4, 8, 16])
+def test_product_that_adds_itself_to_the_residual_stream(M, N, K_, waves):
+    """x += a w^T + bias in one kernel for up to 16 rows, with what it leaves for the norm that follows: the
+    sums of squares of the new rows by strips of 16 columns, and x * norm_w rounded to bfloat16.  Against
+    float64; rows beyond M stay zero in the sums; a row's result does not depend on the rows beside it."""
+    rng = np.random.default_rng(M * 100 + N + waves)
+    a, w = _t(rng.standard_normal((M, K_)), torch.bfloat16), _t(rng.standard_normal((N, K_)) * 0.05, torch.bfloat16)
+    bias, norm_w = _t(rng.standard_normal(N)), _t(1 + 0.1 * rng.standard_normal(N))
+    x0 = _t(rng.standard_normal((M, N)) * 3)
+    pw = K.pack_weights(w)
+    want = _np(x0) + _np(a) @ _np(w).T + _np(bias)
+    x = x0.clone()
+    left = K.gemm_residual_bf16(x, a, pw, bias, waves, norm_w)
+    assert isinstance(left, K.RowSquares) and left.width == N and left.norm_w is norm_w
+    _close(x, want, "float32", scale=np.abs(want).max() * 10)                    # bfloat16 operands, float32 sums
+    strips = -(-N // 16)
+    assert left.sums.shape == (strips, 16)
+    sums = _np(left.sums)
+    assert np.all(sums[:, M:] == 0)
+    padded = np.zeros((M, strips * 16))
+    padded[:, :N] = _np(x)
+    by_strip = (padded ** 2).reshape(M, strips, 16).sum(2).T                      # [strips, M] of the x it wrote
+    assert np.allclose(sums[:, :M], by_strip, rtol=2e-6, atol=1e-30)
+    assert torch.equal(left.unscaled, (x * norm_w).to(torch.bfloat16))           # the same float32 product, rounded once
+    # without a bias and without the norm's rows; one row alone gives the same bits
+    x1 = x0.clone()
+    plain = K.gemm_residual_bf16(x1, a, pw, None, waves)
+    assert plain.unscaled is None
+    _close(x1, want - _np(bias), "float32", scale=np.abs(want).max() * 10)
+    alone = x0[:1].clone()
+    K.gemm_residual_bf16(alone, a[:1].contiguous(), pw, None, waves)
+    assert torch.equal(alone, x1[:1])
+    # refused: more than 16 rows, a packed gate/up matrix
+    assert K.gemm_residual_bf16(torch.zeros(17, N, device=DEV), torch.zeros(17, K_, device=DEV, dtype=torch.bfloat16), pw, None, waves) is None
+
+
+@pytest.mark.parametrize("M,N,K_", [(1, 6144, 4096), (8, 331, 1000), (16, 96, 72), (7, 64, 4112), (11, 200, 16)])
+def test_product_on_norm_rows_without_their_scale(M, N, K_):
+    """The few-row product whose activations are x * w of an rmsnorm, with the sums of squares of x beside
+    them: the row's scale 1 / sqrt(mean square + eps) is applied to the result.  Against float64 on the same
+    bfloat16 rows; parts and a bias; any number of partial sums (also more than 256 and fewer than 16)."""
+    rng = np.random.default_rng(M + N)
+    eps = 1e-5
+    x = _t(rng.standard_normal((M, K_)) * 2)
+    norm_w = _t(1 + 0.1 * rng.standard_normal(K_))
+    w = _t(rng.standard_normal((N, K_)) * 0.05, torch.bfloat16)
+    bias = _t(rng.standard_normal(N))
+    pw = K.pack_weights(w)
+    unscaled = (x * norm_w).to(torch.bfloat16)
+    inv = 1.0 / np.sqrt((_np(x) ** 2).mean(1) + eps)
+    want = (_np(unscaled) @ _np(w).T) * inv[:, None]
+    for strips in (K_ // 8, 3, 300):                                               # the sums arrive in parts of any count
+        cols = np.array_split(np.arange(K_), strips)
+        sums = np.zeros((strips, 16))
+        for i, c in enumerate(cols):
+            sums[i, :M] = (_np(x)[:, c] ** 2).sum(1)
+        left = K.RowSquares(_t(sums), K_, unscaled, norm_w)
+        for splits, chunk in ((1, 128), (3, 256)):
+            out = K.gemm_packed_unscaled_bf16(left, eps, pw, None, torch.float32, splits, chunk)
+            assert out is not None and out.dtype == torch.float32
+            _close(out.sum(0), want, "float32", scale=np.abs(want).max() * 10)
+        out = K.gemm_packed_unscaled_bf16(left, eps, pw, bias, torch.bfloat16, 1, 128)
+        _close(out[0], want + _np(bias), "bfloat16")
+    # the norm's own kernel and the product on its output: the same up to one rounding of the activations
+    normed = K.rmsnorm(x.clone(), norm_w, eps, torch.bfloat16)
+    ref = K.gemm_packed_bf16(normed, pw, None, torch.float32, 1, 128)[0]
+    _close(K.gemm_packed_unscaled_bf16(left, eps, pw, None, torch.float32, 1, 128)[0], _np(ref), "bfloat16")
+
+
+@pytest.mark.parametrize("M,I,H", [(1, 208, 136), (8, 14336, 4096), (16, 64, 72)])
+def test_gate_up_product_on_norm_rows_without_their_scale(M, I, H):
+    rng = np.random.default_rng(M + I)
+    eps = 1e-6
+    wg, wu = (_t(rng.standard_normal((I, H)) * 0.08, torch.bfloat16) for _ in range(2))
+    pw = K.pack_weights(torch.cat([wg, wu]).contiguous(), gate_rows=I)
+    x = _t(rng.standard_normal((M, H)) * 4)
+    norm_w = _t(1 + 0.1 * rng.standard_normal(H))
+    unscaled = (x * norm_w).to(torch.bfloat16)
+    strips = -(-H // 16)
+    sums = np.zeros((strips, 16))
+    for i in range(strips):
+        sums[i, :M] = (_np(x)[:, 16 * i: 16 * i + 16] ** 2).sum(1)
+    inv = 1.0 / np.sqrt((_np(x) ** 2).mean(1) + eps)
+    a = _np(unscaled)
+    want = pm.silu((a @ _np(wg).T) * inv[:, None]) * ((a @ _np(wu).T) * inv[:, None])
+    left = K.RowSquares(_t(sums), H, unscaled, norm_w)
+    for chunk in (128, 256):
+        got = K.gemm_packed_unscaled_bf16(left, eps, pw, None, torch.float32, 1, chunk)
+        assert got is not None and got.shape == (M, I)
+        _close(got, want, "float32", scale=np.abs(want).max() * 50)
+    _close(K.gemm_packed_unscaled_bf16(left, eps, pw, None, torch.bfloat16, 1, 128), want, "bfloat16")
+
+
 @pytest.mark.parametrize("M,N,K_", [(65, 256, 64), (300, 1000, 512), (2048, 4096, 4096), (129, 6144, 1024), (700, 130, 192),
                                     (1500, 2300, 640)])
 @pytest.mark.parametrize("token_tiles", [0, 4, 2])

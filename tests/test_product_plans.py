@@ -93,3 +93,23 @@ def test_where_the_tiled_product_serves_prompts(monkeypatch):
     assert K.tiles_plan(300, *down) is None and not K.tiles_serve_gated(4096)
     monkeypatch.setattr(K, "PROMPT_PRODUCT", "tiles")
     assert K.tiles_plan(300, 4096, 4096) == (1, 0) and K.tiles_serve_gated(65)
+
+
+def test_where_the_product_that_adds_itself_to_the_stream_serves():
+    """The one-pass product with blocks of 16 rows of w serves up to 16 rows where its blocks fill the compute
+    units evenly (256 of them here): the 1B, 3B, 8B and 70B widths, the 14B output projection but not its down
+    projection (320 blocks), not the 70B down projection beyond 8 rows, never more than 16 rows or a k that is
+    no multiple of 8; tiny matrices always."""
+    plan = lambda M, N, K_: K.residual_plan(M, N, K_, n_cus=256)
+    for M in (1, 8, 16):
+        assert plan(M, 4096, 4096) == 8 and plan(M, 4096, 14336) == 8           # 8B
+        assert plan(M, 2048, 2048) == 8 and plan(M, 2048, 8192) == 8            # 1B
+        assert plan(M, 3072, 3072) == 8 and plan(M, 3072, 8192) == 8            # 3B
+        assert plan(M, 8192, 8192) == 4                                          # 70B o
+        assert plan(M, 5120, 5120) == 4 and plan(M, 5120, 17408) == 0           # 14B
+        assert plan(M, 1024, 8192) == 0                                          # 64 blocks on 256 units
+        assert plan(M, 120, 384) == 4 and plan(M, 64, 176) == 4                 # tiny: only the kernel count matters
+        assert plan(M, 4096, 4100) == 0
+    assert plan(8, 8192, 28672) == 4 and plan(16, 8192, 28672) == 0
+    assert plan(17, 4096, 4096) == 0 and plan(0, 4096, 4096) == 0
+    assert K.residual_plan(8, 4096, 4096, n_cus=64) == 4                         # four blocks a unit: fewer waves each
