@@ -676,43 +676,44 @@ RESIDUAL_PRODUCT = os.environ.get("LLOGOS_RESIDUAL_PRODUCT", "on")
 
 @dataclass
 class RowSquares:
-    """What a product that has added itself to the residual stream x leaves beside it: sums [strips, 16],
-    float32, strip s holding for each row of x the sum of the squares of columns 16 s .. 16 s + 15.  A
-    norm over the rows of x needs no other pass over them (gemm_packed_normed_bf16)."""
+    """What a product that has added itself to the residual stream x leaves beside it: sums [blocks, 16],
+    float32, each of the product's blocks holding for each row of x the sum of the squares of its 16 or 32
+    columns.  A norm over the rows of x needs no other pass over them (gemm_packed_unscaled_bf16)."""
     sums: torch.Tensor
     width: int                                  # columns of x that the sums cover
     unscaled: Optional[torch.Tensor] = None     # bfloat16 [M, width]: x * norm_w, the rmsnorm's rows without their scale
     norm_w: Optional[torch.Tensor] = None       # the weight that `unscaled` was made with
 
 
-def residual_plan(M: int, N: int, K: int, n_cus: Optional[int] = None) -> int:
-    """Waves of a block of gemm_residual_bf16 (0: not served; then the product in parts over k and the norm's
-    own kernel do the work).  A block owns 16 rows of w and all of k, so there are N / 16 blocks, and a
-    compute unit streams what its blocks own at a bounded rate: the blocks have to fill the units evenly.
-    Measured on the MI355X (256 units) at 1, 8 and 16 rows against the product in parts plus the norm kernel:
-      N / 16 <= units (1B, 3B, 8B widths): always ahead, 8 waves a block (8B at 8 rows: o 8.9 us against 12.4,
-        down 20.9 against 24.2);
-      N / 16 a multiple of the units (70B: 512): ahead with 4 waves (o 22.5 against 27.3, down 75.6 against
-        78.8), but behind at 16 rows with k beyond 16K (83 against 79), where a block's copy of the
-        activations is as many bytes as its weights;
-      N / 16 = 1.25 units (14B: 320): a quarter of the units get two blocks; ahead only for the small
-        matrix (o 14.0 against 16.1; down 38 against 33)."""
+def residual_plan(M: int, N: int, K: int, n_cus: Optional[int] = None) -> Tuple[int, int]:
+    """(waves of a block, strips of 16 rows of w a block) of gemm_residual_bf16; (0, 0): not served (then the
+    product in parts over k and the norm's own kernel do the work).  A block owns its rows of w and all of k,
+    and a compute unit streams what its blocks own at a bounded rate: the blocks have to fill the units evenly,
+    one block a unit at best.  Measured on the MI355X (256 units) at 1, 8 and 16 rows against the product in
+    parts plus the norm kernel (us):
+      N / 16 <= units (1B, 3B, 8B widths): blocks of one strip, 8 waves: 8B o 9.0 against 12.4, down 21.0
+        against 24.2 (two strips a block: 10.5 and 27.8: half the units idle);
+      more strips than units: two strips a block, which share a wave's copy of the activations: 70B (256
+        blocks) o 24.2 against 27.5, down 71.2 against 79.4 (one strip a block, two blocks a unit: 76.1); 14B
+        (160 blocks) o 12.8 against 16.1; its down projection, 89 M weights on 160 of 256 units, only up to 4
+        rows (31.6 against 35.4 at one row, 34.6 against 33.6 at 8, 38.4 against 34.1 at 16)."""
     if RESIDUAL_PRODUCT != "on" or not (0 < M <= RESIDUAL_MAX_ROWS and K % 8 == 0):
-        return 0
+        return 0, 0
     n_cus = n_cus or compute_units()
     strips = -(-N // 16)
-    if N * K > (1 << 22):                     # (smaller ones: only the number of kernels counts)
-        if strips < n_cus // 2:
-            return 0
-        if strips > n_cus and strips % n_cus and N * K > (1 << 25):
-            return 0
-        if M > 8 and K > 16384:
-            return 0
-    return 8 if strips <= n_cus and K >= 1024 else 4
+    waves = 8 if K >= 1024 else 4
+    if N * K <= (1 << 22):                    # so small that only the number of kernels counts
+        return waves, 1
+    if strips <= n_cus:
+        return (waves, 1) if strips >= n_cus // 2 else (0, 0)
+    blocks = -(-strips // 2)
+    if blocks < (3 * n_cus) // 4 and N * K > (1 << 25) and M > 4:
+        return 0, 0
+    return 8, 2
 
 
 def gemm_residual_bf16(x: torch.Tensor, a: torch.Tensor, pw: PackedWeight, bias: Optional[torch.Tensor],
-                       waves: int, norm_w: Optional[torch.Tensor] = None) -> Optional[RowSquares]:
+                       waves: int, norm_w: Optional[torch.Tensor] = None, strips: int = 1) -> Optional[RowSquares]:
     """x [M, N] (float32, in place) += a [M, K] . w^T (+ bias) for up to 16 rows of bfloat16 activations in
     one kernel, every sum in an order fixed by the shapes; returns the sums of squares of x's new rows, by
     strips of 16 columns, and with `norm_w` [N] also x * norm_w in bfloat16 (the rows of the rmsnorm with
@@ -731,9 +732,9 @@ def gemm_residual_bf16(x: torch.Tensor, a: torch.Tensor, pw: PackedWeight, bias:
     if norm_w is not None:
         _need(norm_w.dtype == torch.float32 and norm_w.shape == (N,) and norm_w.is_contiguous(), "gemm: norm weight must be float32 [N]")
         unscaled = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
-    sums = torch.empty((-(-N // 16), 16), dtype=torch.float32, device=x.device)
+    sums = torch.empty((-(-(-(-N // 16)) // int(strips)), 16), dtype=torch.float32, device=x.device)
     code = _lib().llogos_gemm_residual_bf16(_p(x), x.stride(0), _p(sums), _p(unscaled), N, _p(norm_w), _p(a), a.stride(0),
-                                            _p(pw.data), _p(bias), M, N, K, int(waves), _stream())
+                                            _p(pw.data), _p(bias), M, N, K, int(waves), int(strips), _stream())
     if code == -2:
         return None
     _check(code, "gemm_residual_bf16")

@@ -122,11 +122,11 @@ class Linear(Part):
         x = residual.x
         if x.dim() != 2 or x.shape != (a.shape[0], self.packed.N):
             return None
-        waves = K.residual_plan(a.shape[0], self.packed.N, self.packed.K)
+        waves, strips = K.residual_plan(a.shape[0], self.packed.N, self.packed.K)
         if not waves:
             return None
         norm_w = residual.norm.row_weight() if residual.norm is not None else None
-        return K.gemm_residual_bf16(x, a, self.packed, self.bias, waves, norm_w)
+        return K.gemm_residual_bf16(x, a, self.packed, self.bias, waves, norm_w, strips)
 
     def gated_product(self, a) -> Optional[torch.Tensor]:
         """silu(a . gate^T) * (a . up^T) as [M, out] in the runtime's type, made in one kernel from the

@@ -654,37 +654,37 @@ def test_gate_up_product_with_the_swiglu_epilogue(M, I, H):
 
 @pytest.mark.parametrize("M,N,K_", [(1, 4096, 4096), (8, 4096, 14336), (16, 48, 200), (5, 80, 8), (13, 5120, 1000), (3, 16, 72), (9, 120, 200),
                                     (2, 7, 16)])
-@pytest.mark.parametrize("waves", [4, 8, 16])
-def test_product_that_adds_itself_to_the_residual_stream(M, N, K_, waves):
+@pytest.mark.parametrize("waves,strips", [(4, 1), (8, 1), (16, 1), (8, 2), (4, 2)])
+def test_product_that_adds_itself_to_the_residual_stream(M, N, K_, waves, strips):
     """x += a w^T + bias in one kernel for up to 16 rows, with what it leaves for the norm that follows: the
     sums of squares of the new rows by strips of 16 columns, and x * norm_w rounded to bfloat16.  Against
     float64; rows beyond M stay zero in the sums; a row's result does not depend on the rows beside it."""
-    rng = np.random.default_rng(M * 100 + N + waves)
+    rng = np.random.default_rng(M * 100 + N + waves + strips)
     a, w = _t(rng.standard_normal((M, K_)), torch.bfloat16), _t(rng.standard_normal((N, K_)) * 0.05, torch.bfloat16)
     bias, norm_w = _t(rng.standard_normal(N)), _t(1 + 0.1 * rng.standard_normal(N))
     x0 = _t(rng.standard_normal((M, N)) * 3)
     pw = K.pack_weights(w)
     want = _np(x0) + _np(a) @ _np(w).T + _np(bias)
     x = x0.clone()
-    left = K.gemm_residual_bf16(x, a, pw, bias, waves, norm_w)
+    left = K.gemm_residual_bf16(x, a, pw, bias, waves, norm_w, strips)
     assert isinstance(left, K.RowSquares) and left.width == N and left.norm_w is norm_w
     _close(x, want, "float32", scale=np.abs(want).max() * 10)                    # bfloat16 operands, float32 sums
-    strips = -(-N // 16)
-    assert left.sums.shape == (strips, 16)
+    n_strips = -(-(-(-N // 16)) // strips)                                        # blocks of 16 * strips columns
+    assert left.sums.shape == (n_strips, 16)
     sums = _np(left.sums)
     assert np.all(sums[:, M:] == 0)
-    padded = np.zeros((M, strips * 16))
+    padded = np.zeros((M, n_strips * 16 * strips))
     padded[:, :N] = _np(x)
-    by_strip = (padded ** 2).reshape(M, strips, 16).sum(2).T                      # [strips, M] of the x it wrote
+    by_strip = (padded ** 2).reshape(M, n_strips, 16 * strips).sum(2).T                      # [strips, M] of the x it wrote
     assert np.allclose(sums[:, :M], by_strip, rtol=2e-6, atol=1e-30)
     assert torch.equal(left.unscaled, (x * norm_w).to(torch.bfloat16))           # the same float32 product, rounded once
     # without a bias and without the norm's rows; one row alone gives the same bits
     x1 = x0.clone()
-    plain = K.gemm_residual_bf16(x1, a, pw, None, waves)
+    plain = K.gemm_residual_bf16(x1, a, pw, None, waves, strips=strips)
     assert plain.unscaled is None
     _close(x1, want - _np(bias), "float32", scale=np.abs(want).max() * 10)
     alone = x0[:1].clone()
-    K.gemm_residual_bf16(alone, a[:1].contiguous(), pw, None, waves)
+    K.gemm_residual_bf16(alone, a[:1].contiguous(), pw, None, waves, strips=strips)
     assert torch.equal(alone, x1[:1])
     # refused: more than 16 rows, a packed gate/up matrix
     assert K.gemm_residual_bf16(torch.zeros(17, N, device=DEV), torch.zeros(17, K_, device=DEV, dtype=torch.bfloat16), pw, None, waves) is None

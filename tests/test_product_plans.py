@@ -96,20 +96,20 @@ def test_where_the_tiled_product_serves_prompts(monkeypatch):
 
 
 def test_where_the_product_that_adds_itself_to_the_stream_serves():
-    """The one-pass product with blocks of 16 rows of w serves up to 16 rows where its blocks fill the compute
-    units evenly (256 of them here): the 1B, 3B, 8B and 70B widths, the 14B output projection but not its down
-    projection (320 blocks), not the 70B down projection beyond 8 rows, never more than 16 rows or a k that is
-    no multiple of 8; tiny matrices always."""
+    """The one-pass product whose blocks own 16 or 32 rows of w and all of k serves up to 16 rows where its
+    blocks fill the compute units evenly (256 of them here): one strip a block up to 256 strips (1B, 3B, 8B), two
+    above (14B, 70B); the 14B down projection (160 blocks, 89 M weights) only up to 4 rows; never more than 16
+    rows or a k that is no multiple of 8; tiny matrices always."""
     plan = lambda M, N, K_: K.residual_plan(M, N, K_, n_cus=256)
     for M in (1, 8, 16):
-        assert plan(M, 4096, 4096) == 8 and plan(M, 4096, 14336) == 8           # 8B
-        assert plan(M, 2048, 2048) == 8 and plan(M, 2048, 8192) == 8            # 1B
-        assert plan(M, 3072, 3072) == 8 and plan(M, 3072, 8192) == 8            # 3B
-        assert plan(M, 8192, 8192) == 4                                          # 70B o
-        assert plan(M, 5120, 5120) == 4 and plan(M, 5120, 17408) == 0           # 14B
-        assert plan(M, 1024, 8192) == 0                                          # 64 blocks on 256 units
-        assert plan(M, 120, 384) == 4 and plan(M, 64, 176) == 4                 # tiny: only the kernel count matters
-        assert plan(M, 4096, 4100) == 0
-    assert plan(8, 8192, 28672) == 4 and plan(16, 8192, 28672) == 0
-    assert plan(17, 4096, 4096) == 0 and plan(0, 4096, 4096) == 0
-    assert K.residual_plan(8, 4096, 4096, n_cus=64) == 4                         # four blocks a unit: fewer waves each
+        assert plan(M, 4096, 4096) == (8, 1) and plan(M, 4096, 14336) == (8, 1)         # 8B
+        assert plan(M, 2048, 2048) == (8, 1) and plan(M, 2048, 8192) == (8, 1)          # 1B
+        assert plan(M, 3072, 3072) == (8, 1) and plan(M, 3072, 8192) == (8, 1)          # 3B
+        assert plan(M, 8192, 8192) == (8, 2) and plan(M, 8192, 28672) == (8, 2)         # 70B
+        assert plan(M, 5120, 5120) == (8, 2)                                             # 14B o
+        assert plan(M, 5120, 17408) == ((8, 2) if M <= 4 else (0, 0))                    # 14B down
+        assert plan(M, 1024, 8192) == (0, 0)                                             # 64 blocks on 256 units
+        assert plan(M, 120, 384) == (4, 1) and plan(M, 64, 176) == (4, 1)               # tiny: only the kernel count matters
+        assert plan(M, 4096, 4100) == (0, 0)
+    assert plan(17, 4096, 4096) == (0, 0) and plan(0, 4096, 4096) == (0, 0)
+    assert K.residual_plan(8, 4096, 4096, n_cus=64) == (8, 2)                            # fewer units: two strips a block
