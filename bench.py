@@ -241,31 +241,26 @@ def main(argv=None) -> int:
             return out if out is not None else layer.ffn.gate_up.product(rows)
         P = llogos.parts
         x = torch.randn(batch, cfg["hidden_size"], device=dev)
-        # steps of few rows: o and down add themselves to the stream and leave the next norm's rows, which
-        # gate/up and qkv take as they are (no norm kernel between); otherwise products in parts and the norm
-        left = [l.mixer.o.add_to(a, P.Residual(x, l.ffn_norm)) for l in layers]
-        if all(v is not None for v in left):
-            rows_ffn = [l.ffn_norm.forward(x, v, lazy=True) for l, v in zip(layers, left)]
-            left = [l.ffn.down.add_to(act, P.Residual(x, l.mixer_norm)) for l in layers]
-            rows_mixer = [l.mixer_norm.forward(x, v, lazy=True) for l, v in zip(layers, left)]
-            us = {
-                "qkv": probe.repeat([lambda l=l, r=r: l.mixer.qkv.product(r, f32_ok=True) for l, r in zip(layers, rows_mixer)]),
-                "o": probe.repeat([lambda l=l: l.mixer.o.add_to(a, P.Residual(x, l.ffn_norm)) for l in layers]),
-                "gate_up": probe.repeat([lambda l=l, r=r: gate_up(l, r) for l, r in zip(layers, rows_ffn)]),
-                "down": probe.repeat([lambda l=l: l.ffn.down.add_to(act, P.Residual(x, l.mixer_norm)) for l in layers]),
-                "norm": 0.0,
-            }
-        else:
-            us = {
-                "qkv": probe.repeat([lambda l=l: l.mixer.qkv.product(h, f32_ok=True) for l in layers]),
-                "o": probe.repeat([lambda l=l: l.mixer.o.product(a, f32_ok=True) for l in layers]),
-                "gate_up": probe.repeat([lambda l=l: gate_up(l, h) for l in layers]),
-                "down": probe.repeat([lambda l=l: l.ffn.down.product(act, f32_ok=True) for l in layers]),
-                "norm": probe.repeat([lambda l=l: l.mixer_norm.forward(torch.zeros(batch, cfg["hidden_size"], device=dev), None)
-                                      for l in layers]),
-            }
+        # steps of few rows: o and down add themselves to the stream where their shapes allow and leave the next
+        # norm's rows, which gate/up and qkv take as they are (no norm kernel between); otherwise products in
+        # parts and the norm's kernel
+        def closing(product, act, norm):
+            if product.add_to(act, P.Residual(x, norm)) is not None:
+                return (lambda: product.add_to(act, P.Residual(x, norm))), norm.forward(x, product.add_to(act, P.Residual(x, norm)), lazy=True)
+            return (lambda: product.product(act, f32_ok=True)), h
+        o_calls, rows_ffn = zip(*[closing(l.mixer.o, a, l.ffn_norm) for l in layers])
+        down_calls, rows_mixer = zip(*[closing(l.ffn.down, act, l.mixer_norm) for l in layers])
+        norms_a_layer = sum(1 for r in (rows_ffn[0], rows_mixer[0]) if r is h)
+        us = {
+            "qkv": probe.repeat([lambda l=l, r=r: l.mixer.qkv.product(r, f32_ok=True) for l, r in zip(layers, rows_mixer)]),
+            "o": probe.repeat(list(o_calls)),
+            "gate_up": probe.repeat([lambda l=l, r=r: gate_up(l, r) for l, r in zip(layers, rows_ffn)]),
+            "down": probe.repeat(list(down_calls)),
+            "norm": probe.repeat([lambda l=l: l.mixer_norm.forward(torch.zeros(batch, cfg["hidden_size"], device=dev), None)
+                                  for l in layers]) if norms_a_layer else 0.0,
+        }
         us["head"] = probe.repeat([lambda: eng.model.head.forward(h, out_dtype=torch.float32)] * 3)
-        us["attention"] = (step_us - us["head"]) / len(layers) - us["qkv"] - us["o"] - us["gate_up"] - us["down"] - 2 * us["norm"]
+        us["attention"] = (step_us - us["head"]) / len(layers) - us["qkv"] - us["o"] - us["gate_up"] - us["down"] - norms_a_layer * us["norm"]
         out = {}
         for name, (nbytes, _) in part_costs(cfg, batch, batch, context).items():
             out[name + "_us"] = round(us[name], 1)

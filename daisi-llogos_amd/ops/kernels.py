@@ -679,7 +679,7 @@ class RowSquares:
     """What a product that has added itself to the residual stream x leaves beside it: sums [blocks, 16],
     float32, each of the product's blocks holding for each row of x the sum of the squares of its 16 or 32
     columns.  A norm over the rows of x needs no other pass over them (gemm_packed_unscaled_bf16)."""
-    sums: torch.Tensor
+    sums: Optional[torch.Tensor]                # None: the product left nothing but the complete stream
     width: int                                  # columns of x that the sums cover
     unscaled: Optional[torch.Tensor] = None     # bfloat16 [M, width]: x * norm_w, the rmsnorm's rows without their scale
     norm_w: Optional[torch.Tensor] = None       # the weight that `unscaled` was made with
@@ -928,6 +928,26 @@ def gemm_product(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, swigl
             return torch.mm(a, w.t(), out_dtype=torch.float32)
         return torch.matmul(a, w.t())
     return gemm_generic(a, w, None, out_dtype)
+
+
+def gemm_library_add(x: torch.Tensor, a: torch.Tensor, w: torch.Tensor, packed: Optional[PackedWeight] = None) -> bool:
+    """x [M, N] (float32, in place) += a [M, K] . w^T by the library's bfloat16 product with float32
+    accumulation and the sum in its epilogue, where the library serves this product anyway (prompts of
+    more than 128 rows that the tiled product does not take): the stream is read and written once there
+    instead of the product being written, read again and added by the norm's kernel.  False (and x
+    untouched) otherwise.  The result is the float32 product added to x, bit for bit."""
+    if RESIDUAL_PRODUCT != "on":
+        return False
+    if not (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dtype == torch.float32 and a.dim() == 2
+            and x.dim() == 2 and a.is_contiguous() and x.is_contiguous() and w.is_contiguous()):
+        return False
+    M, N = a.shape[0], w.shape[0]
+    if M <= LDS_MAX_ROWS or x.shape != (M, N) or a.shape[1] != w.shape[1] or a.shape[1] % 8:
+        return False
+    if packed is not None and tiles_plan(M, packed.N, packed.K) is not None:
+        return False
+    torch.addmm(x, a, w.t(), out_dtype=torch.float32, out=x)
+    return True
 
 
 def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out_dtype: torch.dtype,

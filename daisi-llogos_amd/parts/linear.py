@@ -113,13 +113,21 @@ class Linear(Part):
                               packed=self._packed_rows(rows_out))
 
     def add_to(self, a: torch.Tensor, residual: Residual):
-        """residual.x += a . W^T + bias in one kernel, for the few rows and the shapes that
-        gemm_residual_bf16 serves: returns what it left for the norm that follows (RowSquares, with that
-        norm's rows without their scale if residual.norm has a row weight), or None when x is untouched
-        and the caller takes the product as a tensor."""
-        if self.packed is None or self.packed.gate_rows or not isinstance(a, torch.Tensor) or a.dim() != 2:
+        """residual.x += a . W^T + bias in one kernel: for the few rows and the shapes that
+        gemm_residual_bf16 serves, and for prompts that the library's product serves (its epilogue adds).
+        Returns what the product left for the norm that follows (RowSquares: with that norm's rows without
+        their scale if residual.norm has a row weight; empty after the library's product), or None when x
+        is untouched and the caller takes the product as a tensor."""
+        if not isinstance(a, torch.Tensor) or a.dim() != 2:
             return None
         x = residual.x
+        if a.shape[0] > K.SKINNY_MAX_ROWS:
+            # prompts: the library's product with the sum in its epilogue, where the library serves anyway
+            if self.bias is None and K.gemm_library_add(x, a, self.weight, self.packed):
+                return K.RowSquares(None, self.weight.shape[0])
+            return None
+        if self.packed is None or self.packed.gate_rows:
+            return None
         if x.dim() != 2 or x.shape != (a.shape[0], self.packed.N):
             return None
         waves, strips = K.residual_plan(a.shape[0], self.packed.N, self.packed.K)

@@ -690,6 +690,27 @@ def test_product_that_adds_itself_to_the_residual_stream(M, N, K_, waves, strips
     assert K.gemm_residual_bf16(torch.zeros(17, N, device=DEV), torch.zeros(17, K_, device=DEV, dtype=torch.bfloat16), pw, None, waves) is None
 
 
+def test_library_product_that_adds_itself_to_the_residual_stream():
+    """For prompts that the library's product serves, the sum with the residual stream is the product's
+    epilogue: the float32 product added to x, bit for bit; refused for few rows, other element types and where
+    the tiled product serves."""
+    rng = np.random.default_rng(5)
+    for M, N, K_ in ((200, 96, 72), (2048, 4096, 4096), (129, 331, 1000)):
+        a, w = _t(rng.standard_normal((M, K_)), torch.bfloat16), _t(rng.standard_normal((N, K_)) * 0.05, torch.bfloat16)
+        x0 = _t(rng.standard_normal((M, N)) * 3)
+        x = x0.clone()
+        assert K.gemm_library_add(x, a, w)
+        assert torch.equal(x, x0 + torch.mm(a, w.t(), out_dtype=torch.float32))
+        _close(x, _np(x0) + _np(a) @ _np(w).T, "float32", scale=np.abs(_np(x)).max() * 10)
+    x = x0[:64].clone()
+    assert not K.gemm_library_add(x, a[:64].contiguous(), w) and torch.equal(x, x0[:64])
+    assert not K.gemm_library_add(x0.clone(), a.float(), w.float())
+    a, w = _t(rng.standard_normal((256, 8192)), torch.bfloat16), _t(rng.standard_normal((1024, 8192)) * 0.05, torch.bfloat16)
+    pw = K.pack_weights(w)
+    if K.tiles_plan(256, 1024, 8192) is not None:                              # much longer than high: the tiled product in parts
+        assert not K.gemm_library_add(torch.zeros(256, 1024, device=DEV), a, w, pw)
+
+
 @pytest.mark.parametrize("M,N,K_", [(1, 6144, 4096), (8, 331, 1000), (16, 96, 72), (7, 64, 4112), (11, 200, 16)])
 def test_product_on_norm_rows_without_their_scale(M, N, K_):
     """The few-row product whose activations are x * w of an rmsnorm, with the sums of squares of x beside

@@ -222,11 +222,14 @@ def test_swiglu_part_alone(dtype):
     assert np.abs(_np(got) - want).max() <= TOL[dtype] * max(1.0, np.abs(want).max())
 
 
+@pytest.mark.parametrize("T", [37, 200])
 @pytest.mark.parametrize("dtype", H.DTYPES)
-def test_block_arrangement_alone(dtype):
+def test_block_arrangement_alone(dtype, T):
     """The pre-norm block built from its parts: the pending sum handed in is added by the first
-    norm, the mixer's output by the second, and the feed-forward's output is handed on; against
-    the plain layer of the first tiny configuration, a prompt and then a single token."""
+    norm, the mixer's output by the second, and the feed-forward's output is handed on (or, in bfloat16,
+    added by the product that made it: the one-pass product for a single token, the library's epilogue for
+    a prompt of more than 128 rows); against the plain layer of the first tiny configuration, a prompt and
+    then a single token."""
     name = "tiny_a"
     cfg, w = H.plain(name)
     rt = P.Runtime(DEV, DT[dtype])
@@ -238,24 +241,27 @@ def test_block_arrangement_alone(dtype):
     tensors = load_file(os.path.join(H.folder(name), "model.safetensors"))
     block.bind(tensors.get, rt)
     rng = np.random.default_rng(12)
-    T = 37
     x0, pend = rng.standard_normal((T + 1, cfg.hidden)), rng.standard_normal((T + 1, cfg.hidden)) * 0.3
     f = cfg.frequencies()
     want = pm.decoder_layer(cfg, w, 1, x0 + pend, list(range(T + 1)), f)
     kv = block.mixer.kv_spec()
-    pool = lambda: torch.zeros((2, kv.n_kv_heads, 64 * kv.head_dim), dtype=DT[dtype], device=DEV)
+    pool = lambda: torch.zeros((6, kv.n_kv_heads, 64 * kv.head_dim), dtype=DT[dtype], device=DEV)
     cache = P.LayerCache(k_pool=pool(), v_pool=pool(),
-                         table=torch.tensor([[1]], dtype=torch.int32, device=DEV))
+                         table=torch.tensor([[1, 4, 2, 5]], dtype=torch.int32, device=DEV))
     got = []
     for lo, hi in ((0, T), (T, T + 1)):
         x = torch.tensor(x0[lo:hi], dtype=torch.float32, device=DEV)
         p = torch.tensor(pend[lo:hi], dtype=torch.float32, device=DEV)
         x_out, pending = block.forward(_ctx(rt, [hi], [hi - lo]), x, p, cache)
         assert x_out is x                                                # the stream is updated in place
-        if isinstance(pending, K.RowSquares):                            # the last product has added itself (few rows)
-            assert hi - lo <= K.RESIDUAL_MAX_ROWS
-            squares = _np(pending.sums).sum(0)[: hi - lo]
-            assert np.allclose(squares, (_np(x_out) ** 2).sum(1), rtol=1e-5)
+        if isinstance(pending, K.RowSquares):                            # the last product has added itself
+            assert dtype == "bfloat16"
+            if pending.sums is not None:                                 # few rows: with the rows' sums of squares
+                assert hi - lo <= K.RESIDUAL_MAX_ROWS
+                squares = _np(pending.sums).sum(0)[: hi - lo]
+                assert np.allclose(squares, (_np(x_out) ** 2).sum(1), rtol=1e-5)
+            else:
+                assert hi - lo > 128
             got.append(_np(x_out))
         else:
             got.append(_np(x_out) + _np(K.sum_parts(pending, None, torch.float32)))
