@@ -149,7 +149,7 @@ class Linear(Part):
         if a.dim() != 2:
             return None
         if a.shape[0] > K.SKINNY_MAX_ROWS:
-            return K.gemm_tiles_bf16(a, self.packed, None, self.rt.dtype) if K.tiles_serve_gated(a.shape[0]) else None
+            return K.gemm_tiles_bf16(a, self.packed, None, self.rt.dtype) if K.tiles_serve_gated(a.shape[0], a.shape[1]) else None
         return K.gemm_packed_gated_bf16(a, self.packed, self.rt.dtype, K.packed_plan(a.shape[0], self.packed.N, self.packed.K)[1])
 
     def bias_rows(self, rows_out: Optional[int] = None) -> Optional[torch.Tensor]:

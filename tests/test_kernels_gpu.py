@@ -848,7 +848,7 @@ def test_long_prompts_take_the_tiled_gate_up_product_by_default():
     """From TILES_MIN_ROWS tokens on the gate/up product with its SwiGLU epilogue is the hand-written one;
     the logits are the plain ones either way, and the two ways agree within bfloat16 rounding."""
     import gpu_helpers as H
-    assert K.PROMPT_PRODUCT == "auto" and K.tiles_serve_gated(K.TILES_MIN_ROWS) and not K.tiles_serve_gated(K.TILES_MIN_ROWS - 1)
+    assert K.PROMPT_PRODUCT == "auto" and K.tiles_serve_gated(K.TILES_MIN_ROWS, 4096) and not K.tiles_serve_gated(K.TILES_MIN_ROWS - 1, 4096)
     name = "layer_8b"
     eng = H.engine(name, "bfloat16", max_tokens=64 * 18, n_slots=1)
     toks = H.tokens(name, K.TILES_MIN_ROWS + 40, 2)

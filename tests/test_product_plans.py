@@ -76,11 +76,12 @@ def test_sets_of_waves_of_the_prompt_attention():
 
 
 def test_where_the_tiled_product_serves_prompts(monkeypatch):
-    """By default the tiled product takes the gate/up product with its SwiGLU epilogue from TILES_MIN_ROWS rows
-    on, and plain products only for matrices much longer than high at 129 to 1,024 rows, in parts of k that
-    hold at least two stages of 64."""
+    """By default the tiled product takes the gate/up product with its SwiGLU epilogue at 1,024 to 2,048 rows and
+    k up to 5,120, and plain products only for matrices much longer than high at 129 to 1,024 rows, in parts of
+    k that hold at least two stages of 64."""
     assert K.PROMPT_PRODUCT == "auto"
-    assert K.tiles_serve_gated(K.TILES_MIN_ROWS) and not K.tiles_serve_gated(K.TILES_MIN_ROWS - 1)
+    assert K.tiles_serve_gated(1024, 4096) and K.tiles_serve_gated(2048, 5120) and not K.tiles_serve_gated(1023, 4096)
+    assert not K.tiles_serve_gated(2049, 4096) and not K.tiles_serve_gated(2048, 8192)
     down = (4096, 14336)
     assert K.tiles_plan(64, *down) is None and K.tiles_plan(128, *down) is None          # the few-row products' rows
     assert K.tiles_plan(129, *down) == (4, 2) and K.tiles_plan(256, *down) == (4, 2)
