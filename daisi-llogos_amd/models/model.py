@@ -211,9 +211,9 @@ class Model:
         blocks = [self.layers[entry.layer] for entry in self.schedule]
         for i, (block, units) in enumerate(zip(blocks, self.entry_units)):
             if block.takes_next_norm:
-                # the norm that reads the stream after this block: the next block's first one (the final
-                # norm reads only the wanted rows and prepares its own)
-                next_norm = blocks[i + 1].entry_norm() if i + 1 < len(blocks) else None
+                # the norm that reads the stream after this block: the next block's first one, the final
+                # norm after the last (None: the next block has no such norm and takes `pending` as a tensor)
+                next_norm = blocks[i + 1].entry_norm() if i + 1 < len(blocks) else self.final_norm
                 x, pending = block.forward(ctx, x, pending, [caches[u] for u in units], next_norm=next_norm)
             else:
                 x, pending = block.forward(ctx, x, pending, [caches[u] for u in units])

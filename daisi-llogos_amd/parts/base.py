@@ -230,6 +230,11 @@ class Norm(Part):
                 write_back: bool = True, lazy: bool = False):
         raise NotImplementedError
 
+    # True when forward takes, as `delta`, what a product that has already added itself to the stream
+    # left (ops.kernels.RowSquares).  A block offers the stream to its parts (Residual) only when the
+    # norm that reads it next says so.
+    takes_row_squares = False
+
     def row_weight(self) -> Optional[torch.Tensor]:
         """float32 [H]: the weight w of a norm of the form x * w * (a scale of the whole row from the
         row's mean square and eps); None for any other norm."""

@@ -35,20 +35,25 @@ class PreNormBlock(Block):
     def entry_norm(self) -> Optional[Norm]:
         return self.mixer_norm
 
+    @staticmethod
+    def _norm(norm: Norm, x: torch.Tensor, delta, lazy: bool):
+        # (only a norm that knows of unscaled rows is asked for them)
+        return norm.forward(x, delta, lazy=True) if lazy and norm.takes_row_squares else norm.forward(x, delta)
+
     def forward(self, ctx: StepContext, x: torch.Tensor, pending, caches, next_norm: Optional[Norm] = None):
         cache = caches[0] if isinstance(caches, (list, tuple)) else caches
         # A part that says so may add its output to x itself and leave the next norm's rows half made
         # (then `a` or `d` is what it left, and the norm that takes it needs no kernel of its own).
-        h = self.mixer_norm.forward(x, pending, lazy=self.mixer.takes_normed_rows)
+        h = self._norm(self.mixer_norm, x, pending, self.mixer.takes_normed_rows)
         mark(ctx, "norm")
-        if self.mixer.adds_to_residual:
+        if self.mixer.adds_to_residual and self.ffn_norm.takes_row_squares:
             a = self.mixer.forward(ctx, h, cache, residual=Residual(x, self.ffn_norm))
         else:
             a = self.mixer.forward(ctx, h, cache)
         mark(ctx, "mixer")
-        h = self.ffn_norm.forward(x, a, lazy=self.ffn.takes_normed_rows)
+        h = self._norm(self.ffn_norm, x, a, self.ffn.takes_normed_rows)
         mark(ctx, "norm")
-        if self.ffn.adds_to_residual:
+        if self.ffn.adds_to_residual and next_norm is not None and next_norm.takes_row_squares:
             d = self.ffn.forward(ctx, h, residual=Residual(x, next_norm))
         else:
             d = self.ffn.forward(ctx, h)

@@ -14,6 +14,8 @@ from .base import Norm, NormedRows, Runtime, TensorSpec, register_norm
 
 @register_norm("rmsnorm")
 class RMSNorm(Norm):
+    takes_row_squares = True
+
     def __init__(self, name: str, width: int, eps: float):
         self.name = name
         self.width = width

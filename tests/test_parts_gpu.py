@@ -481,6 +481,123 @@ def test_the_command_line_runs_a_toy_architecture(tmp_path, capsys):
 # ---------------------------------------------------------------------------
 # a toy feed-forward with routing and a toy position encoding, defined here
 # ---------------------------------------------------------------------------
+@P.register_norm("toy_layernorm")
+class ToyLayerNorm(P.Norm):
+    """(v - mean(v)) / sqrt(var(v) + eps) * w + b with v = x + delta: a norm that is no scale of the whole row,
+    written against the plain interface (a tensor or nothing as delta)."""
+
+    def __init__(self, name, width, eps):
+        self.name, self.width, self.eps = name, width, eps
+
+    def tensor_specs(self):
+        return [P.TensorSpec(self.name + ".weight", (self.width,), "norm"), P.TensorSpec(self.name + ".bias", (self.width,), "bias")]
+
+    def bind(self, get, rt):
+        self.rt = rt
+        self.w = get(self.name + ".weight").to(device=rt.device, dtype=torch.float32)
+        self.b = get(self.name + ".bias").to(device=rt.device, dtype=torch.float32)
+
+    def forward(self, x, delta=None, rows=None, write_back=True):
+        assert delta is None or isinstance(delta, torch.Tensor)
+        v = x
+        if delta is not None:
+            v = x + (delta.float().sum(0) if delta.dim() == 3 else delta.float())
+            if write_back:
+                x.copy_(v)
+        if rows is not None:
+            v = v[rows.long()]
+        out = torch.nn.functional.layer_norm(v, (self.width,), self.w, self.b, self.eps)
+        return out.to(self.rt.dtype)
+
+
+@dataclasses.dataclass(frozen=True)
+class ToyNormConfig:
+    vocab_size: int
+    hidden_size: int
+    n_layers: int
+    architecture: str = "ToyNormForCausalLM"
+
+
+def _toy_norm_kinds(i):
+    """(mixer norm, feed-forward norm) of layer i: every neighbourhood of the two kinds of norm in four layers."""
+    return (("rmsnorm", "toy_layernorm"), ("toy_layernorm", "rmsnorm"), ("rmsnorm", "rmsnorm"), ("toy_layernorm", "toy_layernorm"))[i % 4]
+
+
+def _toy_norm_spec(cfg, **kw):
+    models = importlib.import_module("daisi-llogos_amd.models")
+    rot = P.Rotary(16, 16, 1e4)
+    layers = []
+    for i in range(cfg.n_layers):
+        p = f"layers.{i}."
+        kinds = _toy_norm_kinds(i)
+        layers.append(models.LayerSpec(
+            mixer=("attention", dict(prefix=p + "attn.", hidden=cfg.hidden_size, n_heads=4, n_kv_heads=2, head_dim=16, position=rot)),
+            ffn=("swiglu", dict(prefix=p + "ffn.", hidden=cfg.hidden_size, intermediate=48)),
+            mixer_norm=(kinds[0], dict(name=p + "n1", width=cfg.hidden_size, eps=1e-5)),
+            ffn_norm=(kinds[1], dict(name=p + "n2", width=cfg.hidden_size, eps=1e-5))))
+    return models.ModelSpec(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size, embed_name="embed.weight",
+                            layers=layers, final_norm=("toy_layernorm", dict(name="norm", width=cfg.hidden_size, eps=1e-5)),
+                            head_name="head", tie_head=False)
+
+
+L.register_architecture("ToyNormForCausalLM",
+                        lambda d: ToyNormConfig(d["vocab_size"], d["hidden_size"], d["n_layers"]), _toy_norm_spec)
+
+
+def _plain_toy_norm(w, tokens, n_layers):
+    def norm(kind, x, name):
+        if kind == "rmsnorm":
+            return pm.rms_norm(x, w[name + ".weight"], 1e-5)
+        c = x - x.mean(1, keepdims=True)
+        return c / np.sqrt((c * c).mean(1, keepdims=True) + 1e-5) * w[name + ".weight"] + w[name + ".bias"]
+    T = len(tokens)
+    x = pm.embedding(w["embed.weight"], tokens)
+    f = pm.rope_frequencies(16, 1e4)
+    for i in range(n_layers):
+        p = f"layers.{i}."
+        kinds = _toy_norm_kinds(i)
+        n = norm(kinds[0], x, p + "n1")
+        q = pm.rope_split_half(pm.linear(n, w[p + "attn.q_proj.weight"]), range(T), 4, 16, f)
+        k = pm.rope_split_half(pm.linear(n, w[p + "attn.k_proj.weight"]), range(T), 2, 16, f)
+        x = x + pm.linear(pm.attention(q, k, pm.linear(n, w[p + "attn.v_proj.weight"]), 4, 2, 16), w[p + "attn.o_proj.weight"])
+        n = norm(kinds[1], x, p + "n2")
+        x = x + pm.swiglu_mlp(n, w[p + "ffn.gate_proj.weight"], w[p + "ffn.up_proj.weight"], w[p + "ffn.down_proj.weight"])
+    return pm.linear(norm("toy_layernorm", x, "norm"), w["head.weight"])
+
+
+@pytest.mark.parametrize("dtype", H.DTYPES)
+def test_a_toy_norm_beside_the_products_that_add_themselves_to_the_stream(tmp_path, dtype, monkeypatch):
+    """A norm of another form, registered here and written against the plain interface, stands before, between and
+    after the built-in parts in every neighbourhood: a product hands its sum to such a norm as a tensor, as
+    before, and adds itself to the stream only where an rmsnorm reads next.  Prompts and single tokens against
+    the plain model; in bfloat16 the single-token steps do use the one-pass product where they may."""
+    from safetensors.torch import load_file
+    cfg = {"architectures": ["ToyNormForCausalLM"], "vocab_size": 90, "hidden_size": 64, "n_layers": 5,
+           "torch_dtype": "float32"}
+    folder = L.write_random_model(str(tmp_path / "toy"), cfg, seed=4)
+    w = {k: v.double().numpy() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    eng = L.Engine.from_folder(folder, dtype=dtype, max_tokens=1024, n_slots=3, use_graphs=False)
+    calls = []
+    real = K.gemm_residual_bf16
+    monkeypatch.setattr(K, "gemm_residual_bf16", lambda *a, **kw: (calls.append(a[1].shape), real(*a, **kw))[1])
+    rng = np.random.default_rng(3)
+    seqs = [rng.integers(0, 90, size=n).tolist() for n in (33, 150, 9)]
+    want = [_plain_toy_norm(w, s, 5) for s in seqs]
+    tol = 1e-4 if dtype == "float32" else 3e-2
+    slots = [eng.alloc_slot() for _ in seqs]
+    out = _np(eng.step([(sl, s[:-2]) for sl, s in zip(slots, seqs)], want="last"))
+    for i, s in enumerate(seqs):
+        assert np.abs(out[i] - want[i][len(s) - 3]).max() <= tol * max(1.0, np.abs(want[i]).max())
+    assert not calls                                                     # prompts: more than 16 rows
+    for j in (2, 1):
+        out = _np(eng.step([(sl, [s[-j]]) for sl, s in zip(slots, seqs)], want="last"))
+        for i, s in enumerate(seqs):
+            assert np.abs(out[i] - want[i][len(s) - j]).max() <= tol * max(1.0, np.abs(want[i]).max())
+    # layers 0..4 have (rms, toy), (toy, rms), (rms, rms), (toy, toy), (rms, toy) and the final norm is a toy: the
+    # one-pass product closes a part only where an rmsnorm reads next: o of layers 1 and 2, down of layers 1 and 3
+    assert len(calls) == (2 * 4 if dtype == "bfloat16" else 0)
+
+
 @P.register_feed_forward("toy_routed")
 class ToyRoutedFeedForward(P.FeedForward):
     """A router picks one of `n_experts` SwiGLU experts for each token; the expert's output is
