@@ -241,6 +241,11 @@ def test_float32_product_of_few_rows_is_the_tiled_product_bit_for_bit(N, K_):
     for M in (1, 2, 3, 4, 7, 8, 9, 16, 31, 32):
         few = K.gemm_generic(a[:M], w, b, torch.float32)
         assert torch.equal(few, tiled[:M]), (M, N, K_, (few - tiled[:M]).abs().max().item())
+    # several tiles of rows: the same bits again
+    big = torch.cat([a, _t(rng.standard_normal((160, K_)))])
+    out = K.gemm_generic(big, w, b, torch.float32)
+    assert torch.equal(out[:40], tiled)
+    assert torch.equal(out[195:200], K.gemm_generic(big[195:200].contiguous(), w, b, torch.float32))
     wide = _t(rng.standard_normal((5, K_ + 3)))                            # rows that do not start at a multiple of 16 bytes
     few = K.gemm_generic(wide[:, :K_], w, None, torch.float32)
     many = K.gemm_generic(torch.cat([wide, wide * 0 + 1.0] * 4)[:, :K_], w, None, torch.float32)
