@@ -4,10 +4,10 @@
 //
 // A block owns 16 (or 32) rows of w (as many columns of x) and the whole of k: its waves take equal runs of
 // k, each with one MFMA accumulator; LDS adds the waves' sums in ascending order of k, the
-// block adds them to its 16 columns of x (float32, in place) and writes for every row of x the
+// block adds them to its columns of x (float32, in place) and writes for every row of x the
 // sum of the squares of its new values: sums[block][16], and x * norm_w in bfloat16, the rows
 // of the rmsnorm that follows without their scale.  The product that takes norm(x) as its
-// activations (gemm_skinny_lds_bf16.hip, PRODUCE_UNSCALED) multiplies these rows, adds the strips'
+// activations (gemm_skinny_lds_bf16.hip, PRODUCE_UNSCALED) multiplies these rows, adds the blocks'
 // sums in ascending order and applies 1 / rms to its result: no other pass over x and no kernel
 // between the two products.  Nothing here depends on what else runs: the order of every addition is
 // fixed by N, K and the number of waves.
@@ -18,8 +18,9 @@
 //
 // Weights: llogos_pack_weights' layout, [N / 64][K / 32][4 strips][64 lanes] fragments of 16
 // bytes; strip s of a 64-row group is every fourth KB of the group's run.  Activations: each
-// wave loads its own MFMA operand from a (rows beyond M: zero); with at most 16 rows that is
-// at most as many bytes as the weights and they come from the L2.
+// wave copies the rows of a for its own run of k (rows beyond M: zero) through its own part of
+// LDS; with at most 16 rows that is at most as many bytes as the weights, and they come from
+// the L2.  A block with 16 waves holds 86 to 102 KB of LDS (the waves' copies and their sums).
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
