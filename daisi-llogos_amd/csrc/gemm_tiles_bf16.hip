@@ -287,7 +287,7 @@ template <typename TO, int EPI>
 __global__ __launch_bounds__(kTileWaves * kWave) void gemm_tiles_kernel(
         TO* __restrict__ out, const bf16_t* __restrict__ a, int lda, const unsigned char* __restrict__ wp,
         const float* __restrict__ bias, int M, int N, int K, int ldo, size_t part_stride, int n_row_blocks,
-        int m_tiles4, int m_tiles2, int n_full, int n_tiles, int blocks4, int parts, int stages_per_part) {
+        int m_tiles4, int m_tiles2, int n_full, int n_tiles, int blocks4, int parts) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char tiles_lds[];
     const int stages = K / kStageK;
     const bool big = (int)blockIdx.x < blocks4;
@@ -297,7 +297,9 @@ __global__ __launch_bounds__(kTileWaves * kWave) void gemm_tiles_kernel(
     const int m_tile = jb % m_tiles, u = xcd + 8 * (jb / m_tiles);
     const int part = u % parts, n_tile = (big ? 0 : n_full) + u / parts;
     if (n_tile >= (big ? n_full : n_tiles)) return;
-    const int s0 = part * stages_per_part, s1 = min(stages, s0 + stages_per_part);
+    // the parts divide the stages evenly: part p takes [stages p / parts, stages (p + 1) / parts), none is empty
+    // when there are at least as many stages as parts
+    const int s0 = (int)((long long)stages * part / parts), s1 = (int)((long long)stages * (part + 1) / parts);
     TO* dst = out + (size_t)part * part_stride;
     if (big) tile_body<4, TO, EPI>(tiles_lds, dst, a, lda, wp, bias, M, N, K, ldo, n_row_blocks, m_tile, n_tile, s0, s1);
     else tile_body<2, TO, EPI>(tiles_lds, dst, a, lda, wp, bias, M, N, K, ldo, n_row_blocks, m_tile, n_tile, s0, s1);
@@ -323,7 +325,6 @@ static int launch_tiles(void* out, const void* a, int lda, const void* wp, const
     const int n_full = tiles_n_full(n_tiles, m4, parts, token_tiles, compute_units);
     const int u4 = n_full * parts, u2 = (n_tiles - n_full) * parts;
     const int blocks4 = m4 * ((u4 + 7) / 8) * 8, blocks2 = m2 * ((u2 + 7) / 8) * 8;
-    const int stages = K / kStageK, stages_per_part = (stages + parts - 1) / parts;
     constexpr size_t smem = (size_t)2 * (kStageW + 256 * kStageK * 2);
     // (the attribute is set once per instance: not per launch, which may be recorded into a graph)
     static bool ready = false;
@@ -335,7 +336,7 @@ static int launch_tiles(void* out, const void* a, int lda, const void* wp, const
     }
     gemm_tiles_kernel<TO, EPI><<<blocks4 + blocks2, kTileWaves * kWave, smem, stream>>>(
         (TO*)out, (const bf16_t*)a, lda, (const unsigned char*)wp, bias, M, N, K, ldo, (size_t)part_stride, n_row_blocks,
-        m4, m2, n_full, n_tiles, blocks4, parts, stages_per_part);
+        m4, m2, n_full, n_tiles, blocks4, parts);
     return LLOGOS_LAUNCH_CHECK();
 }
 
@@ -356,7 +357,7 @@ LLOGOS_EXPORT int llogos_gemm_tiles_bf16(void* out, int out_dtype, const void* a
     if (token_tiles != 4 && token_tiles != 2 && token_tiles != 0) return LLOGOS_BAD_ARGUMENT;
     if (parts < 1 || compute_units < 1) return LLOGOS_BAD_ARGUMENT;
     if (parts > 1 && (out_dtype != DT_F32 || bias != nullptr || part_stride < (long long)M * ldo)) return LLOGOS_BAD_ARGUMENT;
-    if (parts > 1 && (K / kStageK) / parts < 2) return LLOGOS_UNSUPPORTED;          // (then no part is empty either)
+    if (parts > 1 && (K / kStageK) / parts < 2) return LLOGOS_UNSUPPORTED;          // every part holds two stages or more
 #define GO(EPI) do { if (out_dtype == DT_BF16) return launch_tiles<bf16_t, EPI>(out, a, lda, packed_w, bias, M, N, K, ldo, part_stride, parts, token_tiles, compute_units, stream); \
                      return launch_tiles<float, EPI>(out, a, lda, packed_w, bias, M, N, K, ldo, part_stride, parts, token_tiles, compute_units, stream); } while (0)
     if (epilogue == EPI_SWIGLU) GO(EPI_SWIGLU);

@@ -774,7 +774,7 @@ def test_gate_up_product_on_norm_rows_without_their_scale(M, I, H):
 
 
 @pytest.mark.parametrize("M,N,K_", [(65, 256, 64), (300, 1000, 512), (2048, 4096, 4096), (129, 6144, 1024), (700, 130, 192),
-                                    (1500, 2300, 640)])
+                                    (1500, 2300, 640), (190, 136, 576), (318, 40, 576)])
 @pytest.mark.parametrize("token_tiles", [0, 4, 2])
 def test_tiled_product_for_many_rows_on_packed_weights(M, N, K_, token_tiles):
     """The hand-written prompt-size product (tiles of 256 or 128 tokens x 256 rows, 32x32x16 MFMAs on the
@@ -787,14 +787,14 @@ def test_tiled_product_for_many_rows_on_packed_weights(M, N, K_, token_tiles):
     _close(K.gemm_tiles_bf16(a, pw, None, torch.float32, token_tiles=token_tiles), want, "float32", scale=np.abs(want).max() * 10)
     _close(K.gemm_tiles_bf16(a, pw, bias, torch.bfloat16, token_tiles=token_tiles), want + _np(bias), "bfloat16")
     assert K.gemm_tiles_bf16(a[:, :K_ - 8].contiguous(), K.pack_weights(w[:, :K_ - 8].contiguous()), None, torch.float32) is None
-    for parts in (2, 3):
+    for parts in (2, 3, 4):                                             # (9 stages in 4 parts: 2, 2, 2 and 3, none empty)
         got = K.gemm_tiles_bf16(a, pw, None, torch.bfloat16, parts=parts, token_tiles=token_tiles)
         if K_ // 64 // parts < 2:
             assert got is None                                          # a part would hold less than two stages of 64
             continue
         assert got.shape == (parts, M, N) and got.dtype == torch.float32
         if parts == 2:                                                  # the first part is the product over the first half of k
-            half = -(-(K_ // 64) // 2) * 64
+            half = (K_ // 64) // 2 * 64
             _close(got[0], _np(a)[:, :half] @ _np(w)[:, :half].T, "float32", scale=np.abs(want).max() * 10)
         _close(got.sum(0), want, "float32", scale=np.abs(want).max() * 10)
         _close(K.sum_parts(got, bias, torch.float32), want + _np(bias), "float32", scale=np.abs(want).max() * 10)
