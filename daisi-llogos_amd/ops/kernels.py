@@ -757,6 +757,9 @@ def gemm_packed_unscaled_bf16(squares: RowSquares, eps: float, pw: PackedWeight,
             and a.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and pw.data.data_ptr() % 16 == 0):
         return None
     _dev(a, squares.sums, pw.data, bias)
+    _need(squares.sums.dtype == torch.float32 and squares.sums.dim() == 2 and squares.sums.shape[1] == RESIDUAL_MAX_ROWS
+          and squares.sums.is_contiguous() and squares.sums.shape[0] >= 1 and a.dtype == torch.bfloat16,
+          "gemm: the sums of squares are float32 [parts, 16], the unscaled rows bfloat16")
     lib = _lib()
     gated = pw.gate_rows > 0
     if gated:
