@@ -78,6 +78,68 @@ def prefill_flops(cfg, t):
     return 2 * linear * t + attn + 2 * v * h
 
 
+def clocks_under_load(torch, K, seconds=3.0):
+    """The GPU's clock (rocm-smi, read from a thread) while one kind of work runs in a loop: idle, a few-row product
+    that waits for memory, MFMAs on registers, and the gate/up product of 2,048 rows of the 8B sizes by the tiled
+    kernel and by the library.  The prompt's products run against the power limit: the clock says how far."""
+    import re
+    import shutil
+    import subprocess
+    import threading
+    import time
+    if shutil.which("rocm-smi") is None:
+        print("[ceilings] clocks: no rocm-smi on this machine", flush=True)
+        return
+    dev = "cuda:0"
+
+    def sample(stop, out):
+        while not stop.is_set():
+            try:
+                text = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=10).stdout
+                m = re.search(r"sclk clock level[^\n]*\((\d+)Mhz\)", text)
+                if m:
+                    out.append(int(m.group(1)))
+            except (OSError, subprocess.SubprocessError):
+                return
+            time.sleep(0.2)
+
+    def under(label, fn, flops=0.0):
+        stop, seen = threading.Event(), []
+        th = threading.Thread(target=sample, args=(stop, seen))
+        th.start()
+        t0, n = time.time(), 0
+        while time.time() - t0 < seconds:
+            for _ in range(20):
+                fn()
+            torch.cuda.synchronize()
+            n += 20
+        dt = (time.time() - t0) / n
+        stop.set()
+        th.join()
+        mhz = sorted(seen[1:])[len(seen[1:]) // 2] if len(seen) > 1 else 0
+        rate = f", {flops / dt / 1e15:.3f} PFLOP/s, {flops / dt / (MFMA_PEAK['bf16'] * mhz / 2400.0) :.2f} of the peak at that clock" if flops and mhz else ""
+        print(f"[ceilings] clock under {label}: {mhz} MHz ({dt * 1e6:.0f} us a call{rate})", flush=True)
+
+    M, I, H = 2048, 14336, 4096
+    a = (torch.randn(M, H, device=dev) * 0.5).to(torch.bfloat16)
+    w = (torch.randn(2 * I, H, device=dev) * 0.02).to(torch.bfloat16)
+    pw = K.pack_weights(w, I)
+    wd = [K.pack_weights((torch.randn(H, I, device=dev) * 0.02).to(torch.bfloat16)) for _ in range(8)]
+    a8 = torch.randn(8, I, device=dev).to(torch.bfloat16)
+    turn = [0]
+
+    def few_rows():
+        turn[0] = (turn[0] + 1) % len(wd)
+        K.gemm_packed_bf16(a8, wd[turn[0]], None, torch.float32, 8, 128)
+    time.sleep(1.0)
+    under("nothing", lambda: None)
+    under("the down product of 8 rows (memory-bound)", few_rows)
+    under("MFMAs on registers", lambda: K.measure_mfma_rate(iters=2000, shapes=(32,)))
+    flops = 2.0 * M * 2 * I * H
+    under("the tiled gate/up product of 2,048 rows", lambda: K.gemm_tiles_bf16(a, pw, None, torch.bfloat16), flops)
+    under("the library's gate/up product of 2,048 rows", lambda: torch.matmul(a, w.t()), flops)
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -119,6 +181,7 @@ def main(argv=None) -> int:
                 print(f"[ceilings] mfma bf16 {'16x16x32' if shape == 16 else '32x32x16'}, "
                       f"{'random operands' if noisy else 'constant operands'}: {rate / 1e15:.3f} PFLOP/s "
                       f"({rate / MFMA_PEAK['bf16']:.3f} of {MFMA_PEAK['bf16'] / 1e15:g})", flush=True)
+        clocks_under_load(torch, K)
         return 0
 
     model_name, cfg = MODELS[args.model]
