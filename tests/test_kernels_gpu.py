@@ -226,6 +226,35 @@ def test_products_of_random_shapes_through_the_dispatch():
         assert np.abs(got - (want + _np(b))).max() <= 2e-5 * scale, (case, M, N, K_)
 
 
+def test_prompt_products_of_random_shapes_on_packed_weights():
+    """Prompts through the dispatch with a packed copy at hand: whatever the plan picks (the tiled product in one
+    part or in parts of k for matrices much longer than high, the library's elsewhere), every number of stages of
+    64 and every way they fall into parts, heights below one block of rows, token counts that fill no tile."""
+    rng = np.random.default_rng(33)
+    seen = set()
+    for case in range(36):
+        M = int(rng.choice([129, 130, 190, 256, 257, 300, 511, 512, 513, 700, 1024]))
+        K_ = 64 * int(rng.integers(1, 40)) if case % 3 else 64 * int(rng.choice([9, 10, 11, 13, 17, 18, 19, 35]))
+        N = int(rng.integers(1, max(2, K_ // 2))) if case % 2 else int(rng.integers(1, 3000))
+        a = _t(rng.standard_normal((M, K_)), torch.bfloat16)
+        w = torch.randn((N, K_), device=DEV, dtype=torch.bfloat16, generator=torch.Generator(device=DEV).manual_seed(case)) * 0.05
+        pw = K.pack_weights(w)
+        want = _np(a.float() @ w.float().t())
+        scale = max(1.0, np.abs(want).max())
+        plan = K.tiles_plan(M, N, K_)
+        seen.add(plan)
+        prod = K.gemm_product(a, w, torch.bfloat16, f32_ok=True, packed=pw)
+        assert (prod.dim() == 3 and prod.shape[0] == plan[0]) if plan is not None and plan[0] > 1 else prod.shape[-2:] == (M, N)
+        got = _np(K.sum_parts(prod, None, torch.float32))
+        assert np.abs(got - want).max() <= (1e-2 if prod.dtype == torch.bfloat16 else 2e-5) * scale, (case, M, N, K_, plan)
+        for parts in (2, 4):                                               # every split the kernel takes, whether the plan asks for it or not
+            if K_ // 64 // parts >= 2:
+                got = K.gemm_tiles_bf16(a, pw, None, torch.float32, parts=parts, token_tiles=int(rng.choice([0, 2, 4])))
+                assert got.shape == (parts, M, N)
+                assert np.abs(_np(got.sum(0)) - want).max() <= 2e-5 * scale, (case, M, N, K_, parts)
+    assert {p[0] for p in seen if p is not None} >= {1, 2, 4} and None in seen        # what the cases were drawn to cover
+
+
 @pytest.mark.parametrize("N,K_", [(70, 16), (2048, 8192), (17000, 1000), (33000, 2049), (66000, 530), (5, 4099), (300, 7)])
 def test_float32_product_of_few_rows_is_the_tiled_product_bit_for_bit(N, K_):
     """Up to 32 rows in float32 go to a kernel of their own (a wave a few columns, the rows of a in
