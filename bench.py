@@ -344,11 +344,6 @@ def main(argv=None) -> int:
             eng.free_slot(s)
         return 0
 
-    # what this GPU does at best: reading as many bytes as the model's weights, and the matrix cores' issue rate
-    read_peak = K.measure_read_bandwidth(min(weight_bytes(cfg), 4 << 30), repeats=5)
-    mfma_peak = K.measure_mfma_rate()
-    print(f"[bench] measured ceilings: read {read_peak / 1e12:.2f} TB/s, mfma bf16 {mfma_peak / 1e15:.3f} PFLOP/s",
-          file=sys.stderr, flush=True)
     dt, ctx_mid = decode_run(args.batch, args.steps, args.warmup)
     ms_per_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
@@ -366,8 +361,7 @@ def main(argv=None) -> int:
                    "rope_theta": cfg["rope_theta"], "rope_scaling": f"llama3 x{cfg['rope_scaling']['factor']:g}" if cfg.get("rope_scaling") else "none", "rms_eps": cfg["rms_norm_eps"],
                    "sampling": sampling, "hip_graphs": eng.graphs is not None},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK, 4), "measured_peak": round(read_peak / 1e9, 1),
-                     "frac_of_measured": round(achieved / read_peak, 4)},
+                     "frac": round(achieved / HBM_PEAK, 4)},
     }
     print(f"[bench] decode b{args.batch}: {value:.1f} tok/s, {ms_per_step:.3f} ms/step, "
           f"{achieved / 1e12:.2f} TB/s", file=sys.stderr, flush=True)
@@ -401,6 +395,7 @@ def main(argv=None) -> int:
                   f"{fractions[f'decode_b{b}']:.3f} of {HBM_PEAK / 1e12:g} TB/s", file=sys.stderr, flush=True)
         record["points"] = points
         record["points_roofline_frac"] = fractions
+    if not args.no_points:
         prompt = rng.integers(0, cfg["vocab_size"], size=prefill_tokens).tolist()
         times = []
         for it in range(5):                              # the first warms the library up; the best of the rest counts
@@ -414,12 +409,21 @@ def main(argv=None) -> int:
         pt = min(times[1:])
         flops = prefill_flops(cfg, prefill_tokens)
         record["prefill"] = {"value": round(prefill_tokens / pt, 1), "tokens": prefill_tokens, "ms": round(pt * 1e3, 3),
-                             "frac": round(flops / pt / MFMA_PEAK["bf16"], 4),
-                             "measured_peak_tflops": round(mfma_peak / 1e12, 1),
-                             "frac_of_measured": round(flops / pt / mfma_peak, 4)}
+                             "frac": round(flops / pt / MFMA_PEAK["bf16"], 4)}
         print(f"[bench] prefill {prefill_tokens}: {prefill_tokens / pt:.0f} tok/s, {pt * 1e3:.2f} ms (five runs: "
               f"{min(times) * 1e3:.2f} to {max(times[1:]) * 1e3:.2f} after the first)", file=sys.stderr, flush=True)
         record["prefill"]["ms_max"] = round(max(times[1:]) * 1e3, 3)
+    # What this GPU does at best: reading as many bytes as the model's weights, and the matrix cores' issue rate.
+    # (After the timed decode steps and prompts: seconds of MFMAs at the power limit just before them cost the
+    # decode steps 2 %.)
+    read_peak = K.measure_read_bandwidth(min(weight_bytes(cfg), 4 << 30), repeats=5)
+    mfma_peak = K.measure_mfma_rate()
+    print(f"[bench] measured ceilings: read {read_peak / 1e12:.2f} TB/s, mfma bf16 {mfma_peak / 1e15:.3f} PFLOP/s",
+          file=sys.stderr, flush=True)
+    record["roofline"].update(measured_peak=round(read_peak / 1e9, 1), frac_of_measured=round(achieved / read_peak, 4))
+    if not args.no_points:
+        record["prefill"].update(measured_peak_tflops=round(mfma_peak / 1e12, 1),
+                                 frac_of_measured=round(prefill_flops(cfg, prefill_tokens) / pt / mfma_peak, 4))
         # where the time goes: a decode step of the headline batch and the prompt, part by part
         slots = [eng.alloc_slot() for _ in range(args.batch)]
         eng.step([(sl, rng.integers(0, cfg["vocab_size"], size=args.prompt_len).tolist()) for sl in slots], want="last")
